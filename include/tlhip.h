@@ -1,0 +1,259 @@
+/*
+ * tlhip.h — C ABI of the MI355X (gfx950) `hip` backend for torchlette's
+ * quantized-weight linear path.
+ *
+ * This is the boundary a torchlette `Backend` object binds through a Node
+ * N-API addon (or any FFI): plain pointers, sizes and enums, no C++ or torch
+ * types.  Each entry point cites the reference interface it stands in for
+ * (paths relative to the torchlette source tree).
+ *
+ * Conventions
+ *  - Every function that can fail returns int: 0 = ok, non-zero = error.  The
+ *    message is kept per thread and read with tlhip_last_error(); a binding
+ *    turns non-zero into `throw new Error(msg)`, the reference's only error
+ *    channel (src/backend/webgpu/ops/matmul-ops.ts:121-126).
+ *  - Pointers are DEVICE pointers unless the parameter name starts with host_.
+ *  - Work is enqueued on `stream` in order, as WebGPU queue submission is
+ *    (one JavaScript thread, ops enqueue, only `read` waits).  NULL means the
+ *    library's own stream, created by tlhip_init.
+ *  - There is no CPU fallback: without a usable gfx950 device every compute
+ *    entry point fails with an error.
+ */
+#ifndef TLHIP_H
+#define TLHIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TLHIP_OK 0
+#define TLHIP_ERR_INVALID 1 /* bad argument / unsupported combination */
+#define TLHIP_ERR_DEVICE 2  /* a HIP call failed */
+#define TLHIP_ERR_STATE 3   /* library not initialised */
+
+typedef void* tlhip_stream_t;
+typedef void* tlhip_event_t;
+
+/* Storage format of a packed weight: the values of
+ * StorageFormat.packing.scheme (src/backend/types.ts:46-55).  INT8_GROUPED is
+ * the reference's "int8-grouped"; INT4_GROUPED is the value its design doc
+ * plans (docs/quantization-design.md:69-75); INT8_ROW is int8 with one f32
+ * scale per output row (same byte packing, quantize.ts:121-125). */
+typedef enum {
+  TLHIP_FMT_INT8_GROUPED = 0, /* u32 [N,K/4]; f16 abs-max per group; w=(q/127)*s */
+  TLHIP_FMT_INT8_ROW = 1,     /* u32 [N,K/4]; f32 scale per row;      w=q*s      */
+  TLHIP_FMT_INT4_GROUPED = 2  /* u32 [N,K/8]; f16 scale per group;    w=q*s      */
+} tlhip_format_t;
+
+/* DType subset used on this path (src/backend/types.ts DType "f32" | "f16"). */
+typedef enum { TLHIP_F32 = 0, TLHIP_F16 = 1 } tlhip_dtype_t;
+
+/* Unary epilogue ops: the GEMV epilogue vocabulary
+ * (src/backend/webgpu/matmul/gemv.ts:135-143); formulas from
+ * src/ops/semantic/catalog.ts:81-109 and composite.ts:40-65. */
+typedef enum {
+  TLHIP_UNARY_NONE = 0,
+  TLHIP_UNARY_RELU = 1,
+  TLHIP_UNARY_SILU = 2,
+  TLHIP_UNARY_GELU_TANH = 3, /* the reference's "gelu" / "gelu_tanh" */
+  TLHIP_UNARY_GELU_ERF = 4,
+  TLHIP_UNARY_SIGMOID = 5,
+  TLHIP_UNARY_TANH = 6
+} tlhip_unary_t;
+
+typedef enum { TLHIP_EPI_NONE = 0, TLHIP_EPI_BIAS = 1, TLHIP_EPI_UNARY = 2 } tlhip_epilogue_kind_t;
+
+#define TLHIP_MAX_EPILOGUE_OPS 4
+
+/* One step of an epilogue chain: EpilogueOp
+ * (src/backend/webgpu/matmul/types.ts:13-24).  BIAS adds input[n] (indexed by
+ * output column); UNARY applies `unary`. */
+typedef struct {
+  int32_t kind;        /* tlhip_epilogue_kind_t */
+  int32_t unary;       /* tlhip_unary_t, for kind == UNARY */
+  const void* input;   /* device [N], for kind == BIAS */
+  int32_t input_dtype; /* tlhip_dtype_t of input */
+  int32_t reserved;
+} tlhip_epilogue_op_t;
+
+/* EpilogueConfig: ops are applied in order to acc*alpha in f32, then the value
+ * is cast to the output dtype (src/schedule/matmul-skeleton.ts:916-966). */
+typedef struct {
+  int32_t n_ops;
+  int32_t reserved;
+  tlhip_epilogue_op_t ops[TLHIP_MAX_EPILOGUE_OPS];
+} tlhip_epilogue_t;
+
+/* A packed weight operand: what BackendTensor.format + .scales describe
+ * (src/backend/types.ts:5-28) for the logical [N,K] Linear weight.
+ *   packed  u32 words, row-major [N, K/4] (int8) or [N, K/8] (int4)
+ *   scales  INT8_GROUPED/INT4_GROUPED: f16 bit patterns [N, K/G], contiguous
+ *           (the reference's two-per-u32 upload, engine.ts:2077-2087, is the
+ *           same bytes);  INT8_ROW: f32 [N] */
+typedef struct {
+  int32_t format;     /* tlhip_format_t */
+  int32_t group_size; /* G along K; ignored for INT8_ROW */
+  int64_t n;
+  int64_t k;
+  const void* packed;
+  const void* scales;
+} tlhip_qweight_t;
+
+typedef struct {
+  char name[64];     /* device name */
+  char arch[32];     /* gcnArchName, e.g. "gfx950:sramecc+:xnack-" */
+  int32_t compute_units;
+  int32_t wavefront_size;
+  int32_t lds_bytes_per_block;
+  int32_t clock_khz;
+  int32_t memory_clock_khz;
+  int32_t memory_bus_bits;
+  int64_t total_memory_bytes;
+  int64_t l2_bytes;
+} tlhip_device_info_t;
+
+/* ---- runtime: what the WebGPU context/queue provides to the reference
+ * backend (src/backend/webgpu/gpu-context.ts; creation.ts:51-87; `read`). ---- */
+int tlhip_init(int device_index);
+int tlhip_shutdown(void);
+const char* tlhip_last_error(void);
+int tlhip_device_info(tlhip_device_info_t* host_out);
+int tlhip_malloc(size_t bytes, void** host_out_ptr);
+int tlhip_free(void* ptr);
+int tlhip_memset(void* ptr, int value, size_t bytes, tlhip_stream_t stream);
+int tlhip_memcpy_h2d(void* dst, const void* host_src, size_t bytes, tlhip_stream_t stream);
+int tlhip_memcpy_d2h(void* host_dst, const void* src, size_t bytes, tlhip_stream_t stream);
+int tlhip_memcpy_d2d(void* dst, const void* src, size_t bytes, tlhip_stream_t stream);
+int tlhip_host_alloc(size_t bytes, void** host_out_ptr); /* pinned */
+int tlhip_host_free(void* host_ptr);
+int tlhip_stream_create(tlhip_stream_t* host_out);
+int tlhip_stream_destroy(tlhip_stream_t stream);
+int tlhip_stream_synchronize(tlhip_stream_t stream);
+int tlhip_event_create(tlhip_event_t* host_out);
+int tlhip_event_destroy(tlhip_event_t ev);
+int tlhip_event_record(tlhip_event_t ev, tlhip_stream_t stream);
+int tlhip_event_synchronize(tlhip_event_t ev);
+int tlhip_event_elapsed_us(tlhip_event_t start, tlhip_event_t stop, double* host_out_us);
+
+/* ---- host-side weight preparation: src/backend/quantize.ts ---- */
+/* f32ToF16Bits (quantize.ts:22-47), including its round-half-up subnormals. */
+uint16_t tlhip_f32_to_f16_bits(float value);
+/* f16BitsToF32 (quantize.ts:50-60). */
+float tlhip_f16_bits_to_f32(uint16_t bits);
+/* quantizeLinearWeight (quantize.ts:77-131).  Host in, host out:
+ * host_packed u32[n*k/4] (overwritten), host_scales u16[n*k/group_size].
+ * Fails if k%4 != 0 or k%group_size != 0, with the reference's messages. */
+int tlhip_quantize_int8_grouped(const float* host_weight, int64_t n, int64_t k, int64_t group_size,
+                                uint32_t* host_packed, uint16_t* host_scales);
+
+/* ---- compute ---- */
+
+/* Explicit dequantisation to f32 [N,K], bit-exact against dequantizeToF32
+ * (quantize.ts:138-156) for INT8_GROUPED and against f32(q*s) for the other
+ * two formats.  Stands in for dispatchDequantizeInt8Grouped
+ * (src/backend/webgpu/matmul/dispatch.ts:949-1037). */
+int tlhip_dequant(const tlhip_qweight_t* w, float* out, tlhip_stream_t stream);
+
+/* Decode GEMV / skinny GEMM with fused dequant: y[m,n] = epilogue(alpha *
+ * sum_k x[m,k] * w[n,k]), 1 <= m <= 16, f32 accumulation.  x is row-major
+ * [m,k] of x_dtype, y row-major [m,n] of y_dtype.  Stands in for
+ * dispatchQuantizedGemvNT (dispatch.ts:875-931), extended to m <= 16, f16
+ * activations/outputs and the epilogue chain.  epilogue may be NULL. */
+int tlhip_gemv(const tlhip_qweight_t* w, const void* x, int x_dtype, int64_t m, void* y,
+               int y_dtype, float alpha, const tlhip_epilogue_t* epilogue, tlhip_stream_t stream);
+
+/* Prefill GEMM with dequant fused into the LDS stage: same contract as
+ * tlhip_gemv for any m >= 1; x must be f16.  Stands in for the explicit
+ * dequant + stock matmul the reference runs when M > 1
+ * (matmul-ops.ts:163-181) with the tiled kernel's epilogue
+ * (src/schedule/matmul-skeleton.ts:738-966). */
+int tlhip_gemm_prefill(const tlhip_qweight_t* w, const void* x, int x_dtype, int64_t m, void* y,
+                       int y_dtype, float alpha, const tlhip_epilogue_t* epilogue,
+                       tlhip_stream_t stream);
+
+/* The matmul seam for a packed B operand: matmulQuantizedB
+ * (matmul-ops.ts:113-182).  Routes small m to the GEMV kernels and larger m to
+ * the prefill GEMM (or, for f32 activations, to GEMV passes of <= 16 rows). */
+int tlhip_matmul_quantized(const tlhip_qweight_t* w, const void* x, int x_dtype, int64_t m,
+                           void* y, int y_dtype, float alpha, const tlhip_epilogue_t* epilogue,
+                           tlhip_stream_t stream);
+
+/* The ops the frontend issues either side of the matmul when nothing is fused
+ * (BackendOps.add / relu / silu / gelu / cast, src/backend/types.ts:340-679;
+ * api.linear adds the bias as a separate op, src/frontend/torchlette.ts:892-894).
+ * bias_add: out[r,c] = in[r,c] + bias[c] over an [m,n] tensor of `dtype`.
+ * unary: out[i] = op(in[i]).  cast: f32 <-> f16.  In-place (out == in) is fine. */
+int tlhip_bias_add(const void* in, int dtype, const void* bias, int bias_dtype, void* out, int64_t m,
+                   int64_t n, tlhip_stream_t stream);
+int tlhip_unary(int op, const void* in, int dtype, void* out, int64_t count, tlhip_stream_t stream);
+int tlhip_cast(const void* in, int in_dtype, void* out, int out_dtype, int64_t count,
+               tlhip_stream_t stream);
+
+/* ---- kernel choice: variant registry + autotuner
+ * (src/backend/webgpu/matmul/variants.ts:54-260; autotune.ts:48-547;
+ * dispatch.ts:60-207, 405-578) ---- */
+
+/* A launch configuration.  variant 0 = "gemv" (VALU dot), 1 = "gemv_mfma"
+ * (skinny MFMA), 2 = "tiled" (prefill MFMA GEMM).  Unused fields are 0. */
+typedef struct {
+  int32_t variant;
+  int32_t p0; /* gemv: lanes per row (16/32/64)   tiled: tile M */
+  int32_t p1; /* gemv: rows per lane-group        tiled: tile N */
+  int32_t p2; /* gemv: waves per workgroup        tiled: tile K */
+  int32_t p3; /* gemv: K-split waves (LDS combine) tiled: waves M */
+  int32_t p4; /* gemv: reserved                   tiled: waves N */
+  int32_t p5;
+  int32_t p6;
+} tlhip_kernel_config_t;
+
+/* As tlhip_matmul_quantized but with an explicit configuration
+ * (dispatchMatmul's explicit `config`, dispatch.ts:171-176).  Fails if the
+ * configuration is not applicable to the shape. */
+int tlhip_matmul_quantized_config(const tlhip_qweight_t* w, const void* x, int x_dtype, int64_t m,
+                                  void* y, int y_dtype, float alpha,
+                                  const tlhip_epilogue_t* epilogue,
+                                  const tlhip_kernel_config_t* config, tlhip_stream_t stream);
+
+/* Number of candidate configurations for a problem, and the i-th one
+ * (variant.candidates, variants.ts:54-90). */
+int tlhip_candidate_count(const tlhip_qweight_t* w, int x_dtype, int64_t m, int y_dtype,
+                          int* host_out_count);
+int tlhip_candidate_get(const tlhip_qweight_t* w, int x_dtype, int64_t m, int y_dtype, int index,
+                        tlhip_kernel_config_t* host_out);
+/* The configuration tlhip_matmul_quantized would use now (tuned winner if
+ * cached, else the heuristic default) — selectMatmulChoice, dispatch.ts:171-192. */
+int tlhip_selected_config(const tlhip_qweight_t* w, int x_dtype, int64_t m, int y_dtype,
+                          tlhip_kernel_config_t* host_out);
+
+/* setAutotuneEnabled / isAutotuneEnabled (dispatch.ts:128-141).  Also switched
+ * on by the environment variable TORCHLETTE_AUTOTUNE=1 (dispatch.ts:559). */
+int tlhip_set_autotune_enabled(int enabled);
+int tlhip_is_autotune_enabled(void);
+/* Benchmark every candidate for this problem (2 warm-up + 3 timed launches
+ * each, median, as dispatch.ts:324-397) and cache the winner under the key
+ * (m, n, k, format, group, x dtype, y dtype).  Runs on the library stream. */
+int tlhip_autotune(const tlhip_qweight_t* w, const void* x, int x_dtype, int64_t m, void* y,
+                   int y_dtype, double* host_out_best_us);
+/* Backend.pretuneMatmulShapes (src/backend/types.ts:688): [m,n,k] triples.
+ * The hook carries no operand format, so it only records shape hints; tuning
+ * happens at first dispatch of a matching packed operand when enabled. */
+int tlhip_pretune_matmul_shapes(const int64_t* host_mnk, int count);
+/* exportTuningCache / importTuningCache (autotune.ts:309-329): JSON text.
+ * export writes at most cap bytes (NUL-terminated) and the needed size. */
+int tlhip_tune_cache_export(char* host_buf, size_t cap, size_t* host_out_needed);
+int tlhip_tune_cache_import(const char* host_json);
+int tlhip_tune_cache_clear(void);
+
+/* Dispatch counters, the reference's test hooks (dispatch.ts:79-83, 832-864,
+ * 943-947): "quant_gemv_dispatches", "quant_gemm_dispatches",
+ * "dequant_dispatches", "autotune_runs".  Unknown names return 0. */
+uint64_t tlhip_counter(const char* name);
+int tlhip_counters_reset(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TLHIP_H */

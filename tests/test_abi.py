@@ -1,0 +1,142 @@
+"""CPU-side checks of the boundary: the shared library loads, exports every
+symbol include/tlhip.h declares, fails loudly without a GPU, and its host-side
+functions (f16 codec, quantizer) match the oracle bit for bit."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+import torchlette_amd as T
+from oracle import quant_oracle as O
+from torchlette_amd import _lib as L
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "tlhip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(tlhip_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = L.load()
+    names = declared_symbols()
+    assert len(names) >= 40
+    for name in names:
+        assert hasattr(lib, name), name
+    # and the binding declares a signature for each of them
+    assert sorted(L.SIGNATURES) == names
+
+
+def test_struct_sizes_match_the_header_layout():
+    assert ctypes.sizeof(L.EpilogueOp) == 24
+    assert ctypes.sizeof(L.Epilogue) == 8 + 4 * 24
+    assert ctypes.sizeof(L.QWeight) == 40
+    assert ctypes.sizeof(L.KernelConfig) == 32
+    assert ctypes.sizeof(L.DeviceInfo) == 64 + 32 + 6 * 4 + 2 * 8
+
+
+@pytest.mark.skipif(os.path.exists("/dev/kfd"), reason="GPU present")
+def test_compute_fails_loudly_without_a_gpu():
+    with pytest.raises(L.TlhipError, match="no HIP device|no CPU fallback"):
+        T.HipBackend(0)
+    qw = L.QWeight(L.FMT_INT4_GROUPED, 32, 4, 32, 16, 16)
+    rc = L.load().tlhip_dequant(ctypes.byref(qw), 16, None)
+    assert rc == 3 and "not initialised" in L.last_error()
+    rc = L.load().tlhip_matmul_quantized(ctypes.byref(qw), 16, L.F16, 1, 16, L.F16, 1.0, None, None)
+    assert rc == 3
+
+
+def test_host_f16_codec_matches_oracle_everywhere_it_matters():
+    lib = L.load()
+    bits = np.arange(65536, dtype=np.uint16)
+    ref = O.f16_bits_to_f32(bits)
+    got = np.array([lib.tlhip_f16_bits_to_f32(int(b)) for b in bits], np.float32)
+    nan = np.isnan(ref)
+    assert np.array_equal(np.isnan(got), nan)
+    assert np.array_equal(got[~nan].view(np.uint32), ref[~nan].view(np.uint32))
+    rng = np.random.default_rng(1)
+    u = np.concatenate([
+        rng.integers(0, 2 ** 32, 20000, dtype=np.uint64).astype(np.uint32),
+        np.arange(102 << 23, 114 << 23, 40009, dtype=np.uint32),          # subnormal range + first normal
+        (np.arange(113 << 23, 143 << 23, 1 << 13, dtype=np.uint32) | 0x1000)[::7],  # exact ties
+        np.array([0, 0x80000000, 0x7F800000, 0xFF800000, 0x7FC00000, 0x33000000, 0x32FFFFFF,
+                  0x477FE000, 0x477FEFFF, 0x477FF000], np.uint32),
+    ])
+    x = u.view(np.float32)
+    want = O.f32_to_f16_bits(x)
+    got = np.array([lib.tlhip_f32_to_f16_bits(float(v)) if not np.isnan(v) else
+                    lib.tlhip_f32_to_f16_bits(float("nan")) for v in x], np.uint16)
+    ok = ~np.isnan(x)
+    assert np.array_equal(got[ok], want[ok])
+    assert all((g & 0x7FFF) == 0x7C00 for g in got[~ok])
+
+
+@pytest.mark.parametrize("n,k,g", [(1, 4, 4), (3, 64, 64), (64, 256, 64), (17, 384, 128), (300, 1024, 64)])
+def test_host_quantizer_matches_oracle(n, k, g):
+    rng = np.random.default_rng(n * 1000 + k)
+    w = (rng.standard_normal((n, k)) * np.exp(rng.uniform(-8, 3, (n, 1)))).astype(np.float32)
+    if n > 2:
+        w[1, : g] = 0.0                      # all-zero group
+        w[2, 0] = np.float32(1.0004)         # scale rounds below abs-max -> clamp
+    p, s = T.quantizeLinearWeight(w, n, k, g)
+    p2, s2 = O.quantize_int8_grouped(w, n, k, g)
+    assert np.array_equal(s, s2) and np.array_equal(p, p2)
+
+
+def test_host_quantizer_half_integers_nan_inf_and_threads():
+    w = np.array([127.0, 2.5, -2.5, -0.5, 0.5, 1.5, -1.5, -126.5], np.float32)
+    p, s = T.quantizeLinearWeight(w, 1, 8, 8)
+    assert O.np_unpack_int8(p, 1, 8).ravel().tolist() == [127, 3, -2, 0, 1, 2, -1, -126]
+    w = np.zeros(12, np.float32)
+    w[4:8] = [np.nan, 1.0, -0.25, np.nan]
+    w[8:12] = [np.inf, 1.0, -1.0, 0.0]
+    p, s = T.quantizeLinearWeight(w, 1, 12, 4)
+    p2, s2 = O.quantize_int8_grouped(w, 1, 12, 4)
+    assert np.array_equal(p, p2) and np.array_equal(s, s2)
+    # large enough to take the multi-threaded path
+    rng = np.random.default_rng(9)
+    w = rng.standard_normal((2048, 2048)).astype(np.float32)
+    p, s = T.quantizeLinearWeight(w, 2048, 2048, 64)
+    p2, s2 = O.quantize_int8_grouped(w, 2048, 2048, 64)
+    assert np.array_equal(p, p2) and np.array_equal(s, s2)
+
+
+def test_host_quantizer_errors_carry_the_reference_messages():
+    w = np.zeros(16, np.float32)
+    with pytest.raises(L.TlhipError, match="expected 32 elements, got 16"):
+        T.quantizeLinearWeight(w, 4, 8, 4)
+    with pytest.raises(L.TlhipError, match="K=6 must be divisible by 4"):
+        T.quantizeLinearWeight(np.zeros(12, np.float32), 2, 6, 2)
+    with pytest.raises(L.TlhipError, match="K=8 must be divisible by groupSize=3"):
+        T.quantizeLinearWeight(w, 2, 8, 3)
+
+
+def test_tuning_cache_json_round_trip_and_autotune_toggle():
+    T.resetMatmulState()
+    assert not T.isAutotuneEnabled()
+    T.setAutotuneEnabled(True)
+    T.setAutotuneEnabled(True)
+    assert T.isAutotuneEnabled()
+    T.setAutotuneEnabled(False)  # resets the nesting counter (dispatch.ts:128-134)
+    assert not T.isAutotuneEnabled()
+    text = '{"version":1,"entries":{"1_4096_4096_int4-grouped_g32_f16_f16":[0,64,1,4,1,0,0,0],' \
+           '"512_12288_4096_int4-grouped_g32_f16_f16":[2,128,128,64,2,2,0,0]}}'
+    T.importTuningCache(text)
+    out = T.exportTuningCache()
+    assert out == text
+    T.clearTuningCache()
+    assert T.exportTuningCache() == '{"version":1,"entries":{}}'
+    with pytest.raises(L.TlhipError, match="entries"):
+        T.importTuningCache("{}")
+
+
+def test_format_names_resolve_like_the_reference():
+    f = T.resolveWeightFormat("int8-64")
+    assert f.elementType == "f16" and f.packing == T.QuantPacking("int8-grouped", 64, "f16")
+    assert T.resolveWeightFormat("int8-128", "f32").packing.groupSize == 128
+    assert T.resolveWeightFormat("int4-32").packing == T.QuantPacking("int4-grouped", 32, "f16")
+    assert T.resolveWeightFormat("int8-row").packing.scheme == "int8-row"

@@ -1,0 +1,249 @@
+"""GPU parity: decode GEMV / skinny GEMM over packed weights vs the oracle
+(bit-exact dequant -> CPU-backend matmul -> add -> activation).
+
+Tolerance: rel-L2 <= 1e-3 (the stated bar), and for the reference's own format
+the probe's bar max |d|/max(1,|ref|) <= 5e-4 (probe-quant-gemv.ts:182-187)."""
+import json
+import os
+import zlib
+
+import numpy as np
+import pytest
+
+import torchlette_amd as T
+from oracle import quant_oracle as O
+from torchlette_amd import _lib as L
+from helpers import f16_round, fmt_name, make_weight, make_x, per_row_err, rel_l2
+
+pytestmark = pytest.mark.gpu
+REL_L2_TOL = 1e-3
+PROBE_TOL = 5e-4
+GOLD = os.path.join(os.path.dirname(__file__), "golden")
+
+
+@pytest.fixture(scope="module")
+def be():
+    return T.getBackend()
+
+
+def run_linear(be, fmt, packed, scales, n, k, g, x, element, bias=None, act=None, fused=False, config=None):
+    xdt = "f16" if x.dtype == np.float16 else "f32"
+    w = be.createQuantizedWeight(packed, scales, n, k, T.resolveWeightFormat(fmt_name(fmt, g), element))
+    xt = be.ops.tensorFromArray(x, list(x.shape), xdt)
+    bt = None
+    if bias is not None:
+        bt = be.ops.tensorFromArray(bias, [n], "f16" if bias.dtype == np.float16 else "f32")
+    y = be.linear(xt, w, bt, act, fused=fused, config=config)
+    out = y.numpy()
+    y.destroy()
+    xt.destroy()
+    return out
+
+
+@pytest.mark.parametrize("m", [1, 2, 3, 4, 5, 8, 16])
+@pytest.mark.parametrize("fmt,n,k,g,xdt,element", [
+    ("int4-grouped", 2048, 1024, 32, "f16", "f16"),
+    ("int4-grouped", 1024, 3072, 32, "f16", "f16"),
+    ("int8-row", 1024, 1024, 0, "f32", "f32"),
+    ("int8-row", 1536, 2304, 0, "f16", "f32"),
+    ("int8-grouped", 512, 1024, 64, "f32", "f32"),
+    ("int8-grouped", 768, 2048, 128, "f16", "f16"),
+])
+def test_gemv_matches_oracle(be, fmt, n, k, g, xdt, element, m):
+    rng = np.random.default_rng(zlib.crc32(repr((fmt, n, k, m)).encode()))
+    packed, scales, deq = make_weight(fmt, n, k, g, rng)
+    x = make_x(m, k, xdt, rng)
+    before = T.getQuantGemvDispatchCount()
+    got = run_linear(be, fmt, packed, scales, n, k, g, x, element)
+    assert T.getQuantGemvDispatchCount() == before + 1
+    want = O.linear(x.astype(np.float32), deq)
+    assert got.shape == (m, n)
+    assert got.dtype == (np.float16 if (xdt == "f16" and element == "f16") else np.float32)
+    tol = REL_L2_TOL
+    assert rel_l2(got, want) <= tol, rel_l2(got, want)
+    if got.dtype == np.float32:
+        assert rel_l2(got, want) <= 2e-6  # f32 accumulate of exact products: order noise only
+
+
+@pytest.mark.parametrize("fmt,n,k,g", [
+    ("int4-grouped", 4096, 4096, 32), ("int4-grouped", 12288, 4096, 32), ("int4-grouped", 4096, 12288, 32),
+])
+@pytest.mark.parametrize("m", [1, 4, 16])
+def test_qwen3_8b_shapes(be, fmt, n, k, g, m):
+    rng = np.random.default_rng(n + k + m)
+    packed, scales, deq = make_weight(fmt, n, k, g, rng)
+    x = make_x(m, k, "f16", rng)
+    got = run_linear(be, fmt, packed, scales, n, k, g, x, "f16")
+    want = O.linear(x.astype(np.float32), deq, threads=8)
+    assert rel_l2(got, want) <= REL_L2_TOL
+    # f16 output rounding only: within one f16 ulp of the oracle
+    assert per_row_err(got, want) <= 2e-3
+
+
+def test_every_candidate_config_gives_the_same_answer(be):
+    rng = np.random.default_rng(42)
+    n, k, g, m = 777, 2048, 32, 3   # ragged N: every tail path is exercised
+    packed, scales, deq = make_weight("int4-grouped", n, k, g, rng)
+    x = make_x(m, k, "f16", rng)
+    want = O.linear(x.astype(np.float32), deq)
+    w = be.createQuantizedWeight(packed, scales, n, k, T.resolveWeightFormat("int4-32", "f32"))
+    cands = be.candidates(w, "f16", m, "f32")
+    assert len(cands) >= 20
+    xt = be.ops.tensorFromArray(x, [m, k], "f16")
+    for c in cands:
+        y = be.linear(xt, w, config=c)
+        got = y.numpy()
+        y.destroy()
+        assert rel_l2(got, want) <= 2e-6, c.as_tuple()
+
+
+@pytest.mark.parametrize("fmt,g,xdt", [("int8-grouped", 64, "f32"), ("int8-row", 0, "f16"), ("int4-grouped", 64, "f32")])
+def test_candidates_other_formats(be, fmt, g, xdt):
+    rng = np.random.default_rng(43)
+    n, k, m = 515, 1280, 2
+    packed, scales, deq = make_weight(fmt, n, k, g, rng)
+    x = make_x(m, k, xdt, rng)
+    want = O.linear(x.astype(np.float32), deq)
+    w = be.createQuantizedWeight(packed, scales, n, k, T.resolveWeightFormat(fmt_name(fmt, g), "f32"))
+    xt = be.ops.tensorFromArray(x, [m, k], xdt)
+    for c in be.candidates(w, xdt, m, "f32")[::3]:
+        y = be.linear(xt, w, config=c)
+        got = y.numpy()
+        y.destroy()
+        assert rel_l2(got, want) <= 2e-6, c.as_tuple()
+
+
+@pytest.mark.parametrize("act", [None, "relu", "silu", "gelu", "gelu_erf", "sigmoid", "tanh"])
+@pytest.mark.parametrize("fused", [False, True])
+def test_bias_and_activation_fused_and_unfused(be, act, fused):
+    rng = np.random.default_rng(7)
+    n, k, g, m = 1024, 1024, 32, 4
+    packed, scales, deq = make_weight("int4-grouped", n, k, g, rng)
+    x = make_x(m, k, "f16", rng, std=0.5)
+    bias = f16_round(rng.standard_normal(n) * 0.1)
+    got = run_linear(be, "int4-grouped", packed, scales, n, k, g, x, "f16", bias=bias, act=act, fused=fused)
+    want = O.linear(x.astype(np.float32), deq, bias.astype(np.float32), act or "none")
+    assert got.dtype == np.float16
+    assert rel_l2(got, want) <= REL_L2_TOL
+    # f32 output shows the epilogue arithmetic without the f16 store
+    got32 = run_linear(be, "int4-grouped", packed, scales, n, k, g, x, "f32", bias=bias, act=act, fused=fused)
+    assert rel_l2(got32, want) <= 1e-5
+
+
+def test_reference_probe_shapes_int8_grouped(be):
+    """The quant GEMV probe's generator, shapes and bar (probe-quant-gemv.ts),
+    minus its lm_head-sized case which is covered below at full N."""
+    cases = json.load(open(os.path.join(GOLD, "quant_probe_cases.json")))["gemv_probe"]
+    draw = O.make_lcg(cases["seed"])
+    for g in cases["group_sizes"]:
+        for n, k in cases["shapes_nk"]:
+            w = draw(n * k).astype(np.float32)
+            a = draw(k).astype(np.float32)
+            if n > 4096:
+                continue  # keeps the LCG stream in step with the probe; big case tested separately
+            packed, scales = T.quantizeLinearWeight(w, n, k, g)
+            deq = O.dequant_int8_grouped(packed, scales, n, k, g)
+            ref = deq.astype(np.float64) @ a.astype(np.float64)
+            before = T.getQuantGemvDispatchCount()
+            got = run_linear(be, "int8-grouped", packed, scales, n, k, g, a.reshape(1, k), "f32")
+            assert T.getQuantGemvDispatchCount() - before == 1
+            assert per_row_err(got, ref) <= cases["per_row_tol"], (n, k, g)
+            assert per_row_err(got, O.linear(a.reshape(1, k), deq)) <= cases["per_row_tol"]
+
+
+def test_lm_head_sized_n(be):
+    """N = 151936 (the probe's lm_head case) and the Gemma-shaped 256000 x 2304 int8-row."""
+    rng = np.random.default_rng(3)
+    n, k, g = 151936, 2048, 64
+    q = rng.integers(-127, 128, (n, k)).astype(np.int8)
+    packed = O.np_pack_int8(q)
+    scales = f16_round(rng.uniform(0.5, 1.0, n * k // g)).view(np.uint16)
+    a = make_x(1, k, "f32", rng)
+    got = run_linear(be, "int8-grouped", packed, scales, n, k, g, a, "f32")
+    deq = O.dequant_int8_grouped(packed, scales, n, k, g)
+    want = O.linear(a, deq, threads=8)
+    assert per_row_err(got, want) <= PROBE_TOL
+    del deq
+    n, k = 256000, 2304
+    q = rng.integers(-127, 128, (n, k)).astype(np.int8)
+    packed = O.np_pack_int8(q)
+    rs = rng.uniform(0.002, 0.01, n).astype(np.float32)
+    for m in (1, 8):
+        x = make_x(m, k, "f16", rng)
+        got = run_linear(be, "int8-row", packed, rs, n, k, 0, x, "f32")
+        want = O.linear(x.astype(np.float32), O.dequant_int8_row(packed, rs, n, k), threads=8)
+        assert rel_l2(got, want) <= 1e-5
+
+
+def test_linearity_and_row_permutation_at_full_size(be):
+    """Size-independent properties at a config-3 shape: y(x1+x2) = y(x1)+y(x2)
+    for f16-exact sums, and permuting weight rows permutes outputs."""
+    rng = np.random.default_rng(11)
+    n, k, g = 12288, 4096, 32
+    packed, scales, _ = make_weight("int4-grouped", n, k, g, rng)
+    x1 = f16_round(rng.integers(-8, 9, (1, k)) / 8.0)
+    x2 = f16_round(rng.integers(-8, 9, (1, k)) / 8.0)
+    y1 = run_linear(be, "int4-grouped", packed, scales, n, k, g, x1, "f32")
+    y2 = run_linear(be, "int4-grouped", packed, scales, n, k, g, x2, "f32")
+    y12 = run_linear(be, "int4-grouped", packed, scales, n, k, g, f16_round(x1.astype(np.float32) + x2), "f32")
+    assert rel_l2(y12, y1 + y2) <= 1e-6
+    perm = rng.permutation(n)
+    pp = packed.reshape(n, k // 8)[perm].reshape(-1)
+    sp = scales.reshape(n, k // g)[perm].reshape(-1)
+    yp = run_linear(be, "int4-grouped", pp, sp, n, k, g, x1, "f32")
+    assert np.array_equal(yp[0], y1[0][perm])
+
+
+def test_alpha_zero_weights_and_extreme_values(be):
+    rng = np.random.default_rng(5)
+    n, k, g = 256, 512, 32
+    q = np.zeros((n, k), np.int8)
+    q[::2] = -8
+    q[1::2] = 7
+    packed = O.np_pack_int4(q)
+    scales = f16_round(np.full(n * k // g, 0.05)).view(np.uint16)
+    x = f16_round(np.ones((2, k)))
+    got = run_linear(be, "int4-grouped", packed, scales, n, k, g, x, "f32")
+    want = O.linear(x.astype(np.float32), O.dequant_int4_grouped(packed, scales, n, k, g))
+    assert rel_l2(got, want) <= 1e-6
+    # int8 extremes incl. -128 (never produced by the quantizer, representable in the byte)
+    q8 = rng.choice(np.array([-128, -127, 127, 0], np.int8), (n, k))
+    p8 = O.np_pack_int8(q8)
+    s8 = f16_round(rng.uniform(0.5, 2, n * k // 64)).view(np.uint16)
+    x = make_x(1, k, "f32", rng)
+    got = run_linear(be, "int8-grouped", p8, s8, n, k, 64, x, "f32")
+    want = O.linear(x, O.dequant_int8_grouped(p8, s8, n, k, 64))
+    assert rel_l2(got, want) <= 2e-6
+
+
+def test_seam_errors(be):
+    rng = np.random.default_rng(1)
+    packed, scales, _ = make_weight("int4-grouped", 64, 128, 32, rng)
+    w = be.createQuantizedWeight(packed, scales, 64, 128, T.resolveWeightFormat("int4-32"))
+    x = be.ops.tensorFromArray(np.zeros((1, 96), np.float16), [1, 96], "f16")
+    with pytest.raises(ValueError, match="matmul dimension mismatch"):
+        be.linear(x, w)
+    with pytest.raises(ValueError, match="packed length"):
+        be.createQuantizedWeight(packed[:-1], scales, 64, 128, T.resolveWeightFormat("int4-32"))
+    with pytest.raises(ValueError, match="scales length"):
+        be.createQuantizedWeight(packed, scales[:-1], 64, 128, T.resolveWeightFormat("int4-32"))
+    with pytest.raises(ValueError, match="format.packing is required"):
+        be.createQuantizedWeight(packed, scales, 64, 128, T.StorageFormat("f16"))
+    bad = T.HipTensor(be, [64, 128], "f16", w.ptr, w.nbytes, False, None, w.format, None)
+    with pytest.raises(ValueError, match="missing packing/scales"):
+        be.ops.matmul(x, be.ops.transpose(bad))
+    with pytest.raises(L.TlhipError, match="config not applicable"):
+        x2 = be.ops.tensorFromArray(np.zeros((1, 128), np.float16), [1, 128], "f16")
+        be.linear(x2, w, config=L.KernelConfig.of(0, 48, 1, 4, 1))
+    with pytest.raises(ValueError, match="explicitly"):
+        w.numpy()
+
+
+def test_transpose_view_carries_format_and_scales(be):
+    rng = np.random.default_rng(2)
+    packed, scales, _ = make_weight("int8-grouped", 32, 64, 64, rng)
+    w = be.createQuantizedWeight(packed, scales, 32, 64, T.resolveWeightFormat("int8-64"))
+    assert w.shape == [32, 64] and w.dtype == "f16" and w.strides == [64, 1]
+    wt = be.ops.transpose(w)
+    assert wt.shape == [64, 32] and wt.strides == [1, 64]
+    assert wt.format is w.format and wt.scales is w.scales and wt.ownsBuffer is False

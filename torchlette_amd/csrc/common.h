@@ -1,0 +1,80 @@
+// Internal declarations shared by the translation units of libtlhip.so.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+
+#include "tlhip.h"
+
+namespace tlhip {
+
+// Per-thread error text behind tlhip_last_error().
+int set_error(int code, const char* fmt, ...);
+void clear_error();
+
+bool is_initialised();
+hipStream_t resolve_stream(tlhip_stream_t s);  // NULL -> library stream
+int device_cu_count();
+
+#define TLHIP_CHECK_HIP(expr)                                                            \
+  do {                                                                                   \
+    hipError_t _e = (expr);                                                              \
+    if (_e != hipSuccess)                                                                \
+      return ::tlhip::set_error(TLHIP_ERR_DEVICE, "%s failed: %s", #expr, hipGetErrorString(_e)); \
+  } while (0)
+
+#define TLHIP_REQUIRE_INIT()                                                             \
+  do {                                                                                   \
+    if (!::tlhip::is_initialised())                                                      \
+      return ::tlhip::set_error(TLHIP_ERR_STATE, "tlhip: not initialised (call tlhip_init)"); \
+  } while (0)
+
+// Epilogue as the kernels take it (by value, in kernel arguments).
+struct DevEpilogue {
+  int n_ops;
+  int kind[TLHIP_MAX_EPILOGUE_OPS];
+  int unary[TLHIP_MAX_EPILOGUE_OPS];
+  int input_dtype[TLHIP_MAX_EPILOGUE_OPS];
+  const void* input[TLHIP_MAX_EPILOGUE_OPS];
+};
+
+// Validated problem description handed to the launchers.
+struct Problem {
+  int format;
+  int group_size;
+  int64_t n, k, m;
+  const void* packed;
+  const void* scales;
+  const void* x;
+  int x_dtype;
+  void* y;
+  int y_dtype;
+  float alpha;
+  DevEpilogue epi;
+};
+
+// Validation shared by every compute entry point.  Fills `p` on success.
+int make_problem(const tlhip_qweight_t* w, const void* x, int x_dtype, int64_t m, void* y,
+                 int y_dtype, float alpha, const tlhip_epilogue_t* epilogue, Problem* p,
+                 const char* who);
+int validate_weight(const tlhip_qweight_t* w, const char* who);
+
+// Launchers (each returns a TLHIP_* code; launch errors are reported).
+int launch_dequant(const tlhip_qweight_t& w, float* out, hipStream_t stream);
+bool gemv_config_applicable(const Problem& p, const tlhip_kernel_config_t& c, const char** why);
+int launch_gemv(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t stream);
+bool gemm_config_applicable(const Problem& p, const tlhip_kernel_config_t& c, const char** why);
+int launch_gemm(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t stream);
+
+// Counters.
+void count_gemv_dispatch();
+void count_gemm_dispatch();
+void count_dequant_dispatch();
+void count_autotune_run();
+
+enum { VARIANT_GEMV = 0, VARIANT_GEMV_MFMA = 1, VARIANT_TILED = 2 };
+
+}  // namespace tlhip

@@ -1,0 +1,131 @@
+// Device helpers shared by the GEMV and GEMM kernels: the epilogue chain, f16
+// scale decoding, int4/int8 unpacking into packed f16 pairs, and lane
+// reductions over DPP.
+#pragma once
+
+#include "common.h"
+
+namespace tlhip {
+
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+
+__device__ __forceinline__ float half_bits_to_float(uint32_t h) {
+  return (float)__builtin_bit_cast(_Float16, (uint16_t)h);
+}
+
+// ---------------------------------------------------------------- epilogue
+// Formulas: relu/silu/sigmoid from src/ops/semantic/catalog.ts:81-109, gelu
+// (tanh form) from composite.ts:40-51, gelu_erf with the Abramowitz-Stegun
+// polynomial of erf.ts:28-56 — evaluated in f32 as the reference's GPU
+// epilogues are (src/schedule/matmul-skeleton.ts:916-966).
+__device__ __forceinline__ float apply_unary(int op, float v) {
+  switch (op) {
+    case TLHIP_UNARY_RELU: return v > 0.f ? v : 0.f;
+    case TLHIP_UNARY_SILU: return v / (1.f + expf(-v));
+    case TLHIP_UNARY_SIGMOID: return 1.f / (1.f + expf(-v));
+    case TLHIP_UNARY_TANH: return tanhf(v);
+    case TLHIP_UNARY_GELU_TANH:
+      return (0.5f * v) * (1.f + tanhf(0.7978845608f * (v + 0.044715f * (v * (v * v)))));
+    case TLHIP_UNARY_GELU_ERF: {
+      const float u = v * 0.70710678118654752f;
+      const float ax = fabsf(u);
+      const float t = 1.f / (1.f + 0.3275911f * ax);
+      const float poly =
+          ((((1.061405429f * t - 1.453152027f) * t + 1.421413741f) * t - 0.284496736f) * t + 0.254829592f) * t;
+      const float e = 1.f - poly * expf(-ax * ax);
+      return (0.5f * v) * (1.f + (u < 0.f ? -e : e));
+    }
+    default: return v;
+  }
+}
+
+// acc*alpha, then the ops in order; `col` is the output column n.
+__device__ __forceinline__ float apply_epilogue(const DevEpilogue& ep, float v, int64_t col) {
+  for (int i = 0; i < ep.n_ops; ++i) {
+    if (ep.kind[i] == TLHIP_EPI_BIAS) {
+      float b;
+      if (ep.input_dtype[i] == TLHIP_F16) b = (float)((const _Float16*)ep.input[i])[col];
+      else b = ((const float*)ep.input[i])[col];
+      v += b;
+    } else if (ep.kind[i] == TLHIP_EPI_UNARY) {
+      v = apply_unary(ep.unary[i], v);
+    }
+  }
+  return v;
+}
+
+__device__ __forceinline__ void store_out(void* y, int y_dtype, int64_t idx, float v) {
+  if (y_dtype == TLHIP_F16) ((_Float16*)y)[idx] = (_Float16)v;
+  else ((float*)y)[idx] = v;
+}
+
+// ------------------------------------------------------------------ unpack
+// int4: one u32 holds nibbles j=0..7 for k = 8*word + j, two's complement.
+// XOR 0x8 turns a nibble into q+8; OR-ing it into the mantissa of 1024.0h
+// (0x6400) gives the f16 value 1024+q+8 (or 1024+16*(q+8) for a nibble at bit
+// 4), from which q is recovered exactly by one packed add or fma.
+// Output order: pairs (k0,k4) (k1,k5) (k2,k6) (k3,k7).
+__device__ __forceinline__ void unpack_int4_word(uint32_t w, half2_t out[4]) {
+  const uint32_t t = w ^ 0x88888888u;
+  const uint32_t lo = t, hi = t >> 8;
+  const half2_t sub_lo = {(_Float16)-1032.f, (_Float16)-1032.f};  // -(1024 + 8)
+  const half2_t mul_hi = {(_Float16)0.0625f, (_Float16)0.0625f};  // 1/16
+  const half2_t sub_hi = {(_Float16)-72.f, (_Float16)-72.f};      // -(1024/16 + 8)
+  const uint32_t a0 = (lo & 0x000f000fu) | 0x64006400u;
+  const uint32_t a1 = (lo & 0x00f000f0u) | 0x64006400u;
+  const uint32_t a2 = (hi & 0x000f000fu) | 0x64006400u;
+  const uint32_t a3 = (hi & 0x00f000f0u) | 0x64006400u;
+  out[0] = __builtin_bit_cast(half2_t, a0) + sub_lo;
+  out[1] = __builtin_bit_cast(half2_t, a1) * mul_hi + sub_hi;
+  out[2] = __builtin_bit_cast(half2_t, a2) + sub_lo;
+  out[3] = __builtin_bit_cast(half2_t, a3) * mul_hi + sub_hi;
+}
+
+// The matching order for activations: 8 consecutive f16 (one 16-byte load)
+// rearranged to (x0,x4) (x1,x5) (x2,x6) (x3,x7).
+__device__ __forceinline__ u32x4 permute_x_for_int4(u32x4 v) {
+  u32x4 r;
+  r.x = __builtin_amdgcn_perm(v.z, v.x, 0x05040100u);  // lo16(x) | lo16(z) << 16 : (x0, x4)
+  r.y = __builtin_amdgcn_perm(v.z, v.x, 0x07060302u);  // hi16(x) | hi16(z) << 16 : (x1, x5)
+  r.z = __builtin_amdgcn_perm(v.w, v.y, 0x05040100u);  // (x2, x6)
+  r.w = __builtin_amdgcn_perm(v.w, v.y, 0x07060302u);  // (x3, x7)
+  return r;
+}
+
+// int8: bytes b0..b3 hold k = 4*word + 0..3.  XOR 0x80 gives q+128; placed in
+// the low mantissa byte of 1024.0h it reads 1024+q+128.  Natural pair order.
+__device__ __forceinline__ void unpack_int8_word(uint32_t w, half2_t out[2]) {
+  const uint32_t t = w ^ 0x80808080u;
+  const half2_t sub = {(_Float16)-1152.f, (_Float16)-1152.f};
+  // v_perm_b32 selects bytes from {src0 (bytes 7..4), src1 (bytes 3..0)}
+  const uint32_t a0 = __builtin_amdgcn_perm(0x64646464u, t, 0x04010400u);  // 0x64,b1,0x64,b0
+  const uint32_t a1 = __builtin_amdgcn_perm(0x64646464u, t, 0x04030402u);  // 0x64,b3,0x64,b2
+  out[0] = __builtin_bit_cast(half2_t, a0) + sub;
+  out[1] = __builtin_bit_cast(half2_t, a1) + sub;
+}
+
+// ------------------------------------------------------------- reductions
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float v) {
+  const int moved = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true);
+  return v + __builtin_bit_cast(float, moved);
+}
+
+// Sum over groups of `lanes` consecutive lanes (16, 32 or 64); every lane of a
+// group ends with the group's sum.
+__device__ __forceinline__ float group_sum(float v, int lanes) {
+  v = dpp_add<0xB1>(v);   // quad_perm [1,0,3,2]
+  v = dpp_add<0x4E>(v);   // quad_perm [2,3,0,1]
+  v = dpp_add<0x141>(v);  // row_half_mirror
+  v = dpp_add<0x140>(v);  // row_mirror
+  if (lanes >= 32) v += __shfl_xor(v, 16);
+  if (lanes >= 64) v += __shfl_xor(v, 32);
+  return v;
+}
+
+}  // namespace tlhip

@@ -1,0 +1,515 @@
+// The matmul seam for packed weights and the kernel-choice machinery around it.
+//
+// Mirrors, for this path only:
+//  * matmulQuantizedB's routing (src/backend/webgpu/ops/matmul-ops.ts:113-182):
+//    the operand format is read here and nowhere above;
+//  * the variant registry / selection order of
+//    src/backend/webgpu/matmul/dispatch.ts:171-192: explicit config, then the
+//    per-shape tuned winner (re-gated on applicability), then the first
+//    applicable variant's heuristic default;
+//  * the autotuner of dispatch.ts:405-547 (2 warm-up + 3 timed runs per
+//    candidate, median) with a per-exact-shape cache that, unlike the
+//    reference's m_n_k_dtype key, also carries the operand format, because the
+//    winner differs per packing;
+//  * exportTuningCache / importTuningCache (autotune.ts:309-329) as JSON text.
+#include <algorithm>
+#include <array>
+#include <cstdlib>
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <sstream>
+#include <string>
+#include <vector>
+
+#include "common.h"
+
+namespace tlhip {
+namespace {
+
+std::mutex g_tune_mutex;
+std::map<std::string, tlhip_kernel_config_t> g_tuned;  // per exact problem key
+std::vector<std::array<int64_t, 3>> g_shape_hints;
+int g_autotune_counter = 0;
+bool g_autotuning = false;  // no recursive tuning (dispatch.ts autotuningInProgress)
+
+bool is_pow2(int64_t v) { return v > 0 && (v & (v - 1)) == 0; }
+
+const char* format_name(int f) {
+  switch (f) {
+    case TLHIP_FMT_INT8_GROUPED: return "int8-grouped";
+    case TLHIP_FMT_INT8_ROW: return "int8-row";
+    case TLHIP_FMT_INT4_GROUPED: return "int4-grouped";
+  }
+  return "?";
+}
+
+std::string problem_key(const Problem& p) {
+  char buf[160];
+  snprintf(buf, sizeof buf, "%lld_%lld_%lld_%s_g%d_%s_%s", (long long)p.m, (long long)p.n, (long long)p.k,
+           format_name(p.format), p.format == TLHIP_FMT_INT8_ROW ? 0 : p.group_size,
+           p.x_dtype == TLHIP_F16 ? "f16" : "f32", p.y_dtype == TLHIP_F16 ? "f16" : "f32");
+  return buf;
+}
+
+bool env_autotune() {
+  const char* e = getenv("TORCHLETTE_AUTOTUNE");
+  return e && !strcmp(e, "1");
+}
+
+tlhip_kernel_config_t gemv_cfg(int lpr, int r, int waves, int kw) {
+  tlhip_kernel_config_t c;
+  memset(&c, 0, sizeof c);
+  c.variant = VARIANT_GEMV;
+  c.p0 = lpr;
+  c.p1 = r;
+  c.p2 = waves;
+  c.p3 = kw;
+  return c;
+}
+
+tlhip_kernel_config_t tiled_cfg(int tm, int tn, int tk, int wm, int wn) {
+  tlhip_kernel_config_t c;
+  memset(&c, 0, sizeof c);
+  c.variant = VARIANT_TILED;
+  c.p0 = tm;
+  c.p1 = tn;
+  c.p2 = tk;
+  c.p3 = wm;
+  c.p4 = wn;
+  return c;
+}
+
+bool config_applicable(const Problem& p, const tlhip_kernel_config_t& c, const char** why) {
+  if (c.variant == VARIANT_TILED) return gemm_config_applicable(p, c, why);
+  return gemv_config_applicable(p, c, why);
+}
+
+// Heuristic default, used when nothing is tuned.
+tlhip_kernel_config_t default_config(const Problem& p) {
+  const int cw = p.format == TLHIP_FMT_INT4_GROUPED ? 32 : 16;
+  const int64_t nchunks = p.k / cw;
+  if (p.m > 16 && p.x_dtype == TLHIP_F16) {
+    tlhip_kernel_config_t c = tiled_cfg(128, 128, 64, 2, 2);
+    if (gemm_config_applicable(p, c, nullptr)) return c;
+  }
+  // lanes per row: keep every lane busy for short rows
+  int lpr = 64;
+  if (nchunks % 64 != 0) lpr = (nchunks % 32 == 0) ? 32 : 16;
+  if (nchunks < 64) lpr = nchunks >= 32 ? 32 : 16;
+  const int r = p.m >= 4 ? 2 : 1;
+  // enough row blocks to give every CU several waves; big N walks with a stride
+  int waves = 4;
+  return gemv_cfg(lpr, r, waves, 1);
+}
+
+std::vector<tlhip_kernel_config_t> candidates(const Problem& p) {
+  std::vector<tlhip_kernel_config_t> out;
+  if (p.m <= 16) {
+    for (int lpr : {16, 32, 64})
+      for (int r : {1, 2, 4})
+        for (int waves : {2, 4, 8})
+          for (int kw : {1, 2, 4}) {
+            if (kw > waves) continue;
+            tlhip_kernel_config_t c = gemv_cfg(lpr, r, waves, kw);
+            if (gemv_config_applicable(p, c, nullptr)) out.push_back(c);
+          }
+  }
+  if (p.x_dtype == TLHIP_F16 && p.m >= 16) {
+    static const int tiles[][5] = {
+        {128, 128, 64, 2, 2}, {256, 128, 64, 2, 2}, {128, 256, 64, 2, 2}, {256, 256, 64, 2, 2},
+        {64, 128, 64, 2, 2},  {128, 64, 64, 2, 2},  {64, 64, 64, 2, 2},   {256, 128, 32, 2, 2},
+    };
+    for (auto& t : tiles) {
+      tlhip_kernel_config_t c = tiled_cfg(t[0], t[1], t[2], t[3], t[4]);
+      if (gemm_config_applicable(p, c, nullptr)) out.push_back(c);
+    }
+  }
+  return out;
+}
+
+tlhip_kernel_config_t select_config(const Problem& p) {
+  {
+    std::lock_guard<std::mutex> lock(g_tune_mutex);
+    auto it = g_tuned.find(problem_key(p));
+    if (it != g_tuned.end() && config_applicable(p, it->second, nullptr)) return it->second;
+  }
+  return default_config(p);
+}
+
+int run_config(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t stream) {
+  if (c.variant == VARIANT_TILED) return launch_gemm(p, c, stream);
+  return launch_gemv(p, c, stream);
+}
+
+int autotune_problem(const Problem& p, double* best_us_out) {
+  if (g_autotuning) return TLHIP_OK;
+  g_autotuning = true;
+  hipStream_t stream = resolve_stream(nullptr);
+  hipEvent_t e0, e1;
+  int rc = TLHIP_OK;
+  if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) {
+    g_autotuning = false;
+    return set_error(TLHIP_ERR_DEVICE, "autotune: hipEventCreate failed");
+  }
+  double best = 1e30;
+  tlhip_kernel_config_t best_cfg = default_config(p);
+  for (const auto& c : candidates(p)) {
+    bool ok = true;
+    for (int i = 0; i < 2 && ok; ++i) ok = run_config(p, c, stream) == TLHIP_OK;  // warm-up
+    if (!ok) continue;
+    double t[3];
+    for (int i = 0; i < 3 && ok; ++i) {
+      hipEventRecord(e0, stream);
+      ok = run_config(p, c, stream) == TLHIP_OK;
+      hipEventRecord(e1, stream);
+      if (hipEventSynchronize(e1) != hipSuccess) {
+        ok = false;
+        rc = set_error(TLHIP_ERR_DEVICE, "autotune: hipEventSynchronize failed");
+        break;
+      }
+      float ms = 0;
+      hipEventElapsedTime(&ms, e0, e1);
+      t[i] = ms * 1000.0;
+    }
+    if (rc) break;
+    if (!ok) continue;
+    std::sort(t, t + 3);
+    if (t[1] < best) {
+      best = t[1];
+      best_cfg = c;
+    }
+  }
+  hipEventDestroy(e0);
+  hipEventDestroy(e1);
+  g_autotuning = false;
+  if (rc) return rc;
+  {
+    std::lock_guard<std::mutex> lock(g_tune_mutex);
+    g_tuned[problem_key(p)] = best_cfg;
+  }
+  count_autotune_run();
+  if (best_us_out) *best_us_out = best;
+  if (getenv("TORCHLETTE_DEBUG_AUTOTUNE"))
+    fprintf(stderr, "[tlhip autotune] %s -> variant %d (%d,%d,%d,%d,%d) %.2f us\n", problem_key(p).c_str(),
+            best_cfg.variant, best_cfg.p0, best_cfg.p1, best_cfg.p2, best_cfg.p3, best_cfg.p4, best);
+  return TLHIP_OK;
+}
+
+}  // namespace
+
+int validate_weight(const tlhip_qweight_t* w, const char* who) {
+  if (!w) return set_error(TLHIP_ERR_INVALID, "%s: missing packing/scales on B operand", who);
+  if (w->format != TLHIP_FMT_INT8_GROUPED && w->format != TLHIP_FMT_INT8_ROW &&
+      w->format != TLHIP_FMT_INT4_GROUPED)
+    return set_error(TLHIP_ERR_INVALID, "%s: unsupported scheme %d", who, w->format);
+  if (w->n < 0 || w->k < 0) return set_error(TLHIP_ERR_INVALID, "%s: negative shape", who);
+  if (w->n > 0 && w->k > 0 && (!w->packed || !w->scales))
+    return set_error(TLHIP_ERR_INVALID, "%s: missing packing/scales on B operand", who);
+  const int per_word = w->format == TLHIP_FMT_INT4_GROUPED ? 8 : 4;
+  if (w->k % per_word != 0)
+    return set_error(TLHIP_ERR_INVALID, "%s: K=%lld must be divisible by %d", who, (long long)w->k, per_word);
+  if (w->format != TLHIP_FMT_INT8_ROW) {
+    if (w->group_size <= 0 || !is_pow2(w->group_size))
+      return set_error(TLHIP_ERR_INVALID, "%s: groupSize %d must be a power of two", who, w->group_size);
+    if (w->k % w->group_size != 0)
+      return set_error(TLHIP_ERR_INVALID, "%s: K=%lld must be divisible by groupSize=%d", who,
+                       (long long)w->k, w->group_size);
+  }
+  if (w->k > (int64_t)1 << 24 || w->n > (int64_t)1 << 30)
+    return set_error(TLHIP_ERR_INVALID, "%s: shape [%lld,%lld] exceeds the supported range", who,
+                     (long long)w->n, (long long)w->k);
+  if (((uintptr_t)w->packed & 15) != 0)
+    return set_error(TLHIP_ERR_INVALID, "%s: packed weights must be 16-byte aligned", who);
+  return TLHIP_OK;
+}
+
+int make_problem(const tlhip_qweight_t* w, const void* x, int x_dtype, int64_t m, void* y, int y_dtype,
+                 float alpha, const tlhip_epilogue_t* epilogue, Problem* p, const char* who) {
+  int rc = validate_weight(w, who);
+  if (rc) return rc;
+  if (m < 0) return set_error(TLHIP_ERR_INVALID, "%s: negative M", who);
+  if (x_dtype != TLHIP_F32 && x_dtype != TLHIP_F16) return set_error(TLHIP_ERR_INVALID, "%s: bad x dtype %d", who, x_dtype);
+  if (y_dtype != TLHIP_F32 && y_dtype != TLHIP_F16) return set_error(TLHIP_ERR_INVALID, "%s: bad y dtype %d", who, y_dtype);
+  if (m > 0 && w->k > 0 && !x) return set_error(TLHIP_ERR_INVALID, "%s: null activations", who);
+  if (m > 0 && w->n > 0 && !y) return set_error(TLHIP_ERR_INVALID, "%s: null output", who);
+  if (((uintptr_t)x & 15) != 0) return set_error(TLHIP_ERR_INVALID, "%s: activations must be 16-byte aligned", who);
+  p->format = w->format;
+  p->group_size = w->group_size;
+  p->n = w->n;
+  p->k = w->k;
+  p->m = m;
+  p->packed = w->packed;
+  p->scales = w->scales;
+  p->x = x;
+  p->x_dtype = x_dtype;
+  p->y = y;
+  p->y_dtype = y_dtype;
+  p->alpha = alpha;
+  memset(&p->epi, 0, sizeof p->epi);
+  if (epilogue) {
+    if (epilogue->n_ops < 0 || epilogue->n_ops > TLHIP_MAX_EPILOGUE_OPS)
+      return set_error(TLHIP_ERR_INVALID, "%s: epilogue has %d ops (max %d)", who, epilogue->n_ops,
+                       TLHIP_MAX_EPILOGUE_OPS);
+    p->epi.n_ops = epilogue->n_ops;
+    for (int i = 0; i < epilogue->n_ops; ++i) {
+      const tlhip_epilogue_op_t& op = epilogue->ops[i];
+      if (op.kind != TLHIP_EPI_NONE && op.kind != TLHIP_EPI_BIAS && op.kind != TLHIP_EPI_UNARY)
+        return set_error(TLHIP_ERR_INVALID, "%s: unknown epilogue op kind %d", who, op.kind);
+      if (op.kind == TLHIP_EPI_BIAS) {
+        if (!op.input && w->n > 0) return set_error(TLHIP_ERR_INVALID, "%s: bias epilogue without input", who);
+        if (op.input_dtype != TLHIP_F32 && op.input_dtype != TLHIP_F16)
+          return set_error(TLHIP_ERR_INVALID, "%s: bad bias dtype %d", who, op.input_dtype);
+      }
+      if (op.kind == TLHIP_EPI_UNARY && (op.unary < TLHIP_UNARY_NONE || op.unary > TLHIP_UNARY_TANH))
+        return set_error(TLHIP_ERR_INVALID, "%s: unknown unary op %d", who, op.unary);
+      p->epi.kind[i] = op.kind;
+      p->epi.unary[i] = op.unary;
+      p->epi.input[i] = op.input;
+      p->epi.input_dtype[i] = op.input_dtype;
+    }
+  }
+  return TLHIP_OK;
+}
+
+}  // namespace tlhip
+
+using namespace tlhip;
+
+extern "C" {
+
+int tlhip_dequant(const tlhip_qweight_t* w, float* out, tlhip_stream_t stream) {
+  TLHIP_REQUIRE_INIT();
+  int rc = validate_weight(w, "dequant");
+  if (rc) return rc;
+  if (w->n > 0 && w->k > 0 && !out) return set_error(TLHIP_ERR_INVALID, "dequant: null output");
+  if (((uintptr_t)out & 15) != 0) return set_error(TLHIP_ERR_INVALID, "dequant: output must be 16-byte aligned");
+  return launch_dequant(*w, out, resolve_stream(stream));
+}
+
+int tlhip_gemv(const tlhip_qweight_t* w, const void* x, int x_dtype, int64_t m, void* y, int y_dtype,
+               float alpha, const tlhip_epilogue_t* epilogue, tlhip_stream_t stream) {
+  TLHIP_REQUIRE_INIT();
+  Problem p;
+  int rc = make_problem(w, x, x_dtype, m, y, y_dtype, alpha, epilogue, &p, "gemv");
+  if (rc) return rc;
+  if (m > 16) return set_error(TLHIP_ERR_INVALID, "gemv: M=%lld above 16; use tlhip_gemm_prefill", (long long)m);
+  tlhip_kernel_config_t c = select_config(p);
+  if (c.variant == VARIANT_TILED) c = default_config(p);
+  return launch_gemv(p, c, resolve_stream(stream));
+}
+
+int tlhip_gemm_prefill(const tlhip_qweight_t* w, const void* x, int x_dtype, int64_t m, void* y, int y_dtype,
+                       float alpha, const tlhip_epilogue_t* epilogue, tlhip_stream_t stream) {
+  TLHIP_REQUIRE_INIT();
+  Problem p;
+  int rc = make_problem(w, x, x_dtype, m, y, y_dtype, alpha, epilogue, &p, "gemm_prefill");
+  if (rc) return rc;
+  if (x_dtype != TLHIP_F16) return set_error(TLHIP_ERR_INVALID, "gemm_prefill: activations must be f16");
+  tlhip_kernel_config_t c = select_config(p);
+  if (c.variant != VARIANT_TILED) {
+    c = tiled_cfg(128, 128, 64, 2, 2);
+    const char* why = nullptr;
+    if (!gemm_config_applicable(p, c, &why))
+      return set_error(TLHIP_ERR_INVALID, "gemm_prefill: shape not supported: %s", why ? why : "?");
+  }
+  return launch_gemm(p, c, resolve_stream(stream));
+}
+
+static int matmul_with(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t stream) {
+  if (c.variant == VARIANT_TILED) return launch_gemm(p, c, stream);
+  if (p.m <= 16) return launch_gemv(p, c, stream);
+  // f32 activations (or a shape the tiled kernel rejects) above 16 rows: GEMV
+  // passes of 16 rows.  Declared, slow: every pass streams the weights again.
+  const int xb = p.x_dtype == TLHIP_F16 ? 2 : 4, yb = p.y_dtype == TLHIP_F16 ? 2 : 4;
+  for (int64_t m0 = 0; m0 < p.m; m0 += 16) {
+    Problem q = p;
+    q.m = std::min<int64_t>(16, p.m - m0);
+    q.x = (const char*)p.x + m0 * p.k * xb;
+    q.y = (char*)p.y + m0 * p.n * yb;
+    int rc = launch_gemv(q, c, stream);
+    if (rc) return rc;
+  }
+  return TLHIP_OK;
+}
+
+int tlhip_matmul_quantized(const tlhip_qweight_t* w, const void* x, int x_dtype, int64_t m, void* y,
+                           int y_dtype, float alpha, const tlhip_epilogue_t* epilogue, tlhip_stream_t stream) {
+  TLHIP_REQUIRE_INIT();
+  Problem p;
+  int rc = make_problem(w, x, x_dtype, m, y, y_dtype, alpha, epilogue, &p, "matmulQuantizedB");
+  if (rc) return rc;
+  if (p.m == 0 || p.n == 0) return TLHIP_OK;
+  if ((g_autotune_counter > 0 || env_autotune()) && !g_autotuning) {
+    bool have;
+    {
+      std::lock_guard<std::mutex> lock(g_tune_mutex);
+      have = g_tuned.count(problem_key(p)) != 0;
+    }
+    if (!have) {
+      // Tuning launches write y; the real launch below overwrites it.
+      hipStreamSynchronize(resolve_stream(stream));
+      rc = autotune_problem(p, nullptr);
+      if (rc) return rc;
+    }
+  }
+  return matmul_with(p, select_config(p), resolve_stream(stream));
+}
+
+int tlhip_matmul_quantized_config(const tlhip_qweight_t* w, const void* x, int x_dtype, int64_t m, void* y,
+                                  int y_dtype, float alpha, const tlhip_epilogue_t* epilogue,
+                                  const tlhip_kernel_config_t* config, tlhip_stream_t stream) {
+  TLHIP_REQUIRE_INIT();
+  if (!config) return set_error(TLHIP_ERR_INVALID, "matmul: null config");
+  Problem p;
+  int rc = make_problem(w, x, x_dtype, m, y, y_dtype, alpha, epilogue, &p, "matmulQuantizedB");
+  if (rc) return rc;
+  if (p.m == 0 || p.n == 0) return TLHIP_OK;
+  const char* why = nullptr;
+  if (!config_applicable(p, *config, &why))
+    return set_error(TLHIP_ERR_INVALID, "matmul: config not applicable: %s", why ? why : "?");
+  return matmul_with(p, *config, resolve_stream(stream));
+}
+
+static int shape_problem(const tlhip_qweight_t* w, int x_dtype, int64_t m, int y_dtype, Problem* p) {
+  int rc = validate_weight(w, "config");
+  if (rc) return rc;
+  memset(p, 0, sizeof *p);
+  p->format = w->format;
+  p->group_size = w->group_size;
+  p->n = w->n;
+  p->k = w->k;
+  p->m = m;
+  p->x_dtype = x_dtype;
+  p->y_dtype = y_dtype;
+  p->alpha = 1.f;
+  return TLHIP_OK;
+}
+
+int tlhip_candidate_count(const tlhip_qweight_t* w, int x_dtype, int64_t m, int y_dtype, int* out) {
+  Problem p;
+  int rc = shape_problem(w, x_dtype, m, y_dtype, &p);
+  if (rc) return rc;
+  if (!out) return set_error(TLHIP_ERR_INVALID, "candidate_count: null output");
+  *out = (int)candidates(p).size();
+  return TLHIP_OK;
+}
+
+int tlhip_candidate_get(const tlhip_qweight_t* w, int x_dtype, int64_t m, int y_dtype, int index,
+                        tlhip_kernel_config_t* out) {
+  Problem p;
+  int rc = shape_problem(w, x_dtype, m, y_dtype, &p);
+  if (rc) return rc;
+  auto c = candidates(p);
+  if (!out || index < 0 || index >= (int)c.size())
+    return set_error(TLHIP_ERR_INVALID, "candidate_get: index %d out of range [0,%d)", index, (int)c.size());
+  *out = c[index];
+  return TLHIP_OK;
+}
+
+int tlhip_selected_config(const tlhip_qweight_t* w, int x_dtype, int64_t m, int y_dtype,
+                          tlhip_kernel_config_t* out) {
+  Problem p;
+  int rc = shape_problem(w, x_dtype, m, y_dtype, &p);
+  if (rc) return rc;
+  if (!out) return set_error(TLHIP_ERR_INVALID, "selected_config: null output");
+  *out = select_config(p);
+  return TLHIP_OK;
+}
+
+int tlhip_set_autotune_enabled(int enabled) {
+  // dispatch.ts:128-134: true increments (nested regions), false resets to 0.
+  if (enabled) g_autotune_counter++;
+  else g_autotune_counter = 0;
+  return TLHIP_OK;
+}
+
+int tlhip_is_autotune_enabled(void) { return g_autotune_counter > 0 || env_autotune(); }
+
+int tlhip_autotune(const tlhip_qweight_t* w, const void* x, int x_dtype, int64_t m, void* y, int y_dtype,
+                   double* best_us) {
+  TLHIP_REQUIRE_INIT();
+  Problem p;
+  int rc = make_problem(w, x, x_dtype, m, y, y_dtype, 1.f, nullptr, &p, "autotune");
+  if (rc) return rc;
+  if (p.m == 0 || p.n == 0 || p.k == 0) return set_error(TLHIP_ERR_INVALID, "autotune: empty problem");
+  return autotune_problem(p, best_us);
+}
+
+int tlhip_pretune_matmul_shapes(const int64_t* mnk, int count) {
+  if (count < 0 || (count > 0 && !mnk)) return set_error(TLHIP_ERR_INVALID, "pretune: bad arguments");
+  std::lock_guard<std::mutex> lock(g_tune_mutex);
+  for (int i = 0; i < count; ++i) g_shape_hints.push_back({mnk[3 * i], mnk[3 * i + 1], mnk[3 * i + 2]});
+  return TLHIP_OK;
+}
+
+int tlhip_tune_cache_export(char* buf, size_t cap, size_t* needed) {
+  std::ostringstream os;
+  os << "{\"version\":1,\"entries\":{";
+  {
+    std::lock_guard<std::mutex> lock(g_tune_mutex);
+    bool first = true;
+    for (auto& kv : g_tuned) {
+      if (!first) os << ",";
+      first = false;
+      const auto& c = kv.second;
+      os << "\"" << kv.first << "\":[" << c.variant << "," << c.p0 << "," << c.p1 << "," << c.p2 << "," << c.p3
+         << "," << c.p4 << "," << c.p5 << "," << c.p6 << "]";
+    }
+  }
+  os << "}}";
+  const std::string s = os.str();
+  if (needed) *needed = s.size() + 1;
+  if (buf && cap > 0) {
+    const size_t nc = std::min(cap - 1, s.size());
+    memcpy(buf, s.data(), nc);
+    buf[nc] = '\0';
+  }
+  return TLHIP_OK;
+}
+
+// Accepts exactly what export writes: {"version":1,"entries":{"key":[8 ints],...}}
+int tlhip_tune_cache_import(const char* json) {
+  if (!json) return set_error(TLHIP_ERR_INVALID, "tune_cache_import: null text");
+  const char* p = strstr(json, "\"entries\"");
+  if (!p) return set_error(TLHIP_ERR_INVALID, "tune_cache_import: no \"entries\" object");
+  p = strchr(p, '{');
+  if (!p) return set_error(TLHIP_ERR_INVALID, "tune_cache_import: malformed entries");
+  ++p;
+  std::map<std::string, tlhip_kernel_config_t> parsed;
+  for (;;) {
+    while (*p == ' ' || *p == '\n' || *p == '\t' || *p == ',' || *p == '\r') ++p;
+    if (*p == '}') break;
+    if (*p != '"') return set_error(TLHIP_ERR_INVALID, "tune_cache_import: expected a key");
+    const char* ke = strchr(p + 1, '"');
+    if (!ke) return set_error(TLHIP_ERR_INVALID, "tune_cache_import: unterminated key");
+    std::string key(p + 1, ke);
+    p = strchr(ke, '[');
+    if (!p) return set_error(TLHIP_ERR_INVALID, "tune_cache_import: expected an array for %s", key.c_str());
+    ++p;
+    int v[8];
+    for (int i = 0; i < 8; ++i) {
+      char* end = nullptr;
+      v[i] = (int)strtol(p, &end, 10);
+      if (end == p) return set_error(TLHIP_ERR_INVALID, "tune_cache_import: expected 8 integers for %s", key.c_str());
+      p = end;
+      while (*p == ' ' || *p == ',') ++p;
+    }
+    if (*p != ']') return set_error(TLHIP_ERR_INVALID, "tune_cache_import: expected ] after %s", key.c_str());
+    ++p;
+    tlhip_kernel_config_t c = {v[0], v[1], v[2], v[3], v[4], v[5], v[6], v[7]};
+    parsed[key] = c;
+  }
+  std::lock_guard<std::mutex> lock(g_tune_mutex);
+  for (auto& kv : parsed) g_tuned[kv.first] = kv.second;
+  return TLHIP_OK;
+}
+
+int tlhip_tune_cache_clear(void) {
+  std::lock_guard<std::mutex> lock(g_tune_mutex);
+  g_tuned.clear();
+  g_shape_hints.clear();
+  return TLHIP_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,248 @@
+// Runtime half of the C ABI: device selection, memory, streams, events, the
+// per-thread error string and the dispatch counters.  It plays the part the
+// WebGPU device/queue plays for the reference backend
+// (src/backend/webgpu/gpu-context.ts): ops enqueue on one in-order stream and
+// only a read waits.
+#include <atomic>
+#include <cstring>
+#include <mutex>
+#include <string>
+
+#include "common.h"
+
+namespace tlhip {
+
+namespace {
+thread_local char g_error[512] = "";
+std::mutex g_mutex;
+bool g_init = false;
+int g_device = -1;
+hipStream_t g_stream = nullptr;
+hipDeviceProp_t g_props;
+
+std::atomic<uint64_t> g_gemv_dispatches{0};
+std::atomic<uint64_t> g_gemm_dispatches{0};
+std::atomic<uint64_t> g_dequant_dispatches{0};
+std::atomic<uint64_t> g_autotune_runs{0};
+}  // namespace
+
+int set_error(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+void clear_error() { g_error[0] = '\0'; }
+
+bool is_initialised() { return g_init; }
+
+hipStream_t resolve_stream(tlhip_stream_t s) { return s ? static_cast<hipStream_t>(s) : g_stream; }
+
+int device_cu_count() { return g_init ? g_props.multiProcessorCount : 0; }
+
+void count_gemv_dispatch() { g_gemv_dispatches++; }
+void count_gemm_dispatch() { g_gemm_dispatches++; }
+void count_dequant_dispatch() { g_dequant_dispatches++; }
+void count_autotune_run() { g_autotune_runs++; }
+
+}  // namespace tlhip
+
+using namespace tlhip;
+
+extern "C" {
+
+const char* tlhip_last_error(void) { return g_error; }
+
+int tlhip_init(int device_index) {
+  std::lock_guard<std::mutex> lock(g_mutex);
+  if (g_init) {
+    if (device_index == g_device) return TLHIP_OK;
+    return set_error(TLHIP_ERR_STATE, "tlhip_init: already initialised on device %d", g_device);
+  }
+  int count = 0;
+  hipError_t e = hipGetDeviceCount(&count);
+  if (e != hipSuccess || count == 0) {
+    return set_error(TLHIP_ERR_DEVICE, "tlhip_init: no HIP device available (%s); this backend has no CPU fallback",
+                     e != hipSuccess ? hipGetErrorString(e) : "device count is 0");
+  }
+  if (device_index < 0 || device_index >= count)
+    return set_error(TLHIP_ERR_INVALID, "tlhip_init: device index %d out of range [0,%d)", device_index, count);
+  TLHIP_CHECK_HIP(hipSetDevice(device_index));
+  TLHIP_CHECK_HIP(hipGetDeviceProperties(&g_props, device_index));
+  if (strncmp(g_props.gcnArchName, "gfx950", 6) != 0) {
+    return set_error(TLHIP_ERR_DEVICE, "tlhip_init: device %d is %s; this library carries gfx950 code only",
+                     device_index, g_props.gcnArchName);
+  }
+  // Default priority only: mixed stream priorities are not used anywhere.
+  TLHIP_CHECK_HIP(hipStreamCreateWithFlags(&g_stream, hipStreamNonBlocking));
+  g_device = device_index;
+  g_init = true;
+  clear_error();
+  return TLHIP_OK;
+}
+
+int tlhip_shutdown(void) {
+  std::lock_guard<std::mutex> lock(g_mutex);
+  if (!g_init) return TLHIP_OK;
+  hipStreamSynchronize(g_stream);
+  hipStreamDestroy(g_stream);
+  g_stream = nullptr;
+  g_init = false;
+  g_device = -1;
+  return TLHIP_OK;
+}
+
+int tlhip_device_info(tlhip_device_info_t* out) {
+  TLHIP_REQUIRE_INIT();
+  if (!out) return set_error(TLHIP_ERR_INVALID, "tlhip_device_info: null output");
+  memset(out, 0, sizeof(*out));
+  strncpy(out->name, g_props.name, sizeof(out->name) - 1);
+  strncpy(out->arch, g_props.gcnArchName, sizeof(out->arch) - 1);
+  out->compute_units = g_props.multiProcessorCount;
+  out->wavefront_size = g_props.warpSize;
+  out->lds_bytes_per_block = (int32_t)g_props.sharedMemPerBlock;
+  out->clock_khz = g_props.clockRate;
+  out->memory_clock_khz = g_props.memoryClockRate;
+  out->memory_bus_bits = g_props.memoryBusWidth;
+  out->total_memory_bytes = (int64_t)g_props.totalGlobalMem;
+  out->l2_bytes = (int64_t)g_props.l2CacheSize;
+  return TLHIP_OK;
+}
+
+int tlhip_malloc(size_t bytes, void** out) {
+  TLHIP_REQUIRE_INIT();
+  if (!out) return set_error(TLHIP_ERR_INVALID, "tlhip_malloc: null output");
+  *out = nullptr;
+  if (bytes == 0) return TLHIP_OK;
+  TLHIP_CHECK_HIP(hipMalloc(out, bytes));
+  return TLHIP_OK;
+}
+
+int tlhip_free(void* ptr) {
+  TLHIP_REQUIRE_INIT();
+  if (!ptr) return TLHIP_OK;
+  TLHIP_CHECK_HIP(hipFree(ptr));
+  return TLHIP_OK;
+}
+
+int tlhip_memset(void* ptr, int value, size_t bytes, tlhip_stream_t stream) {
+  TLHIP_REQUIRE_INIT();
+  if (bytes == 0) return TLHIP_OK;
+  TLHIP_CHECK_HIP(hipMemsetAsync(ptr, value, bytes, resolve_stream(stream)));
+  return TLHIP_OK;
+}
+
+int tlhip_memcpy_h2d(void* dst, const void* host_src, size_t bytes, tlhip_stream_t stream) {
+  TLHIP_REQUIRE_INIT();
+  if (bytes == 0) return TLHIP_OK;
+  TLHIP_CHECK_HIP(hipMemcpyAsync(dst, host_src, bytes, hipMemcpyHostToDevice, resolve_stream(stream)));
+  return TLHIP_OK;
+}
+
+int tlhip_memcpy_d2h(void* host_dst, const void* src, size_t bytes, tlhip_stream_t stream) {
+  TLHIP_REQUIRE_INIT();
+  if (bytes == 0) return TLHIP_OK;
+  TLHIP_CHECK_HIP(hipMemcpyAsync(host_dst, src, bytes, hipMemcpyDeviceToHost, resolve_stream(stream)));
+  return TLHIP_OK;
+}
+
+int tlhip_memcpy_d2d(void* dst, const void* src, size_t bytes, tlhip_stream_t stream) {
+  TLHIP_REQUIRE_INIT();
+  if (bytes == 0) return TLHIP_OK;
+  TLHIP_CHECK_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, resolve_stream(stream)));
+  return TLHIP_OK;
+}
+
+int tlhip_host_alloc(size_t bytes, void** out) {
+  TLHIP_REQUIRE_INIT();
+  if (!out) return set_error(TLHIP_ERR_INVALID, "tlhip_host_alloc: null output");
+  TLHIP_CHECK_HIP(hipHostMalloc(out, bytes ? bytes : 1, hipHostMallocDefault));
+  return TLHIP_OK;
+}
+
+int tlhip_host_free(void* host_ptr) {
+  TLHIP_REQUIRE_INIT();
+  if (!host_ptr) return TLHIP_OK;
+  TLHIP_CHECK_HIP(hipHostFree(host_ptr));
+  return TLHIP_OK;
+}
+
+int tlhip_stream_create(tlhip_stream_t* out) {
+  TLHIP_REQUIRE_INIT();
+  if (!out) return set_error(TLHIP_ERR_INVALID, "tlhip_stream_create: null output");
+  hipStream_t s;
+  TLHIP_CHECK_HIP(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+  *out = s;
+  return TLHIP_OK;
+}
+
+int tlhip_stream_destroy(tlhip_stream_t stream) {
+  TLHIP_REQUIRE_INIT();
+  if (!stream) return TLHIP_OK;
+  TLHIP_CHECK_HIP(hipStreamDestroy(static_cast<hipStream_t>(stream)));
+  return TLHIP_OK;
+}
+
+int tlhip_stream_synchronize(tlhip_stream_t stream) {
+  TLHIP_REQUIRE_INIT();
+  TLHIP_CHECK_HIP(hipStreamSynchronize(resolve_stream(stream)));
+  return TLHIP_OK;
+}
+
+int tlhip_event_create(tlhip_event_t* out) {
+  TLHIP_REQUIRE_INIT();
+  if (!out) return set_error(TLHIP_ERR_INVALID, "tlhip_event_create: null output");
+  hipEvent_t e;
+  TLHIP_CHECK_HIP(hipEventCreate(&e));
+  *out = e;
+  return TLHIP_OK;
+}
+
+int tlhip_event_destroy(tlhip_event_t ev) {
+  TLHIP_REQUIRE_INIT();
+  if (!ev) return TLHIP_OK;
+  TLHIP_CHECK_HIP(hipEventDestroy(static_cast<hipEvent_t>(ev)));
+  return TLHIP_OK;
+}
+
+int tlhip_event_record(tlhip_event_t ev, tlhip_stream_t stream) {
+  TLHIP_REQUIRE_INIT();
+  TLHIP_CHECK_HIP(hipEventRecord(static_cast<hipEvent_t>(ev), resolve_stream(stream)));
+  return TLHIP_OK;
+}
+
+int tlhip_event_synchronize(tlhip_event_t ev) {
+  TLHIP_REQUIRE_INIT();
+  TLHIP_CHECK_HIP(hipEventSynchronize(static_cast<hipEvent_t>(ev)));
+  return TLHIP_OK;
+}
+
+int tlhip_event_elapsed_us(tlhip_event_t start, tlhip_event_t stop, double* out_us) {
+  TLHIP_REQUIRE_INIT();
+  if (!out_us) return set_error(TLHIP_ERR_INVALID, "tlhip_event_elapsed_us: null output");
+  float ms = 0.f;
+  TLHIP_CHECK_HIP(hipEventElapsedTime(&ms, static_cast<hipEvent_t>(start), static_cast<hipEvent_t>(stop)));
+  *out_us = (double)ms * 1000.0;
+  return TLHIP_OK;
+}
+
+uint64_t tlhip_counter(const char* name) {
+  if (!name) return 0;
+  if (!strcmp(name, "quant_gemv_dispatches")) return g_gemv_dispatches.load();
+  if (!strcmp(name, "quant_gemm_dispatches")) return g_gemm_dispatches.load();
+  if (!strcmp(name, "dequant_dispatches")) return g_dequant_dispatches.load();
+  if (!strcmp(name, "autotune_runs")) return g_autotune_runs.load();
+  return 0;
+}
+
+int tlhip_counters_reset(void) {
+  g_gemv_dispatches = 0;
+  g_gemm_dispatches = 0;
+  g_dequant_dispatches = 0;
+  g_autotune_runs = 0;
+  return TLHIP_OK;
+}
+
+}  // extern "C"
