@@ -68,10 +68,11 @@ _SCHEMES = {"int8-grouped": L.FMT_INT8_GROUPED, "int8-row": L.FMT_INT8_ROW,
 
 
 def resolveWeightFormat(name: str, elementType: str = "f16") -> StorageFormat:
-    """types.ts:58-67 for "int8-64" / "int8-128"; plus "int4-<G>" and "int8-row"."""
-    if name == "int8-64" or name == "int8-128":
+    """types.ts:58-67 for "int8-64" / "int8-128" (any "int8-<G>" is accepted);
+    plus "int4-<G>" and "int8-row"."""
+    if name.startswith("int8-") and name[5:].isdigit():
         return StorageFormat(elementType, QuantPacking("int8-grouped", int(name[5:]), "f16"))
-    if name.startswith("int4-"):
+    if name.startswith("int4-") and name[5:].isdigit():
         return StorageFormat(elementType, QuantPacking("int4-grouped", int(name[5:]), "f16"))
     if name == "int8-row":
         return StorageFormat(elementType, QuantPacking("int8-row", 0, "f32"))

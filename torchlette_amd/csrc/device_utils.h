@@ -14,6 +14,11 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef float float4_t __attribute__((ext_vector_type(4)));
 typedef float float16_t __attribute__((ext_vector_type(16)));
 
+// Reinterpretations take their argument BY VALUE: __builtin_bit_cast applied
+// directly to a vector-element lvalue (v.y) reads the vector's first element.
+__device__ __forceinline__ half2_t as_half2(uint32_t v) { return __builtin_bit_cast(half2_t, v); }
+__device__ __forceinline__ float as_float(uint32_t v) { return __builtin_bit_cast(float, v); }
+
 __device__ __forceinline__ float half_bits_to_float(uint32_t h) {
   return (float)__builtin_bit_cast(_Float16, (uint16_t)h);
 }

@@ -80,10 +80,10 @@ struct ChunkDot<TLHIP_FMT_INT4_GROUPED, _Float16> {
     float d = 0.f;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      d = __builtin_amdgcn_fdot2(q[4 * i + 0], __builtin_bit_cast(half2_t, xv[i].x), d, false);
-      d = __builtin_amdgcn_fdot2(q[4 * i + 1], __builtin_bit_cast(half2_t, xv[i].y), d, false);
-      d = __builtin_amdgcn_fdot2(q[4 * i + 2], __builtin_bit_cast(half2_t, xv[i].z), d, false);
-      d = __builtin_amdgcn_fdot2(q[4 * i + 3], __builtin_bit_cast(half2_t, xv[i].w), d, false);
+      d = __builtin_amdgcn_fdot2(q[4 * i + 0], as_half2(xv[i].x), d, false);
+      d = __builtin_amdgcn_fdot2(q[4 * i + 1], as_half2(xv[i].y), d, false);
+      d = __builtin_amdgcn_fdot2(q[4 * i + 2], as_half2(xv[i].z), d, false);
+      d = __builtin_amdgcn_fdot2(q[4 * i + 3], as_half2(xv[i].w), d, false);
     }
     return d;
   }
@@ -103,10 +103,10 @@ struct ChunkDotInt8Half {
     float d = 0.f;
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
-      d = __builtin_amdgcn_fdot2(q[4 * i + 0], __builtin_bit_cast(half2_t, xv[i].x), d, false);
-      d = __builtin_amdgcn_fdot2(q[4 * i + 1], __builtin_bit_cast(half2_t, xv[i].y), d, false);
-      d = __builtin_amdgcn_fdot2(q[4 * i + 2], __builtin_bit_cast(half2_t, xv[i].z), d, false);
-      d = __builtin_amdgcn_fdot2(q[4 * i + 3], __builtin_bit_cast(half2_t, xv[i].w), d, false);
+      d = __builtin_amdgcn_fdot2(q[4 * i + 0], as_half2(xv[i].x), d, false);
+      d = __builtin_amdgcn_fdot2(q[4 * i + 1], as_half2(xv[i].y), d, false);
+      d = __builtin_amdgcn_fdot2(q[4 * i + 2], as_half2(xv[i].z), d, false);
+      d = __builtin_amdgcn_fdot2(q[4 * i + 3], as_half2(xv[i].w), d, false);
     }
     return d;
   }
@@ -135,10 +135,10 @@ struct ChunkDotInt8Float {
     float d = 0.f;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      d = fmaf(q[4 * i + 0], __uint_as_float(xv[i].x), d);
-      d = fmaf(q[4 * i + 1], __uint_as_float(xv[i].y), d);
-      d = fmaf(q[4 * i + 2], __uint_as_float(xv[i].z), d);
-      d = fmaf(q[4 * i + 3], __uint_as_float(xv[i].w), d);
+      d = fmaf(q[4 * i + 0], as_float(xv[i].x), d);
+      d = fmaf(q[4 * i + 1], as_float(xv[i].y), d);
+      d = fmaf(q[4 * i + 2], as_float(xv[i].z), d);
+      d = fmaf(q[4 * i + 3], as_float(xv[i].w), d);
     }
     return d;
   }
@@ -163,10 +163,10 @@ struct ChunkDot<TLHIP_FMT_INT4_GROUPED, float> {
     float d = 0.f;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      d = fmaf(q[4 * i + 0], __uint_as_float(xv[i].x), d);
-      d = fmaf(q[4 * i + 1], __uint_as_float(xv[i].y), d);
-      d = fmaf(q[4 * i + 2], __uint_as_float(xv[i].z), d);
-      d = fmaf(q[4 * i + 3], __uint_as_float(xv[i].w), d);
+      d = fmaf(q[4 * i + 0], as_float(xv[i].x), d);
+      d = fmaf(q[4 * i + 1], as_float(xv[i].y), d);
+      d = fmaf(q[4 * i + 2], as_float(xv[i].z), d);
+      d = fmaf(q[4 * i + 3], as_float(xv[i].w), d);
     }
     return d;
   }
