@@ -36,6 +36,7 @@ extern "C" {
 
 typedef void* tlhip_stream_t;
 typedef void* tlhip_event_t;
+typedef void* tlhip_graph_t;
 
 /* Storage format of a packed weight: the values of
  * StorageFormat.packing.scheme (src/backend/types.ts:46-55).  INT8_GROUPED is
@@ -138,6 +139,17 @@ int tlhip_event_record(tlhip_event_t ev, tlhip_stream_t stream);
 int tlhip_event_synchronize(tlhip_event_t ev);
 int tlhip_event_elapsed_us(tlhip_event_t start, tlhip_event_t stop, double* host_out_us);
 
+/* Record the work enqueued on `stream` between begin and end into a graph that
+ * can be replayed with one call.  The reference batches a decode step's
+ * dispatches into one command-buffer submission
+ * (src/backend/webgpu/shared-encoder.ts); a captured graph is the HIP
+ * counterpart.  The compute entry points enqueue kernels only (no memset or
+ * allocation), so all of them may be captured; autotuning must be off. */
+int tlhip_graph_begin_capture(tlhip_stream_t stream);
+int tlhip_graph_end_capture(tlhip_stream_t stream, tlhip_graph_t* host_out);
+int tlhip_graph_launch(tlhip_graph_t graph, tlhip_stream_t stream);
+int tlhip_graph_destroy(tlhip_graph_t graph);
+
 /* ---- host-side weight preparation: src/backend/quantize.ts ---- */
 /* f32ToF16Bits (quantize.ts:22-47), including its round-half-up subnormals. */
 uint16_t tlhip_f32_to_f16_bits(float value);
@@ -200,8 +212,8 @@ int tlhip_cast(const void* in, int in_dtype, void* out, int out_dtype, int64_t c
  * (skinny MFMA), 2 = "tiled" (prefill MFMA GEMM).  Unused fields are 0. */
 typedef struct {
   int32_t variant;
-  int32_t p0; /* gemv: lanes per row (16/32/64)   tiled: tile M */
-  int32_t p1; /* gemv: rows per lane-group        tiled: tile N */
+  int32_t p0; /* gemv: lanes per row (16/32/64)   gemv_mfma: waves per workgroup   tiled: tile M */
+  int32_t p1; /* gemv: rows per lane-group        gemv_mfma: iterations in flight  tiled: tile N */
   int32_t p2; /* gemv: waves per workgroup        tiled: tile K */
   int32_t p3; /* gemv: K-split waves (LDS combine) tiled: waves M */
   int32_t p4; /* gemv: reserved                   tiled: waves N */

@@ -88,6 +88,10 @@ SIGNATURES = {
     "tlhip_event_record": (_i, [_vp, _vp]),
     "tlhip_event_synchronize": (_i, [_vp]),
     "tlhip_event_elapsed_us": (_i, [_vp, _vp, C.POINTER(C.c_double)]),
+    "tlhip_graph_begin_capture": (_i, [_vp]),
+    "tlhip_graph_end_capture": (_i, [_vp, C.POINTER(_vp)]),
+    "tlhip_graph_launch": (_i, [_vp, _vp]),
+    "tlhip_graph_destroy": (_i, [_vp]),
     "tlhip_f32_to_f16_bits": (C.c_uint16, [_f]),
     "tlhip_f16_bits_to_f32": (_f, [C.c_uint16]),
     "tlhip_quantize_int8_grouped": (_i, [_vp, _i64, _i64, _i64, _vp, _vp]),

@@ -68,6 +68,15 @@ tlhip_kernel_config_t gemv_cfg(int lpr, int r, int waves, int kw) {
   return c;
 }
 
+tlhip_kernel_config_t mfma_cfg(int waves, int unroll) {
+  tlhip_kernel_config_t c;
+  memset(&c, 0, sizeof c);
+  c.variant = VARIANT_GEMV_MFMA;
+  c.p0 = waves;
+  c.p1 = unroll;
+  return c;
+}
+
 tlhip_kernel_config_t tiled_cfg(int tm, int tn, int tk, int wm, int wn) {
   tlhip_kernel_config_t c;
   memset(&c, 0, sizeof c);
@@ -82,6 +91,7 @@ tlhip_kernel_config_t tiled_cfg(int tm, int tn, int tk, int wm, int wn) {
 
 bool config_applicable(const Problem& p, const tlhip_kernel_config_t& c, const char** why) {
   if (c.variant == VARIANT_TILED) return gemm_config_applicable(p, c, why);
+  if (c.variant == VARIANT_GEMV_MFMA) return gemv_mfma_config_applicable(p, c, why);
   return gemv_config_applicable(p, c, why);
 }
 
@@ -92,6 +102,11 @@ tlhip_kernel_config_t default_config(const Problem& p) {
   if (p.m > 16 && p.x_dtype == TLHIP_F16) {
     tlhip_kernel_config_t c = tiled_cfg(128, 128, 64, 2, 2);
     if (gemm_config_applicable(p, c, nullptr)) return c;
+  }
+  // three or more activation rows: the matrix-core kernel streams the weights once
+  if (p.m >= 3 && p.m <= 16) {
+    tlhip_kernel_config_t c = mfma_cfg(8, 2);
+    if (gemv_mfma_config_applicable(p, c, nullptr)) return c;
   }
   // lanes per row: keep every lane busy for short rows
   int lpr = 64;
@@ -114,6 +129,13 @@ std::vector<tlhip_kernel_config_t> candidates(const Problem& p) {
             tlhip_kernel_config_t c = gemv_cfg(lpr, r, waves, kw);
             if (gemv_config_applicable(p, c, nullptr)) out.push_back(c);
           }
+  }
+  if (p.m <= 16) {
+    for (int waves : {4, 8, 16})
+      for (int unroll : {1, 2, 4}) {
+        tlhip_kernel_config_t c = mfma_cfg(waves, unroll);
+        if (gemv_mfma_config_applicable(p, c, nullptr)) out.push_back(c);
+      }
   }
   if (p.x_dtype == TLHIP_F16 && p.m >= 16) {
     static const int tiles[][5] = {
@@ -139,6 +161,7 @@ tlhip_kernel_config_t select_config(const Problem& p) {
 
 int run_config(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t stream) {
   if (c.variant == VARIANT_TILED) return launch_gemm(p, c, stream);
+  if (c.variant == VARIANT_GEMV_MFMA) return launch_gemv_mfma(p, c, stream);
   return launch_gemv(p, c, stream);
 }
 
@@ -160,16 +183,16 @@ int autotune_problem(const Problem& p, double* best_us_out) {
     if (!ok) continue;
     double t[3];
     for (int i = 0; i < 3 && ok; ++i) {
-      hipEventRecord(e0, stream);
+      (void)hipEventRecord(e0, stream);
       ok = run_config(p, c, stream) == TLHIP_OK;
-      hipEventRecord(e1, stream);
+      (void)hipEventRecord(e1, stream);
       if (hipEventSynchronize(e1) != hipSuccess) {
         ok = false;
         rc = set_error(TLHIP_ERR_DEVICE, "autotune: hipEventSynchronize failed");
         break;
       }
       float ms = 0;
-      hipEventElapsedTime(&ms, e0, e1);
+      (void)hipEventElapsedTime(&ms, e0, e1);
       t[i] = ms * 1000.0;
     }
     if (rc) break;
@@ -180,8 +203,8 @@ int autotune_problem(const Problem& p, double* best_us_out) {
       best_cfg = c;
     }
   }
-  hipEventDestroy(e0);
-  hipEventDestroy(e1);
+  (void)hipEventDestroy(e0);
+  (void)hipEventDestroy(e1);
   g_autotuning = false;
   if (rc) return rc;
   {
@@ -296,7 +319,7 @@ int tlhip_gemv(const tlhip_qweight_t* w, const void* x, int x_dtype, int64_t m, 
   if (m > 16) return set_error(TLHIP_ERR_INVALID, "gemv: M=%lld above 16; use tlhip_gemm_prefill", (long long)m);
   tlhip_kernel_config_t c = select_config(p);
   if (c.variant == VARIANT_TILED) c = default_config(p);
-  return launch_gemv(p, c, resolve_stream(stream));
+  return run_config(p, c, resolve_stream(stream));
 }
 
 int tlhip_gemm_prefill(const tlhip_qweight_t* w, const void* x, int x_dtype, int64_t m, void* y, int y_dtype,
@@ -318,7 +341,7 @@ int tlhip_gemm_prefill(const tlhip_qweight_t* w, const void* x, int x_dtype, int
 
 static int matmul_with(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t stream) {
   if (c.variant == VARIANT_TILED) return launch_gemm(p, c, stream);
-  if (p.m <= 16) return launch_gemv(p, c, stream);
+  if (p.m <= 16) return run_config(p, c, stream);
   // f32 activations (or a shape the tiled kernel rejects) above 16 rows: GEMV
   // passes of 16 rows.  Declared, slow: every pass streams the weights again.
   const int xb = p.x_dtype == TLHIP_F16 ? 2 : 4, yb = p.y_dtype == TLHIP_F16 ? 2 : 4;
@@ -327,7 +350,7 @@ static int matmul_with(const Problem& p, const tlhip_kernel_config_t& c, hipStre
     q.m = std::min<int64_t>(16, p.m - m0);
     q.x = (const char*)p.x + m0 * p.k * xb;
     q.y = (char*)p.y + m0 * p.n * yb;
-    int rc = launch_gemv(q, c, stream);
+    int rc = run_config(q, c, stream);
     if (rc) return rc;
   }
   return TLHIP_OK;
@@ -348,7 +371,7 @@ int tlhip_matmul_quantized(const tlhip_qweight_t* w, const void* x, int x_dtype,
     }
     if (!have) {
       // Tuning launches write y; the real launch below overwrites it.
-      hipStreamSynchronize(resolve_stream(stream));
+      (void)hipStreamSynchronize(resolve_stream(stream));
       rc = autotune_problem(p, nullptr);
       if (rc) return rc;
     }

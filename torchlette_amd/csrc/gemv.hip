@@ -47,21 +47,6 @@ struct GemvArgs {
   DevEpilogue epi;
 };
 
-template <int FMT>
-struct FmtTraits;
-template <>
-struct FmtTraits<TLHIP_FMT_INT4_GROUPED> {
-  static constexpr int CW = 32;
-};
-template <>
-struct FmtTraits<TLHIP_FMT_INT8_GROUPED> {
-  static constexpr int CW = 16;
-};
-template <>
-struct FmtTraits<TLHIP_FMT_INT8_ROW> {
-  static constexpr int CW = 16;
-};
-
 // dot of one 16-byte weight chunk with the matching x chunk held as NQ u32x4.
 template <int FMT, typename XT>
 struct ChunkDot;

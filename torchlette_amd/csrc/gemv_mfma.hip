@@ -1,0 +1,344 @@
+// Skinny GEMM (2 <= M <= 16 activation rows) over packed weights on the matrix
+// cores: the weights are streamed from HBM exactly once whatever M is.
+//
+// One workgroup owns a block of 16 weight rows; its waves split K.  A wave
+// feeds v_mfma_f32_16x16x32_f16 with
+//   A = activations  (lane l supplies x[m = l%16][8 k-values of sub-block l/16])
+//   B = weights      (lane l supplies w[n = l%16][the same 8 k-values])
+//   D = 16 m x 16 n  (lane l holds D[m = 4*(l/16)+r][n = l%16], r = 0..3)
+// so every lane's four accumulators belong to ONE weight row n, and the
+// per-group scale of that row is applied to the f32 result of each MFMA
+// (acc += s * d).  The weights enter the MFMA as exact small integers in f16
+// and the activations are f16 already, so every product is exact and nothing
+// is rounded before the f32 accumulate.
+//
+// Weight loads are 16 bytes per lane.  For int4 (32 weights = one scale group
+// per load) the four lanes that share a row exchange words with
+// v_permlane32_swap / v_permlane16_swap (a 4x4 transpose), so that one MFMA
+// covers exactly one scale group.  For int8 a 16-byte load is half an MFMA's K;
+// the k-order inside an MFMA is free as long as the activations use the same
+// order, so no exchange is needed.
+//
+// Activations are staged in LDS in MFMA operand order (conflict-free 16-byte
+// reads, consecutive lanes on consecutive units), K-sliced when M*K*2 bytes
+// exceed the LDS budget.  Per-wave partial tiles are combined through LDS.
+#include "device_utils.h"
+
+namespace tlhip {
+namespace {
+
+struct MfmaArgs {
+  const u32x4* packed;
+  const void* scales;
+  const _Float16* x;
+  void* y;
+  int64_t n;
+  int k;
+  int m;
+  int nchunks;        // 16-byte chunks per weight row
+  int cpg_shift;      // log2(chunks per scale group), grouped formats
+  int groups_per_row;
+  int iters;          // wave iterations over K: 4 chunks each
+  int slice_iters;    // iterations whose activations are resident in LDS at once
+  int nslices;
+  int nblocks;        // 16-row blocks
+  float alpha;
+  float scale_mul;
+  int y_dtype;
+  DevEpilogue epi;
+};
+
+template <int FMT>
+struct MfmaTraits;
+template <>
+struct MfmaTraits<TLHIP_FMT_INT4_GROUPED> {
+  static constexpr int STEPS = 4;        // MFMAs per iteration (4 chunks x 32 weights)
+};
+template <>
+struct MfmaTraits<TLHIP_FMT_INT8_GROUPED> {
+  static constexpr int STEPS = 2;        // 4 chunks x 16 weights = 64 k
+};
+template <>
+struct MfmaTraits<TLHIP_FMT_INT8_ROW> {
+  static constexpr int STEPS = 2;
+};
+
+__device__ __forceinline__ half8_t join8(const half2_t (&h)[4]) {
+  half8_t r;
+  r[0] = h[0][0]; r[1] = h[0][1]; r[2] = h[1][0]; r[3] = h[1][1];
+  r[4] = h[2][0]; r[5] = h[2][1]; r[6] = h[3][0]; r[7] = h[3][1];
+  return r;
+}
+
+// 4x4 transpose of 32-bit words across the four lanes l, l+16, l+32, l+48:
+// afterwards register i of lane-group g holds what register g of lane-group i
+// held.  Two swap stages: distance 32 on register pairs (0,2) (1,3), then
+// distance 16 on pairs (0,1) (2,3).
+__device__ __forceinline__ void transpose4(uint32_t& r0, uint32_t& r1, uint32_t& r2, uint32_t& r3) {
+  // v_permlane32_swap: lanes 32..63 of the first operand <-> lanes 0..31 of the second
+  auto s02 = __builtin_amdgcn_permlane32_swap(r0, r2, false, false);
+  r0 = s02[0]; r2 = s02[1];
+  auto s13 = __builtin_amdgcn_permlane32_swap(r1, r3, false, false);
+  r1 = s13[0]; r3 = s13[1];
+  // v_permlane16_swap: odd 16-lane rows of the first operand <-> even rows of the second
+  auto s01 = __builtin_amdgcn_permlane16_swap(r0, r1, false, false);
+  r0 = s01[0]; r1 = s01[1];
+  auto s23 = __builtin_amdgcn_permlane16_swap(r2, r3, false, false);
+  r2 = s23[0]; r3 = s23[1];
+}
+
+// LDS unit (16 bytes) index of the activations for MFMA step t (global step
+// index inside the slice), k sub-block g, activation row m.
+__device__ __forceinline__ int x_unit(int t, int g, int m, int mrows) { return (t * 4 + g) * mrows + m; }
+
+template <int FMT, int U>
+__global__ __launch_bounds__(1024) void gemv_mfma_kernel(const MfmaArgs a) {
+  using Tr = MfmaTraits<FMT>;
+  constexpr int STEPS = Tr::STEPS;
+  constexpr bool GROUPED = (FMT != TLHIP_FMT_INT8_ROW);
+  extern __shared__ u32x4 lds[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int nwaves = blockDim.x >> 6;
+  const int nl = lane & 15;   // weight row inside the block / activation row for the A operand
+  const int g = lane >> 4;    // k sub-block
+  const int mrows = a.m;
+  const int ml = nl < mrows ? nl : mrows - 1;  // rows beyond M alias the last row; never stored
+  float* partial = (float*)(lds + (size_t)a.slice_iters * STEPS * 4 * mrows);
+
+  // Stage the activations of one K slice in MFMA operand order.
+  auto stage = [&](int slice) {
+    const int it0 = slice * a.slice_iters;
+    const int nit = min(a.slice_iters, a.iters - it0);
+    const int units = nit * STEPS * 4 * mrows;
+    for (int u = tid; u < units; u += blockDim.x) {
+      const int m = u % mrows;
+      const int tg = u / mrows;
+      const int gg = tg & 3;
+      const int t = tg >> 2;  // step inside the slice
+      int kbase;
+      if (FMT == TLHIP_FMT_INT4_GROUPED) {
+        kbase = (it0 * STEPS + t) * 32 + gg * 8;             // group t, word gg
+      } else {
+        const int it = it0 + (t >> 1), j = t & 1;
+        kbase = it * 64 + gg * 16 + j * 8;                   // chunk gg of the iteration, half j
+      }
+      u32x4 v = *(const u32x4*)(a.x + (size_t)m * a.k + kbase);
+      if (FMT == TLHIP_FMT_INT4_GROUPED) v = permute_x_for_int4(v);
+      lds[u] = v;
+    }
+  };
+
+  if (a.nslices == 1) {
+    stage(0);
+    __syncthreads();
+  }
+
+  for (int rb = blockIdx.x; rb < a.nblocks; rb += gridDim.x) {
+    const int64_t row = min((int64_t)rb * 16 + nl, a.n - 1);
+    const u32x4* wrow = a.packed + row * a.nchunks;
+    const uint16_t* srow = GROUPED ? (const uint16_t*)a.scales + row * a.groups_per_row : nullptr;
+    float4_t acc = {0.f, 0.f, 0.f, 0.f};
+
+    for (int slice = 0; slice < a.nslices; ++slice) {
+      if (a.nslices > 1) {
+        __syncthreads();
+        stage(slice);
+        __syncthreads();
+      }
+      const int it_begin = slice * a.slice_iters;
+      const int it_end = min(it_begin + a.slice_iters, a.iters);
+      for (int itb = it_begin + wave; itb < it_end; itb += nwaves * U) {
+        u32x4 wv[U];
+        float sv[U][STEPS];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const int it = itb + u * nwaves;
+          if (it < it_end) {
+            wv[u] = __builtin_nontemporal_load(wrow + it * 4 + g);
+            if (GROUPED) {
+#pragma unroll
+              for (int s = 0; s < STEPS; ++s) {
+                // int4: step s is chunk 4*it+s; int8: both steps lie in chunks 4*it .. 4*it+3
+                const int chunk = FMT == TLHIP_FMT_INT4_GROUPED ? it * 4 + s : it * 4;
+                sv[u][s] = half_bits_to_float(srow[chunk >> a.cpg_shift]);
+              }
+            }
+          }
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const int it = itb + u * nwaves;
+          if (it < it_end) {
+            const int tl = (it - it_begin) * STEPS;
+            uint32_t w0 = wv[u].x, w1 = wv[u].y, w2 = wv[u].z, w3 = wv[u].w;
+            half8_t bw[STEPS];
+            if (FMT == TLHIP_FMT_INT4_GROUPED) {
+              transpose4(w0, w1, w2, w3);  // register s now holds word g of chunk 4*it+s
+              const uint32_t ws[4] = {w0, w1, w2, w3};
+#pragma unroll
+              for (int s = 0; s < 4; ++s) {
+                half2_t h[4];
+                unpack_int4_word(ws[s], h);
+                bw[s] = join8(h);
+              }
+            } else {
+              const uint32_t ws[4] = {w0, w1, w2, w3};
+#pragma unroll
+              for (int s = 0; s < 2; ++s) {
+                half2_t h[4];
+                unpack_int8_word(ws[2 * s], h);
+                unpack_int8_word(ws[2 * s + 1], h + 2);
+                bw[s] = join8(h);
+              }
+            }
+            float4_t d[STEPS];
+#pragma unroll
+            for (int s = 0; s < STEPS; ++s) {
+              const u32x4 xa = lds[x_unit(tl + s, g, ml, mrows)];
+              const float4_t zero = {0.f, 0.f, 0.f, 0.f};
+              d[s] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, xa), bw[s], zero, 0, 0, 0);
+            }
+#pragma unroll
+            for (int s = 0; s < STEPS; ++s) {
+              if (GROUPED) {
+                acc[0] = fmaf(sv[u][s], d[s][0], acc[0]);
+                acc[1] = fmaf(sv[u][s], d[s][1], acc[1]);
+                acc[2] = fmaf(sv[u][s], d[s][2], acc[2]);
+                acc[3] = fmaf(sv[u][s], d[s][3], acc[3]);
+              } else {
+                acc[0] += d[s][0]; acc[1] += d[s][1]; acc[2] += d[s][2]; acc[3] += d[s][3];
+              }
+            }
+          }
+        }
+      }
+    }
+
+    // combine the waves' partial tiles through LDS: partial[wave][m][n]
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < 4; ++r) partial[(wave * 16 + (4 * g + r)) * 16 + nl] = acc[r];
+    __syncthreads();
+    if (tid < 256) {
+      const int m = tid >> 4, nn = tid & 15;
+      const int64_t orow = (int64_t)rb * 16 + nn;
+      if (m < mrows && orow < a.n) {
+        float s = 0.f;
+        for (int w = 0; w < nwaves; ++w) s += partial[(w * 16 + m) * 16 + nn];
+        float rs = a.scale_mul;
+        if (!GROUPED) rs *= ((const float*)a.scales)[orow];
+        float v = s * rs * a.alpha;
+        v = apply_epilogue(a.epi, v, orow);
+        store_out(a.y, a.y_dtype, (int64_t)m * a.n + orow, v);
+      }
+    }
+  }
+}
+
+constexpr size_t kXLdsBudget = 136 * 1024;
+
+}  // namespace
+
+bool gemv_mfma_config_applicable(const Problem& p, const tlhip_kernel_config_t& c, const char** why) {
+  static const char* reasons[] = {
+      "not the gemv_mfma variant",
+      "waves per workgroup must be 4, 8 or 16",
+      "activations must be f16",
+      "M must be 1..16",
+      "K must be a multiple of 128 (int4) or 64 (int8)",
+      "group size must be a multiple of 32 (int4) or 64 (int8)",
+      "unroll must be 1, 2 or 4",
+  };
+  auto fail = [&](int i) {
+    if (why) *why = reasons[i];
+    return false;
+  };
+  if (c.variant != VARIANT_GEMV_MFMA) return fail(0);
+  if (c.p0 != 4 && c.p0 != 8 && c.p0 != 16) return fail(1);
+  if (p.x_dtype != TLHIP_F16) return fail(2);
+  if (p.m < 1 || p.m > 16) return fail(3);
+  const int kper = p.format == TLHIP_FMT_INT4_GROUPED ? 128 : 64;
+  if (p.k % kper != 0) return fail(4);
+  if (p.format == TLHIP_FMT_INT4_GROUPED && p.group_size % 32 != 0) return fail(5);
+  if (p.format == TLHIP_FMT_INT8_GROUPED && p.group_size % 64 != 0) return fail(5);
+  if (c.p1 != 1 && c.p1 != 2 && c.p1 != 4) return fail(6);
+  return true;
+}
+
+template <int FMT>
+static int launch_mfma_u(int unroll, const MfmaArgs& a, int grid, int threads, size_t lds_bytes, hipStream_t stream) {
+  const void* fn;
+  switch (unroll) {
+    case 1: fn = (const void*)gemv_mfma_kernel<FMT, 1>; break;
+    case 2: fn = (const void*)gemv_mfma_kernel<FMT, 2>; break;
+    default: fn = (const void*)gemv_mfma_kernel<FMT, 4>; break;
+  }
+  if (lds_bytes > 64 * 1024)
+    TLHIP_CHECK_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+  void* args[] = {(void*)&a};
+  TLHIP_CHECK_HIP(hipLaunchKernel(fn, dim3(grid), dim3(threads), args, lds_bytes, stream));
+  return TLHIP_OK;
+}
+
+int launch_gemv_mfma(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t stream) {
+  const char* why = nullptr;
+  if (!gemv_mfma_config_applicable(p, c, &why))
+    return set_error(TLHIP_ERR_INVALID, "gemv_mfma: config not applicable: %s", why);
+  if (p.n == 0 || p.m == 0) return TLHIP_OK;
+  const bool int4 = p.format == TLHIP_FMT_INT4_GROUPED;
+  const int cw = int4 ? 32 : 16;
+  const int steps = int4 ? 4 : 2;
+  MfmaArgs a;
+  a.packed = (const u32x4*)p.packed;
+  a.scales = p.scales;
+  a.x = (const _Float16*)p.x;
+  a.y = p.y;
+  a.n = p.n;
+  a.k = (int)p.k;
+  a.m = (int)p.m;
+  a.nchunks = (int)(p.k / cw);
+  a.cpg_shift = p.format == TLHIP_FMT_INT8_ROW ? 0 : __builtin_ctz((unsigned)(p.group_size / cw));
+  a.groups_per_row = p.format == TLHIP_FMT_INT8_ROW ? 0 : (int)(p.k / p.group_size);
+  a.iters = a.nchunks / 4;
+  a.nblocks = (int)((p.n + 15) / 16);
+  a.alpha = p.alpha;
+  a.scale_mul = p.format == TLHIP_FMT_INT8_GROUPED ? (1.0f / 127.0f) : 1.0f;
+  a.y_dtype = p.y_dtype;
+  a.epi = p.epi;
+  const int waves = c.p0;
+  const size_t partial_bytes = (size_t)waves * 256 * sizeof(float);
+  const size_t iter_x_bytes = (size_t)steps * 4 * a.m * 16;  // LDS bytes of activations per iteration
+  int max_iters = (int)((kXLdsBudget - partial_bytes) / iter_x_bytes);
+  if (max_iters >= a.iters) {
+    a.slice_iters = a.iters;
+    a.nslices = 1;
+  } else {
+    int si = max_iters / waves * waves;  // every slice starts on the same wave phase
+    if (si <= 0) return set_error(TLHIP_ERR_INVALID, "gemv_mfma: K slice does not fit LDS");
+    a.slice_iters = si;
+    a.nslices = (a.iters + si - 1) / si;
+  }
+  const size_t lds_bytes = iter_x_bytes * a.slice_iters + partial_bytes;
+  const int threads = waves * 64;
+  const int cus = device_cu_count();
+  int per_cu = 2048 / threads;
+  const int by_lds = (int)((160 * 1024) / lds_bytes);
+  if (by_lds < per_cu) per_cu = by_lds < 1 ? 1 : by_lds;
+  int grid = a.nblocks < cus * per_cu ? a.nblocks : cus * per_cu;
+  if (grid < 1) grid = 1;
+  int rc;
+  switch (p.format) {
+    case TLHIP_FMT_INT4_GROUPED: rc = launch_mfma_u<TLHIP_FMT_INT4_GROUPED>(c.p1, a, grid, threads, lds_bytes, stream); break;
+    case TLHIP_FMT_INT8_GROUPED: rc = launch_mfma_u<TLHIP_FMT_INT8_GROUPED>(c.p1, a, grid, threads, lds_bytes, stream); break;
+    default: rc = launch_mfma_u<TLHIP_FMT_INT8_ROW>(c.p1, a, grid, threads, lds_bytes, stream); break;
+  }
+  if (rc) return rc;
+  TLHIP_CHECK_HIP(hipGetLastError());
+  count_gemv_dispatch();
+  return TLHIP_OK;
+}
+
+}  // namespace tlhip

@@ -86,8 +86,8 @@ int tlhip_init(int device_index) {
 int tlhip_shutdown(void) {
   std::lock_guard<std::mutex> lock(g_mutex);
   if (!g_init) return TLHIP_OK;
-  hipStreamSynchronize(g_stream);
-  hipStreamDestroy(g_stream);
+  (void)hipStreamSynchronize(g_stream);
+  (void)hipStreamDestroy(g_stream);
   g_stream = nullptr;
   g_init = false;
   g_device = -1;
@@ -225,6 +225,39 @@ int tlhip_event_elapsed_us(tlhip_event_t start, tlhip_event_t stop, double* out_
   float ms = 0.f;
   TLHIP_CHECK_HIP(hipEventElapsedTime(&ms, static_cast<hipEvent_t>(start), static_cast<hipEvent_t>(stop)));
   *out_us = (double)ms * 1000.0;
+  return TLHIP_OK;
+}
+
+int tlhip_graph_begin_capture(tlhip_stream_t stream) {
+  TLHIP_REQUIRE_INIT();
+  TLHIP_CHECK_HIP(hipStreamBeginCapture(resolve_stream(stream), hipStreamCaptureModeThreadLocal));
+  return TLHIP_OK;
+}
+
+int tlhip_graph_end_capture(tlhip_stream_t stream, tlhip_graph_t* out) {
+  TLHIP_REQUIRE_INIT();
+  if (!out) return set_error(TLHIP_ERR_INVALID, "tlhip_graph_end_capture: null output");
+  hipGraph_t graph = nullptr;
+  TLHIP_CHECK_HIP(hipStreamEndCapture(resolve_stream(stream), &graph));
+  hipGraphExec_t exec = nullptr;
+  hipError_t e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+  (void)hipGraphDestroy(graph);
+  if (e != hipSuccess) return set_error(TLHIP_ERR_DEVICE, "hipGraphInstantiate failed: %s", hipGetErrorString(e));
+  *out = exec;
+  return TLHIP_OK;
+}
+
+int tlhip_graph_launch(tlhip_graph_t graph, tlhip_stream_t stream) {
+  TLHIP_REQUIRE_INIT();
+  if (!graph) return set_error(TLHIP_ERR_INVALID, "tlhip_graph_launch: null graph");
+  TLHIP_CHECK_HIP(hipGraphLaunch(static_cast<hipGraphExec_t>(graph), resolve_stream(stream)));
+  return TLHIP_OK;
+}
+
+int tlhip_graph_destroy(tlhip_graph_t graph) {
+  TLHIP_REQUIRE_INIT();
+  if (!graph) return TLHIP_OK;
+  TLHIP_CHECK_HIP(hipGraphExecDestroy(static_cast<hipGraphExec_t>(graph)));
   return TLHIP_OK;
 }
 
