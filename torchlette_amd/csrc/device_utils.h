@@ -114,6 +114,16 @@ __device__ __forceinline__ void unpack_int8_word(uint32_t w, half2_t out[2]) {
   out[1] = __builtin_bit_cast(half2_t, a1) + sub;
 }
 
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits
+// for every outstanding global load of the wave (vmcnt(0)), which would drain
+// the weight loads that were deliberately issued ahead; here only the wave's
+// own LDS operations are waited for (lgkmcnt(0)) before s_barrier.
+// s_waitcnt immediate on gfx9: vmcnt = 63 (no wait), expcnt = 7 (no wait), lgkmcnt = 0.
+__device__ __forceinline__ void lds_barrier() {
+  __builtin_amdgcn_s_waitcnt(0xc07f);
+  __builtin_amdgcn_s_barrier();
+}
+
 // ------------------------------------------------------------- reductions
 template <int CTRL>
 __device__ __forceinline__ float dpp_add(float v) {

@@ -57,7 +57,7 @@ bool env_autotune() {
   return e && !strcmp(e, "1");
 }
 
-tlhip_kernel_config_t gemv_cfg(int lpr, int r, int waves, int kw) {
+tlhip_kernel_config_t gemv_cfg(int lpr, int r, int waves, int kw, int unroll) {
   tlhip_kernel_config_t c;
   memset(&c, 0, sizeof c);
   c.variant = VARIANT_GEMV;
@@ -65,15 +65,17 @@ tlhip_kernel_config_t gemv_cfg(int lpr, int r, int waves, int kw) {
   c.p1 = r;
   c.p2 = waves;
   c.p3 = kw;
+  c.p4 = unroll;
   return c;
 }
 
-tlhip_kernel_config_t mfma_cfg(int waves, int unroll) {
+tlhip_kernel_config_t mfma_cfg(int waves, int unroll, int kw) {
   tlhip_kernel_config_t c;
   memset(&c, 0, sizeof c);
   c.variant = VARIANT_GEMV_MFMA;
   c.p0 = waves;
   c.p1 = unroll;
+  c.p2 = kw;
   return c;
 }
 
@@ -105,7 +107,7 @@ tlhip_kernel_config_t default_config(const Problem& p) {
   }
   // three or more activation rows: the matrix-core kernel streams the weights once
   if (p.m >= 3 && p.m <= 16) {
-    tlhip_kernel_config_t c = mfma_cfg(8, 2);
+    tlhip_kernel_config_t c = mfma_cfg(8, 2, p.n >= 32768 ? 1 : 8);
     if (gemv_mfma_config_applicable(p, c, nullptr)) return c;
   }
   // lanes per row: keep every lane busy for short rows
@@ -115,7 +117,7 @@ tlhip_kernel_config_t default_config(const Problem& p) {
   const int r = p.m >= 4 ? 2 : 1;
   // enough row blocks to give every CU several waves; big N walks with a stride
   int waves = 4;
-  return gemv_cfg(lpr, r, waves, 1);
+  return gemv_cfg(lpr, r, waves, 1, 2);
 }
 
 std::vector<tlhip_kernel_config_t> candidates(const Problem& p) {
@@ -124,18 +126,21 @@ std::vector<tlhip_kernel_config_t> candidates(const Problem& p) {
     for (int lpr : {16, 32, 64})
       for (int r : {1, 2, 4})
         for (int waves : {2, 4, 8})
-          for (int kw : {1, 2, 4}) {
-            if (kw > waves) continue;
-            tlhip_kernel_config_t c = gemv_cfg(lpr, r, waves, kw);
-            if (gemv_config_applicable(p, c, nullptr)) out.push_back(c);
-          }
+          for (int kw : {1, 2, 4})
+            for (int unroll : {2, 4, 8}) {
+              if (kw > waves) continue;
+              tlhip_kernel_config_t c = gemv_cfg(lpr, r, waves, kw, unroll);
+              if (gemv_config_applicable(p, c, nullptr)) out.push_back(c);
+            }
   }
   if (p.m <= 16) {
     for (int waves : {4, 8, 16})
-      for (int unroll : {1, 2, 4}) {
-        tlhip_kernel_config_t c = mfma_cfg(waves, unroll);
-        if (gemv_mfma_config_applicable(p, c, nullptr)) out.push_back(c);
-      }
+      for (int unroll : {1, 2, 4})
+        for (int kw : {1, 2, 4, 8, 16}) {
+          if (kw > waves) continue;
+          tlhip_kernel_config_t c = mfma_cfg(waves, unroll, kw);
+          if (gemv_mfma_config_applicable(p, c, nullptr)) out.push_back(c);
+        }
   }
   if (p.x_dtype == TLHIP_F16 && p.m >= 16) {
     static const int tiles[][5] = {

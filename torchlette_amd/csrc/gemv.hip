@@ -35,9 +35,10 @@ struct GemvArgs {
   int cpg_shift;         // grouped formats: log2(chunks sharing one scale)
   int groups_per_row;
   int lpr;               // lanes per row
-  int kw;                // waves splitting K inside a workgroup
-  int slice_chunks;      // chunks of x resident in LDS at a time
-  int nslices;
+  int lpr_shift;
+  int kw;                // waves splitting K inside a workgroup (power of two)
+  int kw_shift;
+  int nsteps;            // batches per row block
   int nblocks;           // row blocks
   int rows_per_wave;
   int rows_per_wg;
@@ -158,8 +159,17 @@ struct ChunkDot<TLHIP_FMT_INT4_GROUPED, float> {
 };
 
 // LDS layout of the staged activations: 16-byte unit (row m, quarter qd of
-// chunk c) lives at unit index (m*NQ + qd)*slice_chunks + c, so the lanes of a
-// row group, which hold consecutive c, read consecutive units.
+// chunk c) lives at unit index (m*NQ + qd)*nchunks + c, so the lanes of a row
+// group, which hold consecutive c, read consecutive units.
+//
+// Work of one lane is a sequence of batches: U chunks x R rows of 16-byte
+// weight loads (plus their scales).  The batches of all row blocks of the
+// workgroup form one software pipeline: the loads of batch i+1 are issued
+// before batch i is consumed, and the very first batch is issued right after
+// the activation loads and before the LDS store and barrier, so HBM latency
+// overlaps the staging, the arithmetic and the reductions.  The hot path has no
+// per-lane branches: out-of-range chunks load a clamped address and contribute
+// zero through their scale (or a select).
 template <int FMT, typename XT, int MT, int R, int U>
 __global__ __launch_bounds__(512) void gemv_kernel(const GemvArgs a) {
   using Dot = ChunkDot<FMT, XT>;
@@ -170,109 +180,81 @@ __global__ __launch_bounds__(512) void gemv_kernel(const GemvArgs a) {
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  const int kw_idx = wave % a.kw;
-  const int rg = wave / a.kw;
-  const int sub = lane / a.lpr;
-  const int lj = lane - sub * a.lpr;
+  const int kw_idx = wave & (a.kw - 1);
+  const int rg = wave >> a.kw_shift;
+  const int sub = lane >> a.lpr_shift;
+  const int lj = lane & (a.lpr - 1);
   const int cstride = a.lpr * a.kw;
   const int cfirst = kw_idx * a.lpr + lj;
   const int x_units_per_row = a.k * (int)sizeof(XT) / 16;  // 16-byte units per activation row
   const u32x4* xg = (const u32x4*)a.x;
-  u32x4* partial = lds + (size_t)MT * NQ * a.slice_chunks;  // kw x rows_per_wg x MT floats, if kw > 1
+  float* partial = (float*)(lds + (size_t)MT * NQ * a.nchunks);  // kw x rows_per_wg x MT, if kw > 1
+  const int row_in_wg = rg * a.rows_per_wave + sub * R;
+  const int last_chunk = a.nchunks - 1;
 
-  auto stage = [&](int slice) {
-    const int c0 = slice * a.slice_chunks;
-    const int cn = min(a.slice_chunks, a.nchunks - c0);
-    const int units = cn * NQ;
-    for (int m = 0; m < MT; ++m) {
-      const int mm = m < a.m ? m : a.m - 1;  // rows beyond m replicate the last row; never stored
-      for (int u = tid; u < units; u += blockDim.x) {
-        u32x4 v = xg[(size_t)mm * x_units_per_row + (size_t)c0 * NQ + u];
-        if (FMT == TLHIP_FMT_INT4_GROUPED && sizeof(XT) == 2) v = permute_x_for_int4(v);
-        const int c = u / NQ, qd = u - c * NQ;
-        lds[(m * NQ + qd) * a.slice_chunks + c] = v;
+  // Only raw loaded values live here: converting or selecting on a loaded value
+  // at issue time would make the wave wait for the load it has just issued.
+  struct Batch {
+    u32x4 w[U][R];
+    uint16_t s[U][R];  // f16 bits of the chunk's group scale
+    float rs[R];       // int8-row: the row's scale, fetched with the first batch of a row block
+  };
+
+  // Issue the loads of one batch: chunks cb + u*cstride (u < U) of R rows.
+  auto load_batch = [&](Batch& b, int rb, int cb, bool first) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      // tail rows recompute the last row; their store is masked
+      const int64_t row = min((int64_t)rb * a.rows_per_wg + row_in_wg + r, a.n - 1);
+      const u32x4* wrow = a.packed + row * a.nchunks;
+      const uint16_t* srow = (const uint16_t*)a.scales + row * a.groups_per_row;
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int c = cb + u * cstride;
+        const int cc = min(c, last_chunk);
+        b.w[u][r] = __builtin_nontemporal_load(wrow + cc);
+        if (GROUPED) b.s[u][r] = srow[cc >> a.cpg_shift];
+      }
+      if (!GROUPED && first) b.rs[r] = ((const float*)a.scales)[row];
+    }
+  };
+
+  float acc[R][MT];
+  float row_scale[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    row_scale[r] = 1.f;
+#pragma unroll
+    for (int m = 0; m < MT; ++m) acc[r][m] = 0.f;
+  }
+
+  auto compute_batch = [&](const Batch& b, int cb) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int c = cb + u * cstride;
+      const int cc = min(c, last_chunk);
+      u32x4 xv[MT][NQ];
+#pragma unroll
+      for (int m = 0; m < MT; ++m)
+#pragma unroll
+        for (int qd = 0; qd < NQ; ++qd) xv[m][qd] = lds[(m * NQ + qd) * a.nchunks + cc];
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        Dot d;
+        d.unpack(b.w[u][r]);
+        const float sc = GROUPED ? (c <= last_chunk ? half_bits_to_float(b.s[u][r]) : 0.f) : 0.f;
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+          const float part = d.dot(xv[m]);
+          if (GROUPED) acc[r][m] = fmaf(sc, part, acc[r][m]);
+          else acc[r][m] += (c <= last_chunk ? part : 0.f);
+        }
       }
     }
   };
 
-  if (a.nslices == 1) {
-    stage(0);
-    __syncthreads();
-  }
-
-  for (int rb = blockIdx.x; rb < a.nblocks; rb += gridDim.x) {
-    const int64_t row0 = (int64_t)rb * a.rows_per_wg + rg * a.rows_per_wave + sub * R;
-    float acc[R][MT];
-#pragma unroll
-    for (int r = 0; r < R; ++r)
-#pragma unroll
-      for (int m = 0; m < MT; ++m) acc[r][m] = 0.f;
-
-    const u32x4* wrow[R];
-    const uint16_t* srow[R];
-    float row_scale[R];
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-      const int64_t row = min(row0 + r, a.n - 1);  // tail rows recompute the last row; store is masked
-      wrow[r] = a.packed + row * a.nchunks;
-      if (GROUPED) {
-        srow[r] = (const uint16_t*)a.scales + row * a.groups_per_row;
-        row_scale[r] = 1.f;
-      } else {
-        srow[r] = nullptr;
-        row_scale[r] = ((const float*)a.scales)[row];
-      }
-    }
-
-    for (int slice = 0; slice < a.nslices; ++slice) {
-      if (a.nslices > 1) {
-        __syncthreads();
-        stage(slice);
-        __syncthreads();
-      }
-      const int c_begin = slice * a.slice_chunks;
-      const int c_end = min(c_begin + a.slice_chunks, a.nchunks);
-      for (int cb = c_begin + cfirst; cb < c_end; cb += cstride * U) {
-        u32x4 wv[U][R];
-        float sv[U][R];
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-          const int c = cb + u * cstride;
-          if (c < c_end) {
-#pragma unroll
-            for (int r = 0; r < R; ++r) {
-              wv[u][r] = __builtin_nontemporal_load(wrow[r] + c);
-              if (GROUPED) sv[u][r] = half_bits_to_float(srow[r][c >> a.cpg_shift]);
-            }
-          }
-        }
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-          const int c = cb + u * cstride;
-          if (c < c_end) {
-            const int cl = c - c_begin;
-            u32x4 xv[MT][NQ];
-#pragma unroll
-            for (int m = 0; m < MT; ++m)
-#pragma unroll
-              for (int qd = 0; qd < NQ; ++qd) xv[m][qd] = lds[(m * NQ + qd) * a.slice_chunks + cl];
-#pragma unroll
-            for (int r = 0; r < R; ++r) {
-              Dot d;
-              d.unpack(wv[u][r]);
-#pragma unroll
-              for (int m = 0; m < MT; ++m) {
-                const float part = d.dot(xv[m]);
-                if (GROUPED) acc[r][m] = fmaf(sv[u][r], part, acc[r][m]);
-                else acc[r][m] += part;
-              }
-            }
-          }
-        }
-      }
-    }
-
-    // lanes of a row group -> one sum (all lanes of the group hold it)
+  // Reduce, combine K-split partials, apply the epilogue and store one row block.
+  auto finish = [&](int rb) {
 #pragma unroll
     for (int r = 0; r < R; ++r)
 #pragma unroll
@@ -280,24 +262,21 @@ __global__ __launch_bounds__(512) void gemv_kernel(const GemvArgs a) {
 
     if (a.kw > 1) {
       // split-K combine through LDS: partial[kw][row in wg][m]
-      float* pf = (float*)partial;
-      __syncthreads();
+      lds_barrier();
       if (lj == 0) {
 #pragma unroll
         for (int r = 0; r < R; ++r)
 #pragma unroll
-          for (int m = 0; m < MT; ++m)
-            pf[((kw_idx * a.rows_per_wg) + rg * a.rows_per_wave + sub * R + r) * MT + m] = acc[r][m];
+          for (int m = 0; m < MT; ++m) partial[((kw_idx * a.rows_per_wg) + row_in_wg + r) * MT + m] = acc[r][m];
       }
-      __syncthreads();
+      lds_barrier();
       if (kw_idx == 0 && lj == 0) {
 #pragma unroll
         for (int r = 0; r < R; ++r)
 #pragma unroll
           for (int m = 0; m < MT; ++m) {
             float s = 0.f;
-            for (int w = 0; w < a.kw; ++w)
-              s += pf[((w * a.rows_per_wg) + rg * a.rows_per_wave + sub * R + r) * MT + m];
+            for (int w = 0; w < a.kw; ++w) s += partial[((w * a.rows_per_wg) + row_in_wg + r) * MT + m];
             acc[r][m] = s;
           }
       }
@@ -306,7 +285,7 @@ __global__ __launch_bounds__(512) void gemv_kernel(const GemvArgs a) {
     if (kw_idx == 0 && lj == 0) {
 #pragma unroll
       for (int r = 0; r < R; ++r) {
-        const int64_t row = row0 + r;
+        const int64_t row = (int64_t)rb * a.rows_per_wg + row_in_wg + r;
         if (row < a.n) {
 #pragma unroll
           for (int m = 0; m < MT; ++m) {
@@ -319,42 +298,133 @@ __global__ __launch_bounds__(512) void gemv_kernel(const GemvArgs a) {
         }
       }
     }
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+      for (int m = 0; m < MT; ++m) acc[r][m] = 0.f;
+  };
+
+  const int step_chunks = cstride * U;
+  const int nsteps = a.nsteps;
+  int rb = blockIdx.x, step = 0;
+  Batch cur;
+  // Order of issue matters: loads return in order, so the (few) activation
+  // loads go first, then the first weight batch; the LDS store then waits for
+  // the activations only, and the barrier for LDS only.
+  constexpr int XS = 4;  // activation units a thread holds while its weight loads are in flight
+  const int units = a.nchunks * NQ;
+  const int units_total = units * MT;
+  // idx -> (activation row m, 16-byte unit u) without a division: MT <= 4
+  auto split = [&](int idx, int& m, int& u) {
+    m = 0;
+    u = idx;
+#pragma unroll
+    for (int i = 1; i < MT; ++i)
+      if (u >= units) {
+        u -= units;
+        ++m;
+      }
+  };
+  auto x_src = [&](int idx) {
+    int m, u;
+    split(idx, m, u);
+    const int mm = m < a.m ? m : a.m - 1;  // rows beyond m replicate the last row; never stored
+    return xg + (size_t)mm * x_units_per_row + u;
+  };
+  auto x_dst = [&](int idx) {
+    int m, u;
+    split(idx, m, u);
+    const int c = u / NQ, qd = u - c * NQ;
+    return lds + (m * NQ + qd) * a.nchunks + c;
+  };
+  if (units_total <= XS * (int)blockDim.x) {
+    u32x4 xr[XS];
+#pragma unroll
+    for (int i = 0; i < XS; ++i) {
+      const int idx = min(tid + i * (int)blockDim.x, units_total - 1);
+      xr[i] = *x_src(idx);
+    }
+    load_batch(cur, rb, cfirst, true);
+#pragma unroll
+    for (int i = 0; i < XS; ++i) {
+      const int idx = tid + i * (int)blockDim.x;
+      if (idx < units_total) {
+        u32x4 v = xr[i];
+        if (FMT == TLHIP_FMT_INT4_GROUPED && sizeof(XT) == 2) v = permute_x_for_int4(v);
+        *x_dst(idx) = v;
+      }
+    }
+  } else {
+    for (int idx = tid; idx < units_total; idx += blockDim.x) {
+      u32x4 v = *x_src(idx);
+      if (FMT == TLHIP_FMT_INT4_GROUPED && sizeof(XT) == 2) v = permute_x_for_int4(v);
+      *x_dst(idx) = v;
+    }
+    load_batch(cur, rb, cfirst, true);
+  }
+  lds_barrier();
+  while (rb < a.nblocks) {
+    int nrb = rb, nstep = step + 1;
+    if (nstep == nsteps) {
+      nstep = 0;
+      nrb = rb + gridDim.x;
+    }
+    Batch nxt;
+    if (nrb < a.nblocks) load_batch(nxt, nrb, cfirst + nstep * step_chunks, nstep == 0);
+    if (!GROUPED && step == 0) {
+#pragma unroll
+      for (int r = 0; r < R; ++r) row_scale[r] = cur.rs[r];
+    }
+    compute_batch(cur, cfirst + step * step_chunks);
+    if (step == nsteps - 1) finish(rb);
+    cur = nxt;
+    rb = nrb;
+    step = nstep;
   }
 }
 
-constexpr int kLdsBudget = 64 * 1024;
+constexpr int kLdsBudget = 128 * 1024;
 
-template <int FMT, typename XT, int MT, int R>
+template <int FMT, typename XT, int MT, int R, int U>
 int launch_t(const GemvArgs& a, int threads, int grid, size_t lds_bytes, hipStream_t stream) {
-  hipLaunchKernelGGL((gemv_kernel<FMT, XT, MT, R, 2>), dim3(grid), dim3(threads), lds_bytes, stream, a);
+  const void* fn = (const void*)gemv_kernel<FMT, XT, MT, R, U>;
+  if (lds_bytes > 64 * 1024)
+    TLHIP_CHECK_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+  void* args[] = {(void*)&a};
+  TLHIP_CHECK_HIP(hipLaunchKernel(fn, dim3(grid), dim3(threads), args, lds_bytes, stream));
   return TLHIP_OK;
 }
 
+// (rows per lane group, chunks in flight) pairs that are instantiated: R*U <= 8.
 template <int FMT, typename XT, int MT>
-int launch_r(int r, const GemvArgs& a, int threads, int grid, size_t lds_bytes, hipStream_t stream) {
-  switch (r) {
-    case 1: return launch_t<FMT, XT, MT, 1>(a, threads, grid, lds_bytes, stream);
-    case 2: return launch_t<FMT, XT, MT, 2>(a, threads, grid, lds_bytes, stream);
-    case 4: return launch_t<FMT, XT, MT, 4>(a, threads, grid, lds_bytes, stream);
+int launch_r(int r, int u, const GemvArgs& a, int threads, int grid, size_t lds_bytes, hipStream_t stream) {
+  switch (r * 16 + u) {
+    case 1 * 16 + 2: return launch_t<FMT, XT, MT, 1, 2>(a, threads, grid, lds_bytes, stream);
+    case 1 * 16 + 4: return launch_t<FMT, XT, MT, 1, 4>(a, threads, grid, lds_bytes, stream);
+    case 1 * 16 + 8: return launch_t<FMT, XT, MT, 1, 8>(a, threads, grid, lds_bytes, stream);
+    case 2 * 16 + 2: return launch_t<FMT, XT, MT, 2, 2>(a, threads, grid, lds_bytes, stream);
+    case 2 * 16 + 4: return launch_t<FMT, XT, MT, 2, 4>(a, threads, grid, lds_bytes, stream);
+    case 4 * 16 + 2: return launch_t<FMT, XT, MT, 4, 2>(a, threads, grid, lds_bytes, stream);
   }
-  return set_error(TLHIP_ERR_INVALID, "gemv: rows per lane group must be 1, 2 or 4 (got %d)", r);
+  return set_error(TLHIP_ERR_INVALID, "gemv: (rows per lane group, chunks in flight) = (%d,%d) is not built", r, u);
 }
 
 template <int FMT, typename XT>
-int launch_m(int mt, int r, const GemvArgs& a, int threads, int grid, size_t lds_bytes, hipStream_t stream) {
+int launch_m(int mt, int r, int u, const GemvArgs& a, int threads, int grid, size_t lds_bytes,
+             hipStream_t stream) {
   switch (mt) {
-    case 1: return launch_r<FMT, XT, 1>(r, a, threads, grid, lds_bytes, stream);
-    case 2: return launch_r<FMT, XT, 2>(r, a, threads, grid, lds_bytes, stream);
-    case 4: return launch_r<FMT, XT, 4>(r, a, threads, grid, lds_bytes, stream);
+    case 1: return launch_r<FMT, XT, 1>(r, u, a, threads, grid, lds_bytes, stream);
+    case 2: return launch_r<FMT, XT, 2>(r, u, a, threads, grid, lds_bytes, stream);
+    case 4: return launch_r<FMT, XT, 4>(r, u, a, threads, grid, lds_bytes, stream);
   }
   return set_error(TLHIP_ERR_INVALID, "gemv: internal M tile %d", mt);
 }
 
 template <int FMT>
-int launch_x(int x_dtype, int mt, int r, const GemvArgs& a, int threads, int grid, size_t lds_bytes,
+int launch_x(int x_dtype, int mt, int r, int u, const GemvArgs& a, int threads, int grid, size_t lds_bytes,
              hipStream_t stream) {
-  if (x_dtype == TLHIP_F16) return launch_m<FMT, _Float16>(mt, r, a, threads, grid, lds_bytes, stream);
-  return launch_m<FMT, float>(mt, r, a, threads, grid, lds_bytes, stream);
+  if (x_dtype == TLHIP_F16) return launch_m<FMT, _Float16>(mt, r, u, a, threads, grid, lds_bytes, stream);
+  return launch_m<FMT, float>(mt, r, u, a, threads, grid, lds_bytes, stream);
 }
 
 int chunk_weights(int format) { return format == TLHIP_FMT_INT4_GROUPED ? 32 : 16; }
@@ -367,10 +437,11 @@ bool gemv_config_applicable(const Problem& p, const tlhip_kernel_config_t& c, co
       "lanes per row must be 16, 32 or 64",
       "rows per lane group must be 1, 2 or 4",
       "waves per workgroup must be 1..8",
-      "K-split waves must divide waves per workgroup",
+      "K-split waves must be 1, 2, 4 or 8 and divide waves per workgroup",
       "K must be a whole number of 16-byte chunks (K % 32 for int4, K % 16 for int8)",
       "group size must be a multiple of the chunk (32 for int4, 16 for int8)",
       "M above 16",
+      "chunks in flight must be 2, 4 or 8 with rows*chunks <= 8",
   };
   auto fail = [&](int i) {
     if (why) *why = reasons[i];
@@ -380,11 +451,13 @@ bool gemv_config_applicable(const Problem& p, const tlhip_kernel_config_t& c, co
   if (c.p0 != 16 && c.p0 != 32 && c.p0 != 64) return fail(1);
   if (c.p1 != 1 && c.p1 != 2 && c.p1 != 4) return fail(2);
   if (c.p2 < 1 || c.p2 > 8) return fail(3);
-  if (c.p3 < 1 || c.p2 % c.p3 != 0) return fail(4);
+  if (c.p3 < 1 || (c.p3 & (c.p3 - 1)) != 0 || c.p2 % c.p3 != 0) return fail(4);
   const int cw = chunk_weights(p.format);
   if (p.k % cw != 0) return fail(5);
   if (p.format != TLHIP_FMT_INT8_ROW && p.group_size % cw != 0) return fail(6);
   if (p.m > 16) return fail(7);
+  const int u = c.p4 == 0 ? 2 : c.p4;
+  if ((u != 2 && u != 4 && u != 8) || u * c.p1 > 8) return fail(8);
   return true;
 }
 
@@ -398,8 +471,14 @@ int launch_gemv(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t st
   const int xbytes = p.x_dtype == TLHIP_F16 ? 2 : 4;
   const int ybytes = p.y_dtype == TLHIP_F16 ? 2 : 4;
 
-  for (int64_t m0 = 0; m0 < p.m; m0 += 4) {
-    const int mrows = (int)(p.m - m0 < 4 ? p.m - m0 : 4);
+  // activation rows per pass: as many (4, 2 or 1) as fit LDS next to the partials
+  int pass = 4;
+  while (pass > 1 && (size_t)pass * p.k * xbytes + 16 * 1024 > (size_t)kLdsBudget) pass >>= 1;
+  if ((size_t)pass * p.k * xbytes + 16 * 1024 > (size_t)kLdsBudget)
+    return set_error(TLHIP_ERR_INVALID, "gemv: K=%lld is too long for the LDS-resident activation row", (long long)p.k);
+
+  for (int64_t m0 = 0; m0 < p.m; m0 += pass) {
+    const int mrows = (int)(p.m - m0 < pass ? p.m - m0 : pass);
     const int mt = mrows == 1 ? 1 : (mrows == 2 ? 2 : 4);
     GemvArgs a;
     a.packed = (const u32x4*)p.packed;
@@ -413,8 +492,11 @@ int launch_gemv(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t st
     a.cpg_shift = p.format == TLHIP_FMT_INT8_ROW ? 0 : __builtin_ctz((unsigned)(p.group_size / cw));
     a.groups_per_row = p.format == TLHIP_FMT_INT8_ROW ? 0 : (int)(p.k / p.group_size);
     a.lpr = c.p0;
+    a.lpr_shift = __builtin_ctz((unsigned)c.p0);
     a.kw = c.p3;
-    const int r = c.p1, waves = c.p2;
+    a.kw_shift = __builtin_ctz((unsigned)c.p3);
+    const int r = c.p1, waves = c.p2, unroll = c.p4 == 0 ? 2 : c.p4;
+    a.nsteps = (a.nchunks + a.lpr * a.kw * unroll - 1) / (a.lpr * a.kw * unroll);
     a.rows_per_wave = (64 / a.lpr) * r;
     a.rows_per_wg = (waves / a.kw) * a.rows_per_wave;
     a.nblocks = (int)((p.n + a.rows_per_wg - 1) / a.rows_per_wg);
@@ -422,22 +504,10 @@ int launch_gemv(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t st
     a.scale_mul = p.format == TLHIP_FMT_INT8_GROUPED ? (1.0f / 127.0f) : 1.0f;
     a.y_dtype = p.y_dtype;
     a.epi = p.epi;
-    // LDS: staged x (mt rows x slice) + split-K partials
+    // LDS: staged x (mt rows) + split-K partials
     const int chunk_x_bytes = cw * xbytes;
     const size_t partial_bytes = a.kw > 1 ? (size_t)a.kw * a.rows_per_wg * mt * sizeof(float) : 0;
-    int max_slice_chunks = (int)((kLdsBudget - partial_bytes) / ((size_t)mt * chunk_x_bytes));
-    if (max_slice_chunks >= a.nchunks) {
-      a.slice_chunks = a.nchunks;
-      a.nslices = 1;
-    } else {
-      // whole multiples of the chunk stride so every slice starts on the same lane phase
-      const int cstride = a.lpr * a.kw;
-      int sc = max_slice_chunks / cstride * cstride;
-      if (sc <= 0) return set_error(TLHIP_ERR_INVALID, "gemv: K slice does not fit LDS for this configuration");
-      a.slice_chunks = sc;
-      a.nslices = (a.nchunks + sc - 1) / sc;
-    }
-    const size_t lds_bytes = (size_t)mt * chunk_x_bytes * a.slice_chunks + partial_bytes;
+    const size_t lds_bytes = (size_t)mt * chunk_x_bytes * a.nchunks + partial_bytes;
     const int threads = waves * 64;
     const int cus = device_cu_count();
     // resident workgroups per CU: bounded by 2048 lanes and by LDS
@@ -450,13 +520,13 @@ int launch_gemv(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t st
     int rc;
     switch (p.format) {
       case TLHIP_FMT_INT4_GROUPED:
-        rc = launch_x<TLHIP_FMT_INT4_GROUPED>(p.x_dtype, mt, r, a, threads, grid, lds_bytes, stream);
+        rc = launch_x<TLHIP_FMT_INT4_GROUPED>(p.x_dtype, mt, r, unroll, a, threads, grid, lds_bytes, stream);
         break;
       case TLHIP_FMT_INT8_GROUPED:
-        rc = launch_x<TLHIP_FMT_INT8_GROUPED>(p.x_dtype, mt, r, a, threads, grid, lds_bytes, stream);
+        rc = launch_x<TLHIP_FMT_INT8_GROUPED>(p.x_dtype, mt, r, unroll, a, threads, grid, lds_bytes, stream);
         break;
       default:
-        rc = launch_x<TLHIP_FMT_INT8_ROW>(p.x_dtype, mt, r, a, threads, grid, lds_bytes, stream);
+        rc = launch_x<TLHIP_FMT_INT8_ROW>(p.x_dtype, mt, r, unroll, a, threads, grid, lds_bytes, stream);
         break;
     }
     if (rc) return rc;

@@ -1,8 +1,7 @@
 // Skinny GEMM (2 <= M <= 16 activation rows) over packed weights on the matrix
 // cores: the weights are streamed from HBM exactly once whatever M is.
 //
-// One workgroup owns a block of 16 weight rows; its waves split K.  A wave
-// feeds v_mfma_f32_16x16x32_f16 with
+// Weight rows are processed in blocks of 16.  A wave feeds v_mfma_f32_16x16x32_f16 with
 //   A = activations  (lane l supplies x[m = l%16][8 k-values of sub-block l/16])
 //   B = weights      (lane l supplies w[n = l%16][the same 8 k-values])
 //   D = 16 m x 16 n  (lane l holds D[m = 4*(l/16)+r][n = l%16], r = 0..3)
@@ -19,9 +18,12 @@
 // the k-order inside an MFMA is free as long as the activations use the same
 // order, so no exchange is needed.
 //
-// Activations are staged in LDS in MFMA operand order (conflict-free 16-byte
-// reads, consecutive lanes on consecutive units), K-sliced when M*K*2 bytes
-// exceed the LDS budget.  Per-wave partial tiles are combined through LDS.
+// Activations (all of x, M*K f16, which must fit LDS) are staged in MFMA operand
+// order: conflict-free 16-byte reads, consecutive lanes on consecutive units.
+// `kw` waves split K for one row block and combine their partial tiles through
+// LDS; with kw = 1 a wave owns a row block alone and nothing is combined.  The
+// weight loads of all row blocks of a workgroup form one software pipeline, as
+// in the VALU kernel.
 #include "device_utils.h"
 
 namespace tlhip {
@@ -35,13 +37,17 @@ struct MfmaArgs {
   int64_t n;
   int k;
   int m;
+  unsigned m_magic;   // ceil(2^32 / m), for m > 1
   int nchunks;        // 16-byte chunks per weight row
   int cpg_shift;      // log2(chunks per scale group), grouped formats
   int groups_per_row;
   int iters;          // wave iterations over K: 4 chunks each
-  int slice_iters;    // iterations whose activations are resident in LDS at once
-  int nslices;
+  int kw;             // waves that split K for one 16-row block (power of two)
+  int kw_shift;
+  int blocks_per_wg;  // 16-row blocks a workgroup works on at a time = waves / kw
+  int nsteps;         // batches (U iterations each) per row block per wave
   int nblocks;        // 16-row blocks
+  int nwgblocks;      // ceil(nblocks / blocks_per_wg)
   float alpha;
   float scale_mul;
   int y_dtype;
@@ -87,8 +93,8 @@ __device__ __forceinline__ void transpose4(uint32_t& r0, uint32_t& r1, uint32_t&
   r2 = s23[0]; r3 = s23[1];
 }
 
-// LDS unit (16 bytes) index of the activations for MFMA step t (global step
-// index inside the slice), k sub-block g, activation row m.
+// LDS unit (16 bytes) index of the activations for MFMA step t (counted over
+// all of K), k sub-block g, activation row m.
 __device__ __forceinline__ int x_unit(int t, int g, int m, int mrows) { return (t * 4 + g) * mrows + m; }
 
 template <int FMT, int U>
@@ -101,146 +107,188 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(const MfmaArgs a) {
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  const int nwaves = blockDim.x >> 6;
+  const int kw_idx = wave & (a.kw - 1);  // which K part of the row block
+  const int bw_idx = wave >> a.kw_shift; // which row block of the workgroup
   const int nl = lane & 15;   // weight row inside the block / activation row for the A operand
   const int g = lane >> 4;    // k sub-block
   const int mrows = a.m;
   const int ml = nl < mrows ? nl : mrows - 1;  // rows beyond M alias the last row; never stored
-  float* partial = (float*)(lds + (size_t)a.slice_iters * STEPS * 4 * mrows);
+  float* partial = (float*)(lds + (size_t)a.iters * STEPS * 4 * mrows);
+  const int last_iter = a.iters - 1;
 
-  // Stage the activations of one K slice in MFMA operand order.
-  auto stage = [&](int slice) {
-    const int it0 = slice * a.slice_iters;
-    const int nit = min(a.slice_iters, a.iters - it0);
-    const int units = nit * STEPS * 4 * mrows;
-    for (int u = tid; u < units; u += blockDim.x) {
-      const int m = u % mrows;
-      const int tg = u / mrows;
-      const int gg = tg & 3;
-      const int t = tg >> 2;  // step inside the slice
-      int kbase;
-      if (FMT == TLHIP_FMT_INT4_GROUPED) {
-        kbase = (it0 * STEPS + t) * 32 + gg * 8;             // group t, word gg
-      } else {
-        const int it = it0 + (t >> 1), j = t & 1;
-        kbase = it * 64 + gg * 16 + j * 8;                   // chunk gg of the iteration, half j
+  // Raw loaded values only (no conversion at issue time, see gemv.hip).
+  struct Batch {
+    u32x4 w[U];
+    uint16_t s[U][STEPS];
+  };
+
+  auto load_batch = [&](Batch& b, int wgb, int step) {
+    const int rb = min(wgb * a.blocks_per_wg + bw_idx, a.nblocks - 1);
+    const int64_t row = min((int64_t)rb * 16 + nl, a.n - 1);
+    const u32x4* wrow = a.packed + row * a.nchunks;
+    const uint16_t* srow = (const uint16_t*)a.scales + row * a.groups_per_row;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int it = min(kw_idx + (step * U + u) * a.kw, last_iter);
+      b.w[u] = __builtin_nontemporal_load(wrow + it * 4 + g);
+      if (GROUPED) {
+#pragma unroll
+        for (int s = 0; s < STEPS; ++s) {
+          // int4: step s is chunk 4*it+s; int8: both steps lie in chunks 4*it .. 4*it+3
+          const int chunk = FMT == TLHIP_FMT_INT4_GROUPED ? it * 4 + s : it * 4;
+          b.s[u][s] = srow[chunk >> a.cpg_shift];
+        }
       }
-      u32x4 v = *(const u32x4*)(a.x + (size_t)m * a.k + kbase);
-      if (FMT == TLHIP_FMT_INT4_GROUPED) v = permute_x_for_int4(v);
-      lds[u] = v;
     }
   };
 
-  if (a.nslices == 1) {
-    stage(0);
-    __syncthreads();
-  }
+  float4_t acc = {0.f, 0.f, 0.f, 0.f};
 
-  for (int rb = blockIdx.x; rb < a.nblocks; rb += gridDim.x) {
-    const int64_t row = min((int64_t)rb * 16 + nl, a.n - 1);
-    const u32x4* wrow = a.packed + row * a.nchunks;
-    const uint16_t* srow = GROUPED ? (const uint16_t*)a.scales + row * a.groups_per_row : nullptr;
-    float4_t acc = {0.f, 0.f, 0.f, 0.f};
-
-    for (int slice = 0; slice < a.nslices; ++slice) {
-      if (a.nslices > 1) {
-        __syncthreads();
-        stage(slice);
-        __syncthreads();
-      }
-      const int it_begin = slice * a.slice_iters;
-      const int it_end = min(it_begin + a.slice_iters, a.iters);
-      for (int itb = it_begin + wave; itb < it_end; itb += nwaves * U) {
-        u32x4 wv[U];
-        float sv[U][STEPS];
+  auto compute_batch = [&](const Batch& b, int step) {
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-          const int it = itb + u * nwaves;
-          if (it < it_end) {
-            wv[u] = __builtin_nontemporal_load(wrow + it * 4 + g);
-            if (GROUPED) {
+    for (int u = 0; u < U; ++u) {
+      const int it_raw = kw_idx + (step * U + u) * a.kw;
+      const bool valid = it_raw <= last_iter;  // wave-uniform
+      const int it = min(it_raw, last_iter);
+      const int tl = it * STEPS;
+      uint32_t w0 = b.w[u].x, w1 = b.w[u].y, w2 = b.w[u].z, w3 = b.w[u].w;
+      half8_t bw[STEPS];
+      if (FMT == TLHIP_FMT_INT4_GROUPED) {
+        transpose4(w0, w1, w2, w3);  // register s now holds word g of chunk 4*it+s
+        const uint32_t ws[4] = {w0, w1, w2, w3};
 #pragma unroll
-              for (int s = 0; s < STEPS; ++s) {
-                // int4: step s is chunk 4*it+s; int8: both steps lie in chunks 4*it .. 4*it+3
-                const int chunk = FMT == TLHIP_FMT_INT4_GROUPED ? it * 4 + s : it * 4;
-                sv[u][s] = half_bits_to_float(srow[chunk >> a.cpg_shift]);
-              }
-            }
-          }
+        for (int s = 0; s < 4; ++s) {
+          half2_t h[4];
+          unpack_int4_word(ws[s], h);
+          bw[s] = join8(h);
         }
+      } else {
+        const uint32_t ws[4] = {w0, w1, w2, w3};
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-          const int it = itb + u * nwaves;
-          if (it < it_end) {
-            const int tl = (it - it_begin) * STEPS;
-            uint32_t w0 = wv[u].x, w1 = wv[u].y, w2 = wv[u].z, w3 = wv[u].w;
-            half8_t bw[STEPS];
-            if (FMT == TLHIP_FMT_INT4_GROUPED) {
-              transpose4(w0, w1, w2, w3);  // register s now holds word g of chunk 4*it+s
-              const uint32_t ws[4] = {w0, w1, w2, w3};
+        for (int s = 0; s < 2; ++s) {
+          half2_t h[4];
+          unpack_int8_word(ws[2 * s], h);
+          unpack_int8_word(ws[2 * s + 1], h + 2);
+          bw[s] = join8(h);
+        }
+      }
+      float4_t d[STEPS];
 #pragma unroll
-              for (int s = 0; s < 4; ++s) {
-                half2_t h[4];
-                unpack_int4_word(ws[s], h);
-                bw[s] = join8(h);
-              }
-            } else {
-              const uint32_t ws[4] = {w0, w1, w2, w3};
+      for (int s = 0; s < STEPS; ++s) {
+        const u32x4 xa = lds[x_unit(tl + s, g, ml, mrows)];
+        const float4_t zero = {0.f, 0.f, 0.f, 0.f};
+        d[s] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, xa), bw[s], zero, 0, 0, 0);
+      }
 #pragma unroll
-              for (int s = 0; s < 2; ++s) {
-                half2_t h[4];
-                unpack_int8_word(ws[2 * s], h);
-                unpack_int8_word(ws[2 * s + 1], h + 2);
-                bw[s] = join8(h);
-              }
-            }
-            float4_t d[STEPS];
+      for (int s = 0; s < STEPS; ++s) {
+        const float sc = valid ? (GROUPED ? half_bits_to_float(b.s[u][s]) : 1.f) : 0.f;
+        acc[0] = fmaf(sc, d[s][0], acc[0]);
+        acc[1] = fmaf(sc, d[s][1], acc[1]);
+        acc[2] = fmaf(sc, d[s][2], acc[2]);
+        acc[3] = fmaf(sc, d[s][3], acc[3]);
+      }
+    }
+  };
+
+  // Combine the K parts (through LDS when kw > 1), apply the epilogue, store.
+  auto finish = [&](int wgb) {
+    const int rb = wgb * a.blocks_per_wg + bw_idx;
+    if (a.kw > 1) {
+      lds_barrier();  // the previous round's readers are done with `partial`
 #pragma unroll
-            for (int s = 0; s < STEPS; ++s) {
-              const u32x4 xa = lds[x_unit(tl + s, g, ml, mrows)];
-              const float4_t zero = {0.f, 0.f, 0.f, 0.f};
-              d[s] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, xa), bw[s], zero, 0, 0, 0);
-            }
+      for (int r = 0; r < 4; ++r) partial[(wave * 16 + (4 * g + r)) * 16 + nl] = acc[r];
+      lds_barrier();
+      if (kw_idx == 0) {
 #pragma unroll
-            for (int s = 0; s < STEPS; ++s) {
-              if (GROUPED) {
-                acc[0] = fmaf(sv[u][s], d[s][0], acc[0]);
-                acc[1] = fmaf(sv[u][s], d[s][1], acc[1]);
-                acc[2] = fmaf(sv[u][s], d[s][2], acc[2]);
-                acc[3] = fmaf(sv[u][s], d[s][3], acc[3]);
-              } else {
-                acc[0] += d[s][0]; acc[1] += d[s][1]; acc[2] += d[s][2]; acc[3] += d[s][3];
-              }
-            }
-          }
+        for (int r = 0; r < 4; ++r) {
+          float s = 0.f;
+          for (int w = 0; w < a.kw; ++w) s += partial[((wave + w) * 16 + (4 * g + r)) * 16 + nl];
+          acc[r] = s;
         }
       }
     }
-
-    // combine the waves' partial tiles through LDS: partial[wave][m][n]
-    __syncthreads();
-#pragma unroll
-    for (int r = 0; r < 4; ++r) partial[(wave * 16 + (4 * g + r)) * 16 + nl] = acc[r];
-    __syncthreads();
-    if (tid < 256) {
-      const int m = tid >> 4, nn = tid & 15;
-      const int64_t orow = (int64_t)rb * 16 + nn;
-      if (m < mrows && orow < a.n) {
-        float s = 0.f;
-        for (int w = 0; w < nwaves; ++w) s += partial[(w * 16 + m) * 16 + nn];
-        float rs = a.scale_mul;
+    if (kw_idx == 0 && rb < a.nblocks) {
+      const int64_t orow = (int64_t)rb * 16 + nl;
+      if (orow < a.n) {
+        float rs = a.scale_mul * a.alpha;
         if (!GROUPED) rs *= ((const float*)a.scales)[orow];
-        float v = s * rs * a.alpha;
-        v = apply_epilogue(a.epi, v, orow);
-        store_out(a.y, a.y_dtype, (int64_t)m * a.n + orow, v);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int m = 4 * g + r;
+          if (m < mrows) {
+            const float v = apply_epilogue(a.epi, acc[r] * rs, orow);
+            store_out(a.y, a.y_dtype, (int64_t)m * a.n + orow, v);
+          }
+        }
       }
     }
+    acc = (float4_t){0.f, 0.f, 0.f, 0.f};
+  };
+
+  // Activations first (they return first), then the first weight batch, then
+  // the LDS store of the activations in MFMA operand order.
+  constexpr int XS = 4;
+  const int units_total = a.iters * STEPS * 4 * mrows;
+  auto x_src = [&](int u) {
+    // unit u = (t*4 + gg)*mrows + m; mrows <= 16 is not a power of two in general
+    // u / mrows by multiplication with ceil(2^32 / mrows): exact for u * mrows < 2^32
+    const int tg = mrows == 1 ? u : (int)__umulhi((unsigned)u, a.m_magic);
+    const int m = u - tg * mrows;
+    const int gg = tg & 3;
+    const int t = tg >> 2;
+    int kbase;
+    if (FMT == TLHIP_FMT_INT4_GROUPED) {
+      kbase = t * 32 + gg * 8;                        // group t, word gg
+    } else {
+      kbase = (t >> 1) * 64 + gg * 16 + (t & 1) * 8;  // chunk gg of the iteration, half t&1
+    }
+    return (const u32x4*)(a.x + (size_t)m * a.k + kbase);
+  };
+  int wgb = blockIdx.x, step = 0;
+  Batch cur;
+  if (units_total <= XS * (int)blockDim.x) {
+    u32x4 xr[XS];
+#pragma unroll
+    for (int i = 0; i < XS; ++i) xr[i] = *x_src(min(tid + i * (int)blockDim.x, units_total - 1));
+    load_batch(cur, wgb, 0);
+#pragma unroll
+    for (int i = 0; i < XS; ++i) {
+      const int u = tid + i * (int)blockDim.x;
+      if (u < units_total) {
+        u32x4 v = xr[i];
+        if (FMT == TLHIP_FMT_INT4_GROUPED) v = permute_x_for_int4(v);
+        lds[u] = v;
+      }
+    }
+  } else {
+    load_batch(cur, wgb, 0);
+    for (int u = tid; u < units_total; u += blockDim.x) {
+      u32x4 v = *x_src(u);
+      if (FMT == TLHIP_FMT_INT4_GROUPED) v = permute_x_for_int4(v);
+      lds[u] = v;
+    }
+  }
+  lds_barrier();
+
+  while (wgb < a.nwgblocks) {
+    int nwgb = wgb, nstep = step + 1;
+    if (nstep == a.nsteps) {
+      nstep = 0;
+      nwgb = wgb + gridDim.x;
+    }
+    Batch nxt;
+    if (nwgb < a.nwgblocks) load_batch(nxt, nwgb, nstep);
+    compute_batch(cur, step);
+    if (step == a.nsteps - 1) finish(wgb);
+    cur = nxt;
+    wgb = nwgb;
+    step = nstep;
   }
 }
 
-constexpr size_t kXLdsBudget = 136 * 1024;
-
 }  // namespace
+
+static constexpr size_t kXLdsBudget = 144 * 1024;
 
 bool gemv_mfma_config_applicable(const Problem& p, const tlhip_kernel_config_t& c, const char** why) {
   static const char* reasons[] = {
@@ -250,7 +298,9 @@ bool gemv_mfma_config_applicable(const Problem& p, const tlhip_kernel_config_t& 
       "M must be 1..16",
       "K must be a multiple of 128 (int4) or 64 (int8)",
       "group size must be a multiple of 32 (int4) or 64 (int8)",
-      "unroll must be 1, 2 or 4",
+      "iterations in flight must be 1, 2 or 4",
+      "K-split waves must be a power of two that divides the waves per workgroup",
+      "activations (M x K f16) do not fit LDS",
   };
   auto fail = [&](int i) {
     if (why) *why = reasons[i];
@@ -265,6 +315,9 @@ bool gemv_mfma_config_applicable(const Problem& p, const tlhip_kernel_config_t& 
   if (p.format == TLHIP_FMT_INT4_GROUPED && p.group_size % 32 != 0) return fail(5);
   if (p.format == TLHIP_FMT_INT8_GROUPED && p.group_size % 64 != 0) return fail(5);
   if (c.p1 != 1 && c.p1 != 2 && c.p1 != 4) return fail(6);
+  const int kw = c.p2 == 0 ? c.p0 : c.p2;
+  if (kw < 1 || (kw & (kw - 1)) != 0 || c.p0 % kw != 0) return fail(7);
+  if ((size_t)p.m * p.k * 2 + (size_t)c.p0 * 1024 > kXLdsBudget) return fail(8);
   return true;
 }
 
@@ -291,6 +344,7 @@ int launch_gemv_mfma(const Problem& p, const tlhip_kernel_config_t& c, hipStream
   const bool int4 = p.format == TLHIP_FMT_INT4_GROUPED;
   const int cw = int4 ? 32 : 16;
   const int steps = int4 ? 4 : 2;
+  const int waves = c.p0, unroll = c.p1;
   MfmaArgs a;
   a.packed = (const u32x4*)p.packed;
   a.scales = p.scales;
@@ -299,41 +353,35 @@ int launch_gemv_mfma(const Problem& p, const tlhip_kernel_config_t& c, hipStream
   a.n = p.n;
   a.k = (int)p.k;
   a.m = (int)p.m;
+  a.m_magic = p.m > 1 ? (unsigned)((((uint64_t)1 << 32) + p.m - 1) / p.m) : 0u;
   a.nchunks = (int)(p.k / cw);
   a.cpg_shift = p.format == TLHIP_FMT_INT8_ROW ? 0 : __builtin_ctz((unsigned)(p.group_size / cw));
   a.groups_per_row = p.format == TLHIP_FMT_INT8_ROW ? 0 : (int)(p.k / p.group_size);
   a.iters = a.nchunks / 4;
+  a.kw = c.p2 == 0 ? waves : c.p2;
+  a.kw_shift = __builtin_ctz((unsigned)a.kw);
+  a.blocks_per_wg = waves / a.kw;
+  a.nsteps = (a.iters + a.kw * unroll - 1) / (a.kw * unroll);
   a.nblocks = (int)((p.n + 15) / 16);
+  a.nwgblocks = (a.nblocks + a.blocks_per_wg - 1) / a.blocks_per_wg;
   a.alpha = p.alpha;
   a.scale_mul = p.format == TLHIP_FMT_INT8_GROUPED ? (1.0f / 127.0f) : 1.0f;
   a.y_dtype = p.y_dtype;
   a.epi = p.epi;
-  const int waves = c.p0;
   const size_t partial_bytes = (size_t)waves * 256 * sizeof(float);
-  const size_t iter_x_bytes = (size_t)steps * 4 * a.m * 16;  // LDS bytes of activations per iteration
-  int max_iters = (int)((kXLdsBudget - partial_bytes) / iter_x_bytes);
-  if (max_iters >= a.iters) {
-    a.slice_iters = a.iters;
-    a.nslices = 1;
-  } else {
-    int si = max_iters / waves * waves;  // every slice starts on the same wave phase
-    if (si <= 0) return set_error(TLHIP_ERR_INVALID, "gemv_mfma: K slice does not fit LDS");
-    a.slice_iters = si;
-    a.nslices = (a.iters + si - 1) / si;
-  }
-  const size_t lds_bytes = iter_x_bytes * a.slice_iters + partial_bytes;
+  const size_t lds_bytes = (size_t)a.iters * steps * 4 * a.m * 16 + partial_bytes;
   const int threads = waves * 64;
   const int cus = device_cu_count();
   int per_cu = 2048 / threads;
   const int by_lds = (int)((160 * 1024) / lds_bytes);
   if (by_lds < per_cu) per_cu = by_lds < 1 ? 1 : by_lds;
-  int grid = a.nblocks < cus * per_cu ? a.nblocks : cus * per_cu;
+  int grid = a.nwgblocks < cus * per_cu ? a.nwgblocks : cus * per_cu;
   if (grid < 1) grid = 1;
   int rc;
   switch (p.format) {
-    case TLHIP_FMT_INT4_GROUPED: rc = launch_mfma_u<TLHIP_FMT_INT4_GROUPED>(c.p1, a, grid, threads, lds_bytes, stream); break;
-    case TLHIP_FMT_INT8_GROUPED: rc = launch_mfma_u<TLHIP_FMT_INT8_GROUPED>(c.p1, a, grid, threads, lds_bytes, stream); break;
-    default: rc = launch_mfma_u<TLHIP_FMT_INT8_ROW>(c.p1, a, grid, threads, lds_bytes, stream); break;
+    case TLHIP_FMT_INT4_GROUPED: rc = launch_mfma_u<TLHIP_FMT_INT4_GROUPED>(unroll, a, grid, threads, lds_bytes, stream); break;
+    case TLHIP_FMT_INT8_GROUPED: rc = launch_mfma_u<TLHIP_FMT_INT8_GROUPED>(unroll, a, grid, threads, lds_bytes, stream); break;
+    default: rc = launch_mfma_u<TLHIP_FMT_INT8_ROW>(unroll, a, grid, threads, lds_bytes, stream); break;
   }
   if (rc) return rc;
   TLHIP_CHECK_HIP(hipGetLastError());
