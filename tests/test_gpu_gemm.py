@@ -1,0 +1,133 @@
+"""GPU parity: prefill GEMM with dequant fused into the LDS stage and a fused
+epilogue, vs the oracle (bit-exact dequant -> CPU-backend matmul -> add ->
+activation, each storing f32).
+
+Tolerance: rel-L2 <= 1e-3.  The kernel rounds each dequantised weight once to
+f16 before the MFMA (relative 2^-12 rms per weight), which by itself gives
+about 2-3e-4; the f16 output store adds about 2e-4."""
+import numpy as np
+import pytest
+
+import torchlette_amd as T
+from oracle import quant_oracle as O
+from torchlette_amd import _lib as L
+from helpers import f16_round, fmt_name, make_weight, make_x, rel_l2
+
+pytestmark = pytest.mark.gpu
+REL_L2_TOL = 1e-3
+TILES = [(256, 256), (128, 256), (256, 128), (128, 128), (64, 128)]
+
+
+@pytest.fixture(scope="module")
+def be():
+    return T.getBackend()
+
+
+def tiled(bm, bn):
+    return L.KernelConfig.of(L.VARIANT_TILED, bm, bn, 64, 2, 2)
+
+
+def run(be, fmt, packed, scales, n, k, g, x, element, bias=None, act=None, fused=True, config=None):
+    w = be.createQuantizedWeight(packed, scales, n, k, T.resolveWeightFormat(fmt_name(fmt, g), element))
+    xt = be.ops.tensorFromArray(x, list(x.shape), "f16")
+    bt = be.ops.tensorFromArray(bias, [n], "f16" if bias.dtype == np.float16 else "f32") if bias is not None else None
+    y = be.linear(xt, w, bt, act, fused=fused, config=config)
+    out = y.numpy()
+    y.destroy()
+    xt.destroy()
+    return out
+
+
+@pytest.mark.parametrize("bm,bn", TILES)
+@pytest.mark.parametrize("fmt,g", [("int4-grouped", 32), ("int4-grouped", 128), ("int8-grouped", 64), ("int8-row", 0)])
+def test_every_tile_config_ragged_shapes(be, fmt, g, bm, bn):
+    rng = np.random.default_rng(bm * 7 + bn + g)
+    m, n, k = 300, 333, 256          # neither M nor N a multiple of any tile
+    packed, scales, deq = make_weight(fmt, n, k, g, rng)
+    x = make_x(m, k, "f16", rng, std=0.5)
+    before = T.getQuantGemmDispatchCount()
+    got = run(be, fmt, packed, scales, n, k, g, x, "f32", config=tiled(bm, bn))
+    assert T.getQuantGemmDispatchCount() == before + 1
+    want = O.linear(x.astype(np.float32), deq, threads=8)
+    assert got.shape == (m, n) and got.dtype == np.float32
+    assert rel_l2(got, want) <= REL_L2_TOL, rel_l2(got, want)
+
+
+@pytest.mark.parametrize("m,n,k", [(17, 128, 64), (64, 64, 128), (100, 512, 1024), (1000, 256, 2048), (33, 1000, 4096)])
+def test_default_route_for_m_above_16_is_the_gemm(be, m, n, k):
+    rng = np.random.default_rng(m + n + k)
+    packed, scales, deq = make_weight("int4-grouped", n, k, 32, rng)
+    x = make_x(m, k, "f16", rng, std=0.5)
+    g0, v0 = T.getQuantGemmDispatchCount(), T.getQuantGemvDispatchCount()
+    got = run(be, "int4-grouped", packed, scales, n, k, 32, x, "f16", fused=False)
+    assert T.getQuantGemmDispatchCount() == g0 + 1 and T.getQuantGemvDispatchCount() == v0
+    want = O.linear(x.astype(np.float32), deq, threads=8)
+    assert got.dtype == np.float16
+    assert rel_l2(got, want) <= REL_L2_TOL, rel_l2(got, want)
+
+
+@pytest.mark.parametrize("act", ["silu", "gelu", "relu", None])
+def test_fused_epilogue_matches_unfused_ops_and_oracle(be, act):
+    """Config-4 epilogue (f16 bias then silu / gelu-tanh, f16 out) at a reduced size."""
+    rng = np.random.default_rng(21)
+    m, n, k = 256, 768, 1024
+    packed, scales, deq = make_weight("int4-grouped", n, k, 32, rng)
+    x = make_x(m, k, "f16", rng, std=0.5)
+    bias = f16_round(rng.standard_normal(n) * 0.1)
+    want = O.linear(x.astype(np.float32), deq, bias.astype(np.float32), act or "none", threads=8)
+    fused = run(be, "int4-grouped", packed, scales, n, k, 32, x, "f16", bias=bias, act=act, fused=True)
+    unfused = run(be, "int4-grouped", packed, scales, n, k, 32, x, "f16", bias=bias, act=act, fused=False)
+    assert rel_l2(fused, want) <= REL_L2_TOL, rel_l2(fused, want)
+    assert rel_l2(unfused, want) <= REL_L2_TOL
+    # the fused path skips two f16 round trips; the two agree to f16 rounding
+    assert rel_l2(fused, unfused) <= 6e-4
+
+
+def test_gemm_against_gemv_on_the_same_rows(be):
+    """The GEMM's first 16 rows vs the (exact-integer) GEMV kernels on the same rows."""
+    rng = np.random.default_rng(31)
+    m, n, k = 128, 1024, 2048
+    packed, scales, _ = make_weight("int4-grouped", n, k, 32, rng)
+    x = make_x(m, k, "f16", rng, std=0.5)
+    full = run(be, "int4-grouped", packed, scales, n, k, 32, x, "f32")
+    part = run(be, "int4-grouped", packed, scales, n, k, 32, x[:16].copy(), "f32")
+    assert rel_l2(full[:16], part) <= 5e-4
+
+
+@pytest.mark.parametrize("m", [512, 2048])
+def test_config4_full_size(be, m):
+    """M x 4096 x 12288 int4-g32, bias + silu, f16 out: a row sample against the
+    sequential-k oracle, the whole output against numpy float64 (same sums in a
+    different order), and linearity in the activations."""
+    rng = np.random.default_rng(m)
+    n, k = 12288, 4096
+    packed, scales, deq = make_weight("int4-grouped", n, k, 32, rng)
+    x = make_x(m, k, "f16", rng, std=0.5)
+    bias = f16_round(rng.standard_normal(n) * 0.1)
+    got = run(be, "int4-grouped", packed, scales, n, k, 32, x, "f16", bias=bias, act="silu")
+    rows = rng.choice(m, 32, replace=False)
+    want_rows = O.linear(x[rows].astype(np.float32), deq, bias.astype(np.float32), "silu", threads=8)
+    assert rel_l2(got[rows], want_rows) <= REL_L2_TOL, rel_l2(got[rows], want_rows)
+    pre = O.np_matmul_nt(x.astype(np.float32), deq)
+    want = O.np_unary("silu", (pre.astype(np.float64) + bias.astype(np.float64)).astype(np.float32))
+    assert rel_l2(got, want) <= REL_L2_TOL, rel_l2(got, want)
+    # no epilogue, f32 out: y(2*x) == 2*y(x) exactly (scaling by 2 is exact in f16 and f32)
+    y1 = run(be, "int4-grouped", packed, scales, n, k, 32, x, "f32")
+    y2 = run(be, "int4-grouped", packed, scales, n, k, 32, f16_round(2 * x.astype(np.float32)), "f32")
+    assert np.array_equal(y2, 2 * y1)
+    assert rel_l2(y1, pre) <= 5e-4
+
+
+def test_gemm_rejects_f32_activations_and_falls_back_to_gemv_passes(be):
+    rng = np.random.default_rng(41)
+    m, n, k = 40, 256, 512
+    packed, scales, deq = make_weight("int8-grouped", n, k, 64, rng)
+    x = make_x(m, k, "f32", rng)
+    w = be.createQuantizedWeight(packed, scales, n, k, T.resolveWeightFormat("int8-64", "f32"))
+    xt = be.ops.tensorFromArray(x, [m, k], "f32")
+    with pytest.raises(L.TlhipError, match="activations must be f16"):
+        be.linear(xt, w, config=tiled(128, 128))
+    v0 = T.getQuantGemvDispatchCount()
+    y = be.linear(xt, w).numpy()
+    assert T.getQuantGemvDispatchCount() == v0 + 3      # 16 + 16 + 8 rows
+    assert rel_l2(y, O.linear(x, deq)) <= 2e-6

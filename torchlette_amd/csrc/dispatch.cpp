@@ -102,22 +102,31 @@ tlhip_kernel_config_t default_config(const Problem& p) {
   const int cw = p.format == TLHIP_FMT_INT4_GROUPED ? 32 : 16;
   const int64_t nchunks = p.k / cw;
   if (p.m > 16 && p.x_dtype == TLHIP_F16) {
-    tlhip_kernel_config_t c = tiled_cfg(128, 128, 64, 2, 2);
-    if (gemm_config_applicable(p, c, nullptr)) return c;
+    // largest tile that still gives every CU a workgroup
+    const int cus = device_cu_count() > 0 ? device_cu_count() : 256;
+    static const int tiles[][2] = {{256, 256}, {256, 128}, {128, 128}, {64, 128}};
+    for (auto& t : tiles) {
+      const int64_t wgs = ((p.m + t[0] - 1) / t[0]) * ((p.n + t[1] - 1) / t[1]);
+      tlhip_kernel_config_t c = tiled_cfg(t[0], t[1], 64, 2, 2);
+      if ((wgs >= cus || t[0] == 64) && gemm_config_applicable(p, c, nullptr)) return c;
+    }
   }
-  // three or more activation rows: the matrix-core kernel streams the weights once
-  if (p.m >= 3 && p.m <= 16) {
+  // five or more activation rows: the matrix-core kernel streams the weights once
+  // (below that the VALU kernel with its rows held in registers measures faster)
+  if (p.m >= 5 && p.m <= 16) {
     tlhip_kernel_config_t c = mfma_cfg(8, 2, p.n >= 32768 ? 1 : 8);
     if (gemv_mfma_config_applicable(p, c, nullptr)) return c;
   }
-  // lanes per row: keep every lane busy for short rows
+  // lanes per row: every lane busy for short rows; all chunks of a row in flight at once
   int lpr = 64;
   if (nchunks % 64 != 0) lpr = (nchunks % 32 == 0) ? 32 : 16;
   if (nchunks < 64) lpr = nchunks >= 32 ? 32 : 16;
-  const int r = p.m >= 4 ? 2 : 1;
-  // enough row blocks to give every CU several waves; big N walks with a stride
-  int waves = 4;
-  return gemv_cfg(lpr, r, waves, 1, 2);
+  if (p.n >= 32768) lpr = 16;  // long weight matrices: more rows per wave, walked with a stride
+  const int per_lane = (int)((nchunks + lpr - 1) / lpr);
+  const int unroll = per_lane >= 8 ? 8 : (per_lane >= 4 ? 4 : 2);
+  int r = 1;
+  if (p.n >= 32768) r = unroll <= 2 ? 4 : (unroll <= 4 ? 2 : 1);
+  return gemv_cfg(lpr, r, p.n >= 32768 ? 8 : 4, 1, unroll);
 }
 
 std::vector<tlhip_kernel_config_t> candidates(const Problem& p) {
@@ -134,9 +143,9 @@ std::vector<tlhip_kernel_config_t> candidates(const Problem& p) {
             }
   }
   if (p.m <= 16) {
-    for (int waves : {4, 8, 16})
+    for (int waves : {4, 8})
       for (int unroll : {1, 2, 4})
-        for (int kw : {1, 2, 4, 8, 16}) {
+        for (int kw : {1, 2, 4, 8}) {
           if (kw > waves) continue;
           tlhip_kernel_config_t c = mfma_cfg(waves, unroll, kw);
           if (gemv_mfma_config_applicable(p, c, nullptr)) out.push_back(c);
@@ -144,8 +153,8 @@ std::vector<tlhip_kernel_config_t> candidates(const Problem& p) {
   }
   if (p.x_dtype == TLHIP_F16 && p.m >= 16) {
     static const int tiles[][5] = {
-        {128, 128, 64, 2, 2}, {256, 128, 64, 2, 2}, {128, 256, 64, 2, 2}, {256, 256, 64, 2, 2},
-        {64, 128, 64, 2, 2},  {128, 64, 64, 2, 2},  {64, 64, 64, 2, 2},   {256, 128, 32, 2, 2},
+        {128, 128, 64, 2, 2}, {256, 128, 64, 2, 2}, {128, 256, 64, 2, 2},
+        {256, 256, 64, 2, 2}, {64, 128, 64, 2, 2},
     };
     for (auto& t : tiles) {
       tlhip_kernel_config_t c = tiled_cfg(t[0], t[1], t[2], t[3], t[4]);
@@ -336,7 +345,7 @@ int tlhip_gemm_prefill(const tlhip_qweight_t* w, const void* x, int x_dtype, int
   if (x_dtype != TLHIP_F16) return set_error(TLHIP_ERR_INVALID, "gemm_prefill: activations must be f16");
   tlhip_kernel_config_t c = select_config(p);
   if (c.variant != VARIANT_TILED) {
-    c = tiled_cfg(128, 128, 64, 2, 2);
+    c = tiled_cfg(p.m >= 128 ? 128 : 64, 128, 64, 2, 2);
     const char* why = nullptr;
     if (!gemm_config_applicable(p, c, &why))
       return set_error(TLHIP_ERR_INVALID, "gemm_prefill: shape not supported: %s", why ? why : "?");

@@ -1,11 +1,331 @@
-// placeholder until the MFMA prefill kernel lands
+// Prefill GEMM over packed weights: Y[M,N] = epilogue(alpha * X[M,K] * W[N,K]^T)
+// with the dequantisation fused into the LDS stage.  Stands in for the
+// reference's M > 1 route — an explicit dequant to an f32 [N,K] buffer followed
+// by the stock tiled matmul (src/backend/webgpu/ops/matmul-ops.ts:163-181;
+// src/schedule/matmul-skeleton.ts:738-966) — without ever materialising the
+// dequantised weight in HBM.
+//
+// MFMA-bound (f16 inputs, f32 accumulate).  One workgroup of 4 waves (2 x 2)
+// computes a BM x BN tile of Y with v_mfma_f32_32x32x16_f16; a wave owns a
+// (BM/2) x (BN/2) sub-tile, i.e. (BM/64) x (BN/64) MFMA tiles of 16
+// accumulators each.  Per K step of 64:
+//   * global -> registers: the X tile (f16, 16 bytes per lane per load) and the
+//     packed W tile (16 bytes = 32 int4 or 16 int8 weights, plus the group
+//     scale), for the NEXT step, issued before this step's MFMAs;
+//   * registers -> LDS: the weights are unpacked to exact integers in f16 and
+//     multiplied by their scale (packed f16 multiply, one rounding to f16 per
+//     weight), then written k-contiguous; X is written as is (for int4, with
+//     the same within-8 k order the unpack produces);
+//   * LDS -> MFMA operands: rows are padded to 144 bytes so that the 32 lanes of
+//     an operand read hit 16 different 16-byte bank groups.
+// LDS is double buffered: one barrier per K step.
+// Epilogue: acc*alpha -> ops in order (bias indexed by n, unary) -> cast, the
+// order of applyBlockEpilogue (matmul-skeleton.ts:916-966).
 #include "device_utils.h"
+
 namespace tlhip {
-bool gemm_config_applicable(const Problem&, const tlhip_kernel_config_t&, const char** why) {
-  if (why) *why = "prefill GEMM not built";
-  return false;
+namespace {
+
+constexpr int BK = 64;                 // k per step
+constexpr int ROW_BYTES = BK * 2 + 16; // padded LDS row: 144 bytes = 9 units
+constexpr int ROW_UNITS = ROW_BYTES / 16;
+
+struct GemmArgs {
+  const uint8_t* packed;  // bytes; row stride row_bytes
+  const void* scales;
+  const _Float16* x;
+  void* y;
+  int m, n, k;
+  int w_row_bytes;        // K/2 (int4) or K (int8)
+  int cpg_shift;          // log2(16-byte chunks per scale group)
+  int groups_per_row;
+  int ksteps;
+  int tiles_m, tiles_n;
+  float alpha;
+  float scale_mul;
+  int y_dtype;
+  DevEpilogue epi;
+};
+
+// Unpack one 16-byte chunk to f16 values already multiplied by the scale.
+// int4: 32 weights -> 4 units (64 bytes) in the (0,4,1,5,2,6,3,7) order per word.
+// int8: 16 weights -> 2 units (32 bytes), natural order.
+template <int FMT>
+struct WChunk;
+
+template <>
+struct WChunk<TLHIP_FMT_INT4_GROUPED> {
+  static constexpr int WEIGHTS = 32;
+  static constexpr int UNITS = 4;
+  __device__ static __forceinline__ void dequant(const u32x4& w, float scale, u32x4 (&out)[UNITS]) {
+    const _Float16 sh = (_Float16)scale;  // the scale is an f16 value: exact
+    const half2_t s2 = {sh, sh};
+    const uint32_t words[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      half2_t h[4];
+      unpack_int4_word(words[i], h);
+      u32x4 o;
+      o.x = __builtin_bit_cast(uint32_t, h[0] * s2);
+      o.y = __builtin_bit_cast(uint32_t, h[1] * s2);
+      o.z = __builtin_bit_cast(uint32_t, h[2] * s2);
+      o.w = __builtin_bit_cast(uint32_t, h[3] * s2);
+      out[i] = o;
+    }
+  }
+};
+
+template <int FMT>
+struct WChunkInt8 {
+  static constexpr int WEIGHTS = 16;
+  static constexpr int UNITS = 2;
+  // The scale multiplies in f32 here (int8-row scales are f32 and (q/127)*s is
+  // not an f16 product); one rounding to f16 per weight.
+  __device__ static __forceinline__ void dequant(const u32x4& w, float scale, u32x4 (&out)[UNITS]) {
+    const uint32_t words[4] = {w.x, w.y, w.z, w.w};
+    uint32_t packed[8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float f0 = (float)(int8_t)(words[i] & 0xffu) * scale;
+      const float f1 = (float)(int8_t)((words[i] >> 8) & 0xffu) * scale;
+      const float f2 = (float)(int8_t)((words[i] >> 16) & 0xffu) * scale;
+      const float f3 = (float)(int8_t)(words[i] >> 24) * scale;
+      const half2_t a = {(_Float16)f0, (_Float16)f1};
+      const half2_t b = {(_Float16)f2, (_Float16)f3};
+      packed[2 * i] = __builtin_bit_cast(uint32_t, a);
+      packed[2 * i + 1] = __builtin_bit_cast(uint32_t, b);
+    }
+    out[0] = (u32x4){packed[0], packed[1], packed[2], packed[3]};
+    out[1] = (u32x4){packed[4], packed[5], packed[6], packed[7]};
+  }
+};
+template <>
+struct WChunk<TLHIP_FMT_INT8_GROUPED> : WChunkInt8<TLHIP_FMT_INT8_GROUPED> {};
+template <>
+struct WChunk<TLHIP_FMT_INT8_ROW> : WChunkInt8<TLHIP_FMT_INT8_ROW> {};
+
+template <int FMT, int BM, int BN>
+__global__ __launch_bounds__(256) void gemm_prefill_kernel(const GemmArgs a) {
+  using WC = WChunk<FMT>;
+  constexpr bool GROUPED = (FMT != TLHIP_FMT_INT8_ROW);
+  constexpr int TM = BM / 64, TN = BN / 64;        // MFMA tiles per wave
+  constexpr int X_LOADS = BM * 8 / 256;            // 16-byte units of the X tile per thread
+  constexpr int W_CHUNKS_PER_ROW = BK / WC::WEIGHTS;
+  constexpr int W_LOADS = BN * W_CHUNKS_PER_ROW / 256;
+  constexpr int STAGE_UNITS = (BM + BN) * ROW_UNITS;
+  extern __shared__ u32x4 lds[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  // XCD-aware tile order: consecutive workgroup ids are dealt round-robin to the
+  // 8 XCDs, each with its own L2.  When the column blocks divide by 8, XCD x
+  // owns the column blocks congruent to x and walks the row blocks of each in
+  // turn, so a packed W block is fetched into one L2 only.
+  const int tile = blockIdx.x;
+  int tn_idx, tm_idx;
+  if ((a.tiles_n & 7) == 0) {
+    const int xcd = tile & 7, local = tile >> 3;
+    const int q = local / a.tiles_m;
+    tn_idx = q * 8 + xcd;
+    tm_idx = local - q * a.tiles_m;
+  } else {
+    tn_idx = tile / a.tiles_m;
+    tm_idx = tile - tn_idx * a.tiles_m;
+  }
+  const int m0 = tm_idx * BM, n0 = tn_idx * BN;
+
+  // ---- global -> register staging -------------------------------------
+  u32x4 xr[X_LOADS];
+  u32x4 wr[W_LOADS];
+  uint32_t sr[W_LOADS];  // raw scale bits (f16) or f32 bits (int8-row)
+
+  auto load_tiles = [&](int kstep) {
+    const int k0 = kstep * BK;
+#pragma unroll
+    for (int i = 0; i < X_LOADS; ++i) {
+      const int u = tid + i * 256;
+      const int row = min(m0 + (u >> 3), a.m - 1);
+      xr[i] = *(const u32x4*)(a.x + (size_t)row * a.k + k0 + (u & 7) * 8);
+    }
+#pragma unroll
+    for (int i = 0; i < W_LOADS; ++i) {
+      const int u = tid + i * 256;
+      const int r = u / W_CHUNKS_PER_ROW, c = u - r * W_CHUNKS_PER_ROW;
+      const int row = min(n0 + r, a.n - 1);
+      const int chunk = k0 / WC::WEIGHTS + c;
+      wr[i] = *(const u32x4*)(a.packed + (size_t)row * a.w_row_bytes + (size_t)chunk * 16);
+      if (GROUPED) sr[i] = ((const uint16_t*)a.scales)[(size_t)row * a.groups_per_row + (chunk >> a.cpg_shift)];
+      else sr[i] = ((const uint32_t*)a.scales)[row];
+    }
+  };
+
+  auto store_tiles = [&](int buf) {
+    u32x4* xs = lds + buf * STAGE_UNITS;
+    u32x4* ws = xs + BM * ROW_UNITS;
+#pragma unroll
+    for (int i = 0; i < X_LOADS; ++i) {
+      const int u = tid + i * 256;
+      u32x4 v = xr[i];
+      if (FMT == TLHIP_FMT_INT4_GROUPED) v = permute_x_for_int4(v);
+      xs[(u >> 3) * ROW_UNITS + (u & 7)] = v;
+    }
+#pragma unroll
+    for (int i = 0; i < W_LOADS; ++i) {
+      const int u = tid + i * 256;
+      const int r = u / W_CHUNKS_PER_ROW, c = u - r * W_CHUNKS_PER_ROW;
+      const float s = (GROUPED ? half_bits_to_float(sr[i]) : as_float(sr[i])) * a.scale_mul;
+      u32x4 out[WC::UNITS];
+      WC::dequant(wr[i], s, out);
+#pragma unroll
+      for (int j = 0; j < WC::UNITS; ++j) ws[r * ROW_UNITS + c * WC::UNITS + j] = out[j];
+    }
+  };
+
+  float16_t acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  load_tiles(0);
+  store_tiles(0);
+  __syncthreads();
+
+  const int lrow = lane & 31, lk = lane >> 5;
+  for (int ks = 0; ks < a.ksteps; ++ks) {
+    const int buf = ks & 1;
+    const bool more = ks + 1 < a.ksteps;
+    if (more) load_tiles(ks + 1);
+    const u32x4* xs = lds + buf * STAGE_UNITS;
+    const u32x4* ws = xs + BM * ROW_UNITS;
+#pragma unroll
+    for (int kk = 0; kk < BK / 16; ++kk) {
+      half8_t af[TM], bf[TN];
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+        af[i] = __builtin_bit_cast(half8_t, xs[(wm * (BM / 2) + i * 32 + lrow) * ROW_UNITS + kk * 2 + lk]);
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        bf[j] = __builtin_bit_cast(half8_t, ws[(wn * (BN / 2) + j * 32 + lrow) * ROW_UNITS + kk * 2 + lk]);
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
+    }
+    if (more) store_tiles(buf ^ 1);
+    __syncthreads();
+  }
+
+  // ---- epilogue -----------------------------------------------------------
+  // 32x32 accumulator layout: lane l holds column l%32 and rows
+  // 8*(r/4) + 4*(l/32) + r%4 for r = 0..15.
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const int64_t col = n0 + wn * (BN / 2) + j * 32 + lrow;
+    if (col < a.n) {
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int row = m0 + wm * (BM / 2) + i * 32 + 8 * (r >> 2) + 4 * lk + (r & 3);
+          if (row < a.m) {
+            const float v = apply_epilogue(a.epi, acc[i][j][r] * a.alpha, col);
+            store_out(a.y, a.y_dtype, (int64_t)row * a.n + col, v);
+          }
+        }
+      }
+    }
+  }
 }
-int launch_gemm(const Problem&, const tlhip_kernel_config_t&, hipStream_t) {
-  return set_error(TLHIP_ERR_INVALID, "prefill GEMM not built");
+
+template <int FMT, int BM, int BN>
+int launch_tile(const GemmArgs& a, hipStream_t stream) {
+  const void* fn = (const void*)gemm_prefill_kernel<FMT, BM, BN>;
+  const size_t lds_bytes = (size_t)2 * (BM + BN) * ROW_BYTES;
+  if (lds_bytes > 64 * 1024)
+    TLHIP_CHECK_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+  GemmArgs b = a;
+  b.tiles_m = (a.m + BM - 1) / BM;
+  b.tiles_n = (a.n + BN - 1) / BN;
+  void* args[] = {(void*)&b};
+  TLHIP_CHECK_HIP(hipLaunchKernel(fn, dim3(b.tiles_m * b.tiles_n), dim3(256), args, lds_bytes, stream));
+  return TLHIP_OK;
 }
+
+template <int FMT>
+int launch_fmt(int bm, int bn, const GemmArgs& a, hipStream_t stream) {
+  if (bm == 256 && bn == 256) return launch_tile<FMT, 256, 256>(a, stream);
+  if (bm == 128 && bn == 256) return launch_tile<FMT, 128, 256>(a, stream);
+  if (bm == 256 && bn == 128) return launch_tile<FMT, 256, 128>(a, stream);
+  if (bm == 128 && bn == 128) return launch_tile<FMT, 128, 128>(a, stream);
+  if (bm == 64 && bn == 128) return launch_tile<FMT, 64, 128>(a, stream);
+  return set_error(TLHIP_ERR_INVALID, "gemm: tile %dx%d is not built", bm, bn);
+}
+
+}  // namespace
+
+bool gemm_config_applicable(const Problem& p, const tlhip_kernel_config_t& c, const char** why) {
+  static const char* reasons[] = {
+      "not the tiled variant",
+      "activations must be f16",
+      "K must be a multiple of 64",
+      "group size must be a multiple of 32 (int4) or 16 (int8)",
+      "tile must be one of 256x256, 128x256, 256x128, 128x128, 64x128 with tile K 64 and 2x2 waves",
+  };
+  auto fail = [&](int i) {
+    if (why) *why = reasons[i];
+    return false;
+  };
+  if (c.variant != VARIANT_TILED) return fail(0);
+  if (p.x_dtype != TLHIP_F16) return fail(1);
+  if (p.k % 64 != 0 || p.k == 0) return fail(2);
+  if (p.format == TLHIP_FMT_INT4_GROUPED && p.group_size % 32 != 0) return fail(3);
+  if (p.format == TLHIP_FMT_INT8_GROUPED && p.group_size % 16 != 0) return fail(3);
+  const int bm = c.p0, bn = c.p1;
+  const bool ok = (bm == 256 && bn == 256) || (bm == 128 && bn == 256) || (bm == 256 && bn == 128) ||
+                  (bm == 128 && bn == 128) || (bm == 64 && bn == 128);
+  if (!ok || c.p2 != 64 || c.p3 != 2 || c.p4 != 2) return fail(4);
+  return true;
+}
+
+int launch_gemm(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t stream) {
+  const char* why = nullptr;
+  if (!gemm_config_applicable(p, c, &why)) return set_error(TLHIP_ERR_INVALID, "gemm: config not applicable: %s", why);
+  if (p.m == 0 || p.n == 0) return TLHIP_OK;
+  const bool int4 = p.format == TLHIP_FMT_INT4_GROUPED;
+  const int cw = int4 ? 32 : 16;
+  GemmArgs a;
+  a.packed = (const uint8_t*)p.packed;
+  a.scales = p.scales;
+  a.x = (const _Float16*)p.x;
+  a.y = p.y;
+  a.m = (int)p.m;
+  a.n = (int)p.n;
+  a.k = (int)p.k;
+  a.w_row_bytes = (int)(int4 ? p.k / 2 : p.k);
+  a.cpg_shift = p.format == TLHIP_FMT_INT8_ROW ? 0 : __builtin_ctz((unsigned)(p.group_size / cw));
+  a.groups_per_row = p.format == TLHIP_FMT_INT8_ROW ? 0 : (int)(p.k / p.group_size);
+  a.ksteps = (int)(p.k / BK);
+  a.tiles_m = a.tiles_n = 0;
+  a.alpha = p.alpha;
+  a.scale_mul = p.format == TLHIP_FMT_INT8_GROUPED ? (1.0f / 127.0f) : 1.0f;
+  a.y_dtype = p.y_dtype;
+  a.epi = p.epi;
+  int rc;
+  switch (p.format) {
+    case TLHIP_FMT_INT4_GROUPED: rc = launch_fmt<TLHIP_FMT_INT4_GROUPED>(c.p0, c.p1, a, stream); break;
+    case TLHIP_FMT_INT8_GROUPED: rc = launch_fmt<TLHIP_FMT_INT8_GROUPED>(c.p0, c.p1, a, stream); break;
+    default: rc = launch_fmt<TLHIP_FMT_INT8_ROW>(c.p0, c.p1, a, stream); break;
+  }
+  if (rc) return rc;
+  TLHIP_CHECK_HIP(hipGetLastError());
+  count_gemm_dispatch();
+  return TLHIP_OK;
+}
+
 }  // namespace tlhip

@@ -197,11 +197,11 @@ __global__ __launch_bounds__(512) void gemv_kernel(const GemvArgs a) {
   struct Batch {
     u32x4 w[U][R];
     uint16_t s[U][R];  // f16 bits of the chunk's group scale
-    float rs[R];       // int8-row: the row's scale, fetched with the first batch of a row block
+    float rs[R];       // int8-row: the row's scale
   };
 
   // Issue the loads of one batch: chunks cb + u*cstride (u < U) of R rows.
-  auto load_batch = [&](Batch& b, int rb, int cb, bool first) {
+  auto load_batch = [&](Batch& b, int rb, int cb) {
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       // tail rows recompute the last row; their store is masked
@@ -215,7 +215,7 @@ __global__ __launch_bounds__(512) void gemv_kernel(const GemvArgs a) {
         b.w[u][r] = __builtin_nontemporal_load(wrow + cc);
         if (GROUPED) b.s[u][r] = srow[cc >> a.cpg_shift];
       }
-      if (!GROUPED && first) b.rs[r] = ((const float*)a.scales)[row];
+      if (!GROUPED) b.rs[r] = ((const float*)a.scales)[row];  // every batch: no load under a branch
     }
   };
 
@@ -344,7 +344,7 @@ __global__ __launch_bounds__(512) void gemv_kernel(const GemvArgs a) {
       const int idx = min(tid + i * (int)blockDim.x, units_total - 1);
       xr[i] = *x_src(idx);
     }
-    load_batch(cur, rb, cfirst, true);
+    load_batch(cur, rb, cfirst);
 #pragma unroll
     for (int i = 0; i < XS; ++i) {
       const int idx = tid + i * (int)blockDim.x;
@@ -355,31 +355,68 @@ __global__ __launch_bounds__(512) void gemv_kernel(const GemvArgs a) {
       }
     }
   } else {
-    for (int idx = tid; idx < units_total; idx += blockDim.x) {
-      u32x4 v = *x_src(idx);
-      if (FMT == TLHIP_FMT_INT4_GROUPED && sizeof(XT) == 2) v = permute_x_for_int4(v);
-      *x_dst(idx) = v;
+    load_batch(cur, rb, cfirst);
+    // groups of 8 units per thread: 8 loads in flight, then 8 LDS stores
+    for (int base = 0; base < units_total; base += 8 * (int)blockDim.x) {
+      u32x4 xr[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) xr[i] = *x_src(min(base + tid + i * (int)blockDim.x, units_total - 1));
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const int idx = base + tid + i * (int)blockDim.x;
+        if (idx < units_total) {
+          u32x4 v = xr[i];
+          if (FMT == TLHIP_FMT_INT4_GROUPED && sizeof(XT) == 2) v = permute_x_for_int4(v);
+          *x_dst(idx) = v;
+        }
+      }
     }
-    load_batch(cur, rb, cfirst, true);
   }
   lds_barrier();
-  while (rb < a.nblocks) {
-    int nrb = rb, nstep = step + 1;
-    if (nstep == nsteps) {
-      nstep = 0;
-      nrb = rb + gridDim.x;
+
+  // Batches of this lane, in order: j -> (row block round j / nsteps, step j % nsteps).
+  // Two register sets ping-pong with no copies between them, and every load inside
+  // the steady-state loop is unconditional: a load under a branch makes the wait
+  // counters at the join assume it was NOT issued, and the consumer of the other
+  // set would then wait for the load just issued.
+  const int rounds = (a.nblocks - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;
+  const int total = rounds * nsteps;
+  auto advance = [&](int& r, int& st) {
+    if (++st == nsteps) {
+      st = 0;
+      r += gridDim.x;
     }
-    Batch nxt;
-    if (nrb < a.nblocks) load_batch(nxt, nrb, cfirst + nstep * step_chunks, nstep == 0);
-    if (!GROUPED && step == 0) {
+  };
+  auto consume = [&](const Batch& b, int r, int st) {
+    if (!GROUPED) {
 #pragma unroll
-      for (int r = 0; r < R; ++r) row_scale[r] = cur.rs[r];
+      for (int i = 0; i < R; ++i) row_scale[i] = b.rs[i];
     }
-    compute_batch(cur, cfirst + step * step_chunks);
-    if (step == nsteps - 1) finish(rb);
-    cur = nxt;
-    rb = nrb;
-    step = nstep;
+    compute_batch(b, cfirst + st * step_chunks);
+    if (st == nsteps - 1) finish(r);
+  };
+  Batch other;
+  int j = 0;
+  while (total - j >= 3) {
+    int rb1 = rb, step1 = step;
+    advance(rb1, step1);
+    load_batch(other, rb1, cfirst + step1 * step_chunks);
+    consume(cur, rb, step);
+    rb = rb1;
+    step = step1;
+    advance(rb, step);
+    load_batch(cur, rb, cfirst + step * step_chunks);
+    consume(other, rb1, step1);
+    j += 2;
+  }
+  if (total - j == 2) {
+    int rb1 = rb, step1 = step;
+    advance(rb1, step1);
+    load_batch(other, rb1, cfirst + step1 * step_chunks);
+    consume(cur, rb, step);
+    consume(other, rb1, step1);
+  } else if (total - j == 1) {
+    consume(cur, rb, step);
   }
 }
 

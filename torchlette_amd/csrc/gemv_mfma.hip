@@ -18,8 +18,8 @@
 // the k-order inside an MFMA is free as long as the activations use the same
 // order, so no exchange is needed.
 //
-// Activations (all of x, M*K f16, which must fit LDS) are staged in MFMA operand
-// order: conflict-free 16-byte reads, consecutive lanes on consecutive units.
+// Activations (all of x, M*K f16, which must fit LDS) are staged row by row with
+// a padded row stride, so the MFMA operand reads are free of bank conflicts.
 // `kw` waves split K for one row block and combine their partial tiles through
 // LDS; with kw = 1 a wave owns a row block alone and nothing is combined.  The
 // weight loads of all row blocks of a workgroup form one software pipeline, as
@@ -37,7 +37,6 @@ struct MfmaArgs {
   int64_t n;
   int k;
   int m;
-  unsigned m_magic;   // ceil(2^32 / m), for m > 1
   int nchunks;        // 16-byte chunks per weight row
   int cpg_shift;      // log2(chunks per scale group), grouped formats
   int groups_per_row;
@@ -93,12 +92,21 @@ __device__ __forceinline__ void transpose4(uint32_t& r0, uint32_t& r1, uint32_t&
   r2 = s23[0]; r3 = s23[1];
 }
 
-// LDS unit (16 bytes) index of the activations for MFMA step t (counted over
-// all of K), k sub-block g, activation row m.
-__device__ __forceinline__ int x_unit(int t, int g, int m, int mrows) { return (t * 4 + g) * mrows + m; }
+// Activations live in LDS row by row, as in global memory, 16-byte units, each
+// row padded by one unit: the 16 lanes of an MFMA operand read (16 different
+// rows, same k) then fall in 16 different bank groups, and staging is a
+// straight coalesced copy.  The unit of row m that holds the 8 k-values of MFMA
+// step t (counted over all of K), k sub-block g:
+//   int4: k = 32*t + 8*g             -> unit 4*t + g
+//   int8: k = 64*(t/2) + 16*g + 8*(t%2) -> unit 8*(t/2) + 2*g + (t%2)
+template <int FMT>
+__device__ __forceinline__ int x_unit(int t, int g, int m, int row_units) {
+  const int ku = FMT == TLHIP_FMT_INT4_GROUPED ? 4 * t + g : 8 * (t >> 1) + 2 * g + (t & 1);
+  return m * row_units + ku;
+}
 
 template <int FMT, int U>
-__global__ __launch_bounds__(1024) void gemv_mfma_kernel(const MfmaArgs a) {
+__global__ __launch_bounds__(512) void gemv_mfma_kernel(const MfmaArgs a) {
   using Tr = MfmaTraits<FMT>;
   constexpr int STEPS = Tr::STEPS;
   constexpr bool GROUPED = (FMT != TLHIP_FMT_INT8_ROW);
@@ -113,7 +121,9 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(const MfmaArgs a) {
   const int g = lane >> 4;    // k sub-block
   const int mrows = a.m;
   const int ml = nl < mrows ? nl : mrows - 1;  // rows beyond M alias the last row; never stored
-  float* partial = (float*)(lds + (size_t)a.iters * STEPS * 4 * mrows);
+  const int k_units = a.k >> 3;        // 16-byte units per activation row
+  const int row_units = k_units + 1;   // padded LDS row stride
+  float* partial = (float*)(lds + (size_t)row_units * mrows);
   const int last_iter = a.iters - 1;
 
   // Raw loaded values only (no conversion at issue time, see gemv.hip).
@@ -175,7 +185,7 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(const MfmaArgs a) {
       float4_t d[STEPS];
 #pragma unroll
       for (int s = 0; s < STEPS; ++s) {
-        const u32x4 xa = lds[x_unit(tl + s, g, ml, mrows)];
+        const u32x4 xa = lds[x_unit<FMT>(tl + s, g, ml, row_units)];
         const float4_t zero = {0.f, 0.f, 0.f, 0.f};
         d[s] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, xa), bw[s], zero, 0, 0, 0);
       }
@@ -226,63 +236,88 @@ __global__ __launch_bounds__(1024) void gemv_mfma_kernel(const MfmaArgs a) {
   };
 
   // Activations first (they return first), then the first weight batch, then
-  // the LDS store of the activations in MFMA operand order.
-  constexpr int XS = 4;
-  const int units_total = a.iters * STEPS * 4 * mrows;
-  auto x_src = [&](int u) {
-    // unit u = (t*4 + gg)*mrows + m; mrows <= 16 is not a power of two in general
-    // u / mrows by multiplication with ceil(2^32 / mrows): exact for u * mrows < 2^32
-    const int tg = mrows == 1 ? u : (int)__umulhi((unsigned)u, a.m_magic);
-    const int m = u - tg * mrows;
-    const int gg = tg & 3;
-    const int t = tg >> 2;
-    int kbase;
-    if (FMT == TLHIP_FMT_INT4_GROUPED) {
-      kbase = t * 32 + gg * 8;                        // group t, word gg
-    } else {
-      kbase = (t >> 1) * 64 + gg * 16 + (t & 1) * 8;  // chunk gg of the iteration, half t&1
-    }
-    return (const u32x4*)(a.x + (size_t)m * a.k + kbase);
-  };
+  // the LDS store.  Row by row, consecutive threads on consecutive 16-byte units.
+  const u32x4* xg = (const u32x4*)a.x;
   int wgb = blockIdx.x, step = 0;
   Batch cur;
-  if (units_total <= XS * (int)blockDim.x) {
-    u32x4 xr[XS];
+  if (k_units <= (int)blockDim.x && mrows <= 4) {
+    u32x4 xr[4];
+    const int ku = min(tid, k_units - 1);
 #pragma unroll
-    for (int i = 0; i < XS; ++i) xr[i] = *x_src(min(tid + i * (int)blockDim.x, units_total - 1));
+    for (int m = 0; m < 4; ++m) xr[m] = xg[(size_t)min(m, mrows - 1) * k_units + ku];
     load_batch(cur, wgb, 0);
+    if (tid < k_units) {
 #pragma unroll
-    for (int i = 0; i < XS; ++i) {
-      const int u = tid + i * (int)blockDim.x;
-      if (u < units_total) {
-        u32x4 v = xr[i];
-        if (FMT == TLHIP_FMT_INT4_GROUPED) v = permute_x_for_int4(v);
-        lds[u] = v;
+      for (int m = 0; m < 4; ++m) {
+        if (m < mrows) {
+          u32x4 v = xr[m];
+          if (FMT == TLHIP_FMT_INT4_GROUPED) v = permute_x_for_int4(v);
+          lds[m * row_units + ku] = v;
+        }
       }
     }
   } else {
     load_batch(cur, wgb, 0);
-    for (int u = tid; u < units_total; u += blockDim.x) {
-      u32x4 v = *x_src(u);
-      if (FMT == TLHIP_FMT_INT4_GROUPED) v = permute_x_for_int4(v);
-      lds[u] = v;
+    // 8 rows at a time: 8 loads in flight per thread, then 8 LDS stores
+    for (int ku0 = 0; ku0 < k_units; ku0 += blockDim.x) {
+      const int kuv = ku0 + tid;
+      const int ku = min(kuv, k_units - 1);
+      for (int m0 = 0; m0 < mrows; m0 += 8) {
+        u32x4 xr[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) xr[i] = xg[(size_t)min(m0 + i, mrows - 1) * k_units + ku];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          if (m0 + i < mrows && kuv < k_units) {
+            u32x4 v = xr[i];
+            if (FMT == TLHIP_FMT_INT4_GROUPED) v = permute_x_for_int4(v);
+            lds[(m0 + i) * row_units + ku] = v;
+          }
+        }
+      }
     }
   }
   lds_barrier();
 
-  while (wgb < a.nwgblocks) {
-    int nwgb = wgb, nstep = step + 1;
-    if (nstep == a.nsteps) {
-      nstep = 0;
-      nwgb = wgb + gridDim.x;
+  // Batches of this wave, in order: j -> (workgroup round j / nsteps, step j % nsteps).
+  // Two register sets ping-pong with no copies between them, and every load inside
+  // the steady-state loop is unconditional: a load under a branch makes the wait
+  // counters at the join assume it was NOT issued, and the consumer of the other
+  // set would then wait for the load just issued.
+  const int rounds = (a.nwgblocks - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;
+  const int total = rounds * a.nsteps;
+  auto advance = [&](int& b, int& st) {
+    if (++st == a.nsteps) {
+      st = 0;
+      b += gridDim.x;
     }
-    Batch nxt;
-    if (nwgb < a.nwgblocks) load_batch(nxt, nwgb, nstep);
-    compute_batch(cur, step);
-    if (step == a.nsteps - 1) finish(wgb);
-    cur = nxt;
-    wgb = nwgb;
-    step = nstep;
+  };
+  auto consume = [&](const Batch& b, int wb, int st) {
+    compute_batch(b, st);
+    if (st == a.nsteps - 1) finish(wb);
+  };
+  Batch other;
+  int j = 0;
+  while (total - j >= 3) {
+    int wgb1 = wgb, step1 = step;
+    advance(wgb1, step1);
+    load_batch(other, wgb1, step1);
+    consume(cur, wgb, step);
+    wgb = wgb1;
+    step = step1;
+    advance(wgb, step);
+    load_batch(cur, wgb, step);
+    consume(other, wgb1, step1);
+    j += 2;
+  }
+  if (total - j == 2) {
+    int wgb1 = wgb, step1 = step;
+    advance(wgb1, step1);
+    load_batch(other, wgb1, step1);
+    consume(cur, wgb, step);
+    consume(other, wgb1, step1);
+  } else if (total - j == 1) {
+    consume(cur, wgb, step);
   }
 }
 
@@ -293,7 +328,7 @@ static constexpr size_t kXLdsBudget = 144 * 1024;
 bool gemv_mfma_config_applicable(const Problem& p, const tlhip_kernel_config_t& c, const char** why) {
   static const char* reasons[] = {
       "not the gemv_mfma variant",
-      "waves per workgroup must be 4, 8 or 16",
+      "waves per workgroup must be 4 or 8",
       "activations must be f16",
       "M must be 1..16",
       "K must be a multiple of 128 (int4) or 64 (int8)",
@@ -307,7 +342,7 @@ bool gemv_mfma_config_applicable(const Problem& p, const tlhip_kernel_config_t& 
     return false;
   };
   if (c.variant != VARIANT_GEMV_MFMA) return fail(0);
-  if (c.p0 != 4 && c.p0 != 8 && c.p0 != 16) return fail(1);
+  if (c.p0 != 4 && c.p0 != 8) return fail(1);
   if (p.x_dtype != TLHIP_F16) return fail(2);
   if (p.m < 1 || p.m > 16) return fail(3);
   const int kper = p.format == TLHIP_FMT_INT4_GROUPED ? 128 : 64;
@@ -317,7 +352,7 @@ bool gemv_mfma_config_applicable(const Problem& p, const tlhip_kernel_config_t& 
   if (c.p1 != 1 && c.p1 != 2 && c.p1 != 4) return fail(6);
   const int kw = c.p2 == 0 ? c.p0 : c.p2;
   if (kw < 1 || (kw & (kw - 1)) != 0 || c.p0 % kw != 0) return fail(7);
-  if ((size_t)p.m * p.k * 2 + (size_t)c.p0 * 1024 > kXLdsBudget) return fail(8);
+  if ((size_t)p.m * (p.k * 2 + 16) + (size_t)c.p0 * 1024 > kXLdsBudget) return fail(8);
   return true;
 }
 
@@ -343,7 +378,6 @@ int launch_gemv_mfma(const Problem& p, const tlhip_kernel_config_t& c, hipStream
   if (p.n == 0 || p.m == 0) return TLHIP_OK;
   const bool int4 = p.format == TLHIP_FMT_INT4_GROUPED;
   const int cw = int4 ? 32 : 16;
-  const int steps = int4 ? 4 : 2;
   const int waves = c.p0, unroll = c.p1;
   MfmaArgs a;
   a.packed = (const u32x4*)p.packed;
@@ -353,7 +387,6 @@ int launch_gemv_mfma(const Problem& p, const tlhip_kernel_config_t& c, hipStream
   a.n = p.n;
   a.k = (int)p.k;
   a.m = (int)p.m;
-  a.m_magic = p.m > 1 ? (unsigned)((((uint64_t)1 << 32) + p.m - 1) / p.m) : 0u;
   a.nchunks = (int)(p.k / cw);
   a.cpg_shift = p.format == TLHIP_FMT_INT8_ROW ? 0 : __builtin_ctz((unsigned)(p.group_size / cw));
   a.groups_per_row = p.format == TLHIP_FMT_INT8_ROW ? 0 : (int)(p.k / p.group_size);
@@ -369,7 +402,7 @@ int launch_gemv_mfma(const Problem& p, const tlhip_kernel_config_t& c, hipStream
   a.y_dtype = p.y_dtype;
   a.epi = p.epi;
   const size_t partial_bytes = (size_t)waves * 256 * sizeof(float);
-  const size_t lds_bytes = (size_t)a.iters * steps * 4 * a.m * 16 + partial_bytes;
+  const size_t lds_bytes = (size_t)a.m * (p.k * 2 + 16) + partial_bytes;
   const int threads = waves * 64;
   const int cus = device_cu_count();
   int per_cu = 2048 / threads;
