@@ -28,21 +28,32 @@ __device__ __forceinline__ float half_bits_to_float(uint32_t h) {
 // (tanh form) from composite.ts:40-51, gelu_erf with the Abramowitz-Stegun
 // polynomial of erf.ts:28-56 — evaluated in f32 as the reference's GPU
 // epilogues are (src/schedule/matmul-skeleton.ts:916-966).
+// exp and 1/x through the hardware approximations (v_exp_f32 after a scale by
+// log2 e, v_rcp_f32: about 1 ulp each) instead of the correctly rounded library
+// routines, which cost 10-20 VALU instructions per element: the epilogue runs
+// once per output element and is a visible share of a GEMM tile's VALU time.
+__device__ __forceinline__ float fast_exp(float v) { return __expf(v); }
+__device__ __forceinline__ float fast_rcp(float v) { return __builtin_amdgcn_rcpf(v); }
+__device__ __forceinline__ float fast_tanh(float v) {
+  // tanh(v) = 1 - 2 / (1 + exp(2v)); exp overflow -> inf -> 1, underflow -> 0 -> -1
+  return 1.f - 2.f * fast_rcp(1.f + fast_exp(2.f * v));
+}
+
 __device__ __forceinline__ float apply_unary(int op, float v) {
   switch (op) {
     case TLHIP_UNARY_RELU: return v > 0.f ? v : 0.f;
-    case TLHIP_UNARY_SILU: return v / (1.f + expf(-v));
-    case TLHIP_UNARY_SIGMOID: return 1.f / (1.f + expf(-v));
-    case TLHIP_UNARY_TANH: return tanhf(v);
+    case TLHIP_UNARY_SILU: return v * fast_rcp(1.f + fast_exp(-v));
+    case TLHIP_UNARY_SIGMOID: return fast_rcp(1.f + fast_exp(-v));
+    case TLHIP_UNARY_TANH: return fast_tanh(v);
     case TLHIP_UNARY_GELU_TANH:
-      return (0.5f * v) * (1.f + tanhf(0.7978845608f * (v + 0.044715f * (v * (v * v)))));
+      return (0.5f * v) * (1.f + fast_tanh(0.7978845608f * (v + 0.044715f * (v * (v * v)))));
     case TLHIP_UNARY_GELU_ERF: {
       const float u = v * 0.70710678118654752f;
       const float ax = fabsf(u);
-      const float t = 1.f / (1.f + 0.3275911f * ax);
+      const float t = fast_rcp(1.f + 0.3275911f * ax);
       const float poly =
           ((((1.061405429f * t - 1.453152027f) * t + 1.421413741f) * t - 0.284496736f) * t + 0.254829592f) * t;
-      const float e = 1.f - poly * expf(-ax * ax);
+      const float e = 1.f - poly * fast_exp(-ax * ax);
       return (0.5f * v) * (1.f + (u < 0.f ? -e : e));
     }
     default: return v;

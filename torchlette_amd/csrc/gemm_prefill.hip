@@ -11,14 +11,15 @@
 // accumulators each.  Per K step of 64:
 //   * global -> registers: the X tile (f16, 16 bytes per lane per load) and the
 //     packed W tile (16 bytes = 32 int4 or 16 int8 weights, plus the group
-//     scale), for the NEXT step, issued before this step's MFMAs;
+//     scale), three or four steps ahead, in a ring of register stages;
 //   * registers -> LDS: the weights are unpacked to exact integers in f16 and
 //     multiplied by their scale (packed f16 multiply, one rounding to f16 per
 //     weight), then written k-contiguous; X is written as is (for int4, with
 //     the same within-8 k order the unpack produces);
 //   * LDS -> MFMA operands: rows are padded to 144 bytes so that the 32 lanes of
 //     an operand read hit 16 different 16-byte bank groups.
-// LDS is double buffered: one barrier per K step.
+// LDS is double buffered (one barrier per K step, and the barrier waits for LDS
+// traffic only, not for the global loads in flight).
 // Epilogue: acc*alpha -> ops in order (bias indexed by n, unary) -> cast, the
 // order of applyBlockEpilogue (matmul-skeleton.ts:916-966).
 #include "device_utils.h"
@@ -137,17 +138,23 @@ __global__ __launch_bounds__(256) void gemm_prefill_kernel(const GemmArgs a) {
   const int m0 = tm_idx * BM, n0 = tn_idx * BN;
 
   // ---- global -> register staging -------------------------------------
-  u32x4 xr[X_LOADS];
-  u32x4 wr[W_LOADS];
-  uint32_t sr[W_LOADS];  // raw scale bits (f16) or f32 bits (int8-row)
+  // A ring of D register stages: the tiles of K step j live in stage j % D.
+  // At step ks the loads for step ks+D are issued (into the stage that held
+  // step ks, already in LDS), the tiles of step ks+1 go from registers to the
+  // other LDS buffer, and the MFMAs run on step ks: every global load has D-1
+  // full steps to arrive.  All loads are unconditional (clamped at the end).
+  constexpr int D = (BM + BN) >= 512 ? 3 : 4;
+  u32x4 xr[D][X_LOADS];
+  u32x4 wr[D][W_LOADS];
+  uint32_t sr[D][W_LOADS];  // raw scale bits (f16) or f32 bits (int8-row)
 
-  auto load_tiles = [&](int kstep) {
-    const int k0 = kstep * BK;
+  auto load_tiles = [&](int kstep, u32x4 (&xs)[X_LOADS], u32x4 (&ws)[W_LOADS], uint32_t (&ss)[W_LOADS]) {
+    const int k0 = min(kstep, a.ksteps - 1) * BK;
 #pragma unroll
     for (int i = 0; i < X_LOADS; ++i) {
       const int u = tid + i * 256;
       const int row = min(m0 + (u >> 3), a.m - 1);
-      xr[i] = *(const u32x4*)(a.x + (size_t)row * a.k + k0 + (u & 7) * 8);
+      xs[i] = *(const u32x4*)(a.x + (size_t)row * a.k + k0 + (u & 7) * 8);
     }
 #pragma unroll
     for (int i = 0; i < W_LOADS; ++i) {
@@ -155,19 +162,20 @@ __global__ __launch_bounds__(256) void gemm_prefill_kernel(const GemmArgs a) {
       const int r = u / W_CHUNKS_PER_ROW, c = u - r * W_CHUNKS_PER_ROW;
       const int row = min(n0 + r, a.n - 1);
       const int chunk = k0 / WC::WEIGHTS + c;
-      wr[i] = *(const u32x4*)(a.packed + (size_t)row * a.w_row_bytes + (size_t)chunk * 16);
-      if (GROUPED) sr[i] = ((const uint16_t*)a.scales)[(size_t)row * a.groups_per_row + (chunk >> a.cpg_shift)];
-      else sr[i] = ((const uint32_t*)a.scales)[row];
+      ws[i] = *(const u32x4*)(a.packed + (size_t)row * a.w_row_bytes + (size_t)chunk * 16);
+      if (GROUPED) ss[i] = ((const uint16_t*)a.scales)[(size_t)row * a.groups_per_row + (chunk >> a.cpg_shift)];
+      else ss[i] = ((const uint32_t*)a.scales)[row];
     }
   };
 
-  auto store_tiles = [&](int buf) {
+  auto store_tiles = [&](int buf, const u32x4 (&xv)[X_LOADS], const u32x4 (&wv)[W_LOADS],
+                         const uint32_t (&sv)[W_LOADS]) {
     u32x4* xs = lds + buf * STAGE_UNITS;
     u32x4* ws = xs + BM * ROW_UNITS;
 #pragma unroll
     for (int i = 0; i < X_LOADS; ++i) {
       const int u = tid + i * 256;
-      u32x4 v = xr[i];
+      u32x4 v = xv[i];
       if (FMT == TLHIP_FMT_INT4_GROUPED) v = permute_x_for_int4(v);
       xs[(u >> 3) * ROW_UNITS + (u & 7)] = v;
     }
@@ -175,9 +183,9 @@ __global__ __launch_bounds__(256) void gemm_prefill_kernel(const GemmArgs a) {
     for (int i = 0; i < W_LOADS; ++i) {
       const int u = tid + i * 256;
       const int r = u / W_CHUNKS_PER_ROW, c = u - r * W_CHUNKS_PER_ROW;
-      const float s = (GROUPED ? half_bits_to_float(sr[i]) : as_float(sr[i])) * a.scale_mul;
+      const float s = (GROUPED ? half_bits_to_float(sv[i]) : as_float(sv[i])) * a.scale_mul;
       u32x4 out[WC::UNITS];
-      WC::dequant(wr[i], s, out);
+      WC::dequant(wv[i], s, out);
 #pragma unroll
       for (int j = 0; j < WC::UNITS; ++j) ws[r * ROW_UNITS + c * WC::UNITS + j] = out[j];
     }
@@ -191,54 +199,70 @@ __global__ __launch_bounds__(256) void gemm_prefill_kernel(const GemmArgs a) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  load_tiles(0);
-  store_tiles(0);
-  __syncthreads();
+#pragma unroll
+  for (int s = 0; s < D; ++s) load_tiles(s, xr[s], wr[s], sr[s]);
+  store_tiles(0, xr[0], wr[0], sr[0]);
+  lds_barrier();
 
   const int lrow = lane & 31, lk = lane >> 5;
-  for (int ks = 0; ks < a.ksteps; ++ks) {
-    const int buf = ks & 1;
-    const bool more = ks + 1 < a.ksteps;
-    if (more) load_tiles(ks + 1);
-    const u32x4* xs = lds + buf * STAGE_UNITS;
-    const u32x4* ws = xs + BM * ROW_UNITS;
+  for (int ks0 = 0; ks0 < a.ksteps; ks0 += D) {
 #pragma unroll
-    for (int kk = 0; kk < BK / 16; ++kk) {
-      half8_t af[TM], bf[TN];
+    for (int s = 0; s < D; ++s) {
+      const int ks = ks0 + s;
+      if (ks < a.ksteps) {  // uniform
+        const int buf = ks & 1;
+        // stage s held step ks (already in LDS): refill it with step ks + D
+        load_tiles(ks + D, xr[s], wr[s], sr[s]);
+        const u32x4* xs = lds + buf * STAGE_UNITS;
+        const u32x4* ws = xs + BM * ROW_UNITS;
 #pragma unroll
-      for (int i = 0; i < TM; ++i)
-        af[i] = __builtin_bit_cast(half8_t, xs[(wm * (BM / 2) + i * 32 + lrow) * ROW_UNITS + kk * 2 + lk]);
+        for (int kk = 0; kk < BK / 16; ++kk) {
+          half8_t af[TM], bf[TN];
 #pragma unroll
-      for (int j = 0; j < TN; ++j)
-        bf[j] = __builtin_bit_cast(half8_t, ws[(wn * (BN / 2) + j * 32 + lrow) * ROW_UNITS + kk * 2 + lk]);
+          for (int i = 0; i < TM; ++i)
+            af[i] = __builtin_bit_cast(half8_t, xs[(wm * (BM / 2) + i * 32 + lrow) * ROW_UNITS + kk * 2 + lk]);
 #pragma unroll
-      for (int i = 0; i < TM; ++i)
+          for (int j = 0; j < TN; ++j)
+            bf[j] = __builtin_bit_cast(half8_t, ws[(wn * (BN / 2) + j * 32 + lrow) * ROW_UNITS + kk * 2 + lk]);
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
+          for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+              acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
+        }
+        // step ks + 1 (stage s+1) -> the other LDS buffer; harmless past the end
+        store_tiles(buf ^ 1, xr[(s + 1) % D], wr[(s + 1) % D], sr[(s + 1) % D]);
+        lds_barrier();
+      }
     }
-    if (more) store_tiles(buf ^ 1);
-    __syncthreads();
   }
 
   // ---- epilogue -----------------------------------------------------------
   // 32x32 accumulator layout: lane l holds column l%32 and rows
-  // 8*(r/4) + 4*(l/32) + r%4 for r = 0..15.
+  // 8*(r/4) + 4*(l/32) + r%4 for r = 0..15.  Each tile goes through a private
+  // 32 x 33 f32 patch of LDS (the staging buffers are free now): registers are
+  // written with static indices, and a short rolled loop reads the patch back,
+  // applies the epilogue and stores.  Applying the epilogue straight from the
+  // registers would need 16 x TM x TN inlined copies of it; the compiler then
+  // stops unrolling and the accumulators fall into scratch memory.
+  float* patch = (float*)lds + wave * (32 * 33);
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
-    const int64_t col = n0 + wn * (BN / 2) + j * 32 + lrow;
-    if (col < a.n) {
 #pragma unroll
-      for (int i = 0; i < TM; ++i) {
+    for (int i = 0; i < TM; ++i) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int row = m0 + wm * (BM / 2) + i * 32 + 8 * (r >> 2) + 4 * lk + (r & 3);
-          if (row < a.m) {
-            const float v = apply_epilogue(a.epi, acc[i][j][r] * a.alpha, col);
-            store_out(a.y, a.y_dtype, (int64_t)row * a.n + col, v);
-          }
-        }
+      for (int r = 0; r < 16; ++r) patch[(8 * (r >> 2) + 4 * lk + (r & 3)) * 33 + lrow] = acc[i][j][r];
+      __builtin_amdgcn_s_waitcnt(0xc07f);  // this wave's LDS writes have landed (lgkmcnt(0))
+      const int64_t col = n0 + wn * (BN / 2) + j * 32 + lrow;
+      const int row0 = m0 + wm * (BM / 2) + i * 32 + lk;
+#pragma unroll 1
+      for (int it = 0; it < 16; ++it) {
+        const int row = row0 + 2 * it;
+        const float v = patch[(2 * it + lk) * 33 + lrow];
+        if (row < a.m && col < a.n)
+          store_out(a.y, a.y_dtype, (int64_t)row * a.n + col, apply_epilogue(a.epi, v * a.alpha, col));
       }
+      __builtin_amdgcn_s_waitcnt(0xc07f);  // reads done before the patch is overwritten
     }
   }
 }
