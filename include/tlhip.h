@@ -204,6 +204,12 @@ int tlhip_unary(int op, const void* in, int dtype, void* out, int64_t count, tlh
 int tlhip_cast(const void* in, int in_dtype, void* out, int out_dtype, int64_t count,
                tlhip_stream_t stream);
 
+/* Measuring stick for the decode GEMV (no counterpart in the reference): reads
+ * `bytes` bytes at `ptr` once with 16-byte loads and discards them.  Timed like
+ * a GEMV launch of the same size, it gives the rate a single launch of that size
+ * can reach at all.  `sink4` is 4 writable device bytes. */
+int tlhip_hbm_read_probe(const void* ptr, size_t bytes, void* sink4, tlhip_stream_t stream);
+
 /* ---- kernel choice: variant registry + autotuner
  * (src/backend/webgpu/matmul/variants.ts:54-260; autotune.ts:48-547;
  * dispatch.ts:60-207, 405-578) ---- */
@@ -249,6 +255,11 @@ int tlhip_is_autotune_enabled(void);
  * (m, n, k, format, group, x dtype, y dtype).  Runs on the library stream. */
 int tlhip_autotune(const tlhip_qweight_t* w, const void* x, int x_dtype, int64_t m, void* y,
                    int y_dtype, double* host_out_best_us);
+/* seedPerShapeMatmulChoice (dispatch.ts:99-107): record a winner for this
+ * problem without benchmarking (tests, pre-seeded caches, a caller's own
+ * timing loop).  Fails if the configuration is not applicable. */
+int tlhip_tune_cache_seed(const tlhip_qweight_t* w, int x_dtype, int64_t m, int y_dtype,
+                          const tlhip_kernel_config_t* config);
 /* Backend.pretuneMatmulShapes (src/backend/types.ts:688): [m,n,k] triples.
  * The hook carries no operand format, so it only records shape hints; tuning
  * happens at first dispatch of a matching packed operand when enabled. */

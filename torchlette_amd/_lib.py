@@ -103,12 +103,14 @@ SIGNATURES = {
     "tlhip_bias_add": (_i, [_vp, _i, _vp, _i, _vp, _i64, _i64, _vp]),
     "tlhip_unary": (_i, [_i, _vp, _i, _vp, _i64, _vp]),
     "tlhip_cast": (_i, [_vp, _i, _vp, _i, _i64, _vp]),
+    "tlhip_hbm_read_probe": (_i, [_vp, _sz, _vp, _vp]),
     "tlhip_candidate_count": (_i, [_QW, _i, _i64, _i, C.POINTER(_i)]),
     "tlhip_candidate_get": (_i, [_QW, _i, _i64, _i, _i, _KC]),
     "tlhip_selected_config": (_i, [_QW, _i, _i64, _i, _KC]),
     "tlhip_set_autotune_enabled": (_i, [_i]),
     "tlhip_is_autotune_enabled": (_i, []),
     "tlhip_autotune": (_i, [_QW, _vp, _i, _i64, _vp, _i, C.POINTER(C.c_double)]),
+    "tlhip_tune_cache_seed": (_i, [_QW, _i, _i64, _i, _KC]),
     "tlhip_pretune_matmul_shapes": (_i, [C.POINTER(_i64), _i]),
     "tlhip_tune_cache_export": (_i, [C.c_char_p, _sz, C.POINTER(_sz)]),
     "tlhip_tune_cache_import": (_i, [C.c_char_p]),

@@ -480,6 +480,12 @@ class HipBackend:
             out.append(kc)
         return out
 
+    def seedPerShapeMatmulChoice(self, weight: HipTensor, x_dtype: str, m: int, y_dtype: str,
+                                 config: L.KernelConfig) -> None:
+        """dispatch.ts:99-107: record a winner without benchmarking."""
+        qw = self._qweight(weight, transposed=False)
+        L.call("tlhip_tune_cache_seed", C.byref(qw), _DT_CODE[x_dtype], m, _DT_CODE[y_dtype], C.byref(config))
+
     def selectedConfig(self, weight: HipTensor, x_dtype: str, m: int, y_dtype: str) -> L.KernelConfig:
         qw = self._qweight(weight, transposed=False)
         kc = L.KernelConfig()

@@ -454,6 +454,20 @@ int tlhip_selected_config(const tlhip_qweight_t* w, int x_dtype, int64_t m, int 
   return TLHIP_OK;
 }
 
+int tlhip_tune_cache_seed(const tlhip_qweight_t* w, int x_dtype, int64_t m, int y_dtype,
+                          const tlhip_kernel_config_t* config) {
+  Problem p;
+  int rc = shape_problem(w, x_dtype, m, y_dtype, &p);
+  if (rc) return rc;
+  if (!config) return set_error(TLHIP_ERR_INVALID, "tune_cache_seed: null config");
+  const char* why = nullptr;
+  if (!config_applicable(p, *config, &why))
+    return set_error(TLHIP_ERR_INVALID, "tune_cache_seed: config not applicable: %s", why ? why : "?");
+  std::lock_guard<std::mutex> lock(g_tune_mutex);
+  g_tuned[problem_key(p)] = *config;
+  return TLHIP_OK;
+}
+
 int tlhip_set_autotune_enabled(int enabled) {
   // dispatch.ts:128-134: true increments (nested regions), false resets to 0.
   if (enabled) g_autotune_counter++;

@@ -1,0 +1,42 @@
+// A read-only streaming kernel used as the measuring stick for the decode
+// GEMV: it does what the GEMV must do at the very least (fetch every byte of
+// the packed weight once with 16-byte loads) and nothing else.  Timed with the
+// same back-to-back launches as the GEMV, it shows how much of the 8 TB/s peak a
+// single launch of a given size can reach at all once launch overhead and the
+// ramp of the memory pipeline are paid.
+#include "device_utils.h"
+
+namespace tlhip {
+namespace {
+
+__global__ __launch_bounds__(256) void hbm_read_probe_kernel(const u32x4* __restrict__ p, size_t n16,
+                                                            uint32_t* __restrict__ sink) {
+  const size_t tid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  uint32_t acc = 0;
+  for (size_t i = tid; i < n16; i += stride) {
+    const u32x4 v = __builtin_nontemporal_load(p + i);
+    acc ^= v.x ^ v.y ^ v.z ^ v.w;
+  }
+  if (acc == 0x9e3779b9u) sink[0] = acc;  // keeps the loads alive; practically never taken
+}
+
+}  // namespace
+}  // namespace tlhip
+
+using namespace tlhip;
+
+extern "C" int tlhip_hbm_read_probe(const void* ptr, size_t bytes, void* sink4, tlhip_stream_t stream) {
+  TLHIP_REQUIRE_INIT();
+  if (!ptr || !sink4) return set_error(TLHIP_ERR_INVALID, "hbm_read_probe: null pointer");
+  if (((uintptr_t)ptr & 15) != 0) return set_error(TLHIP_ERR_INVALID, "hbm_read_probe: pointer must be 16-byte aligned");
+  const size_t n16 = bytes / 16;
+  if (n16 == 0) return TLHIP_OK;
+  const size_t blocks = (n16 + 255) / 256;
+  const size_t cap = (size_t)device_cu_count() * 8;  // 8 workgroups of 4 waves per CU: the best measured shape
+  const int grid = (int)(blocks < cap ? blocks : cap);
+  hipLaunchKernelGGL(hbm_read_probe_kernel, dim3(grid), dim3(256), 0, resolve_stream(stream), (const u32x4*)ptr, n16,
+                     (uint32_t*)sink4);
+  TLHIP_CHECK_HIP(hipGetLastError());
+  return TLHIP_OK;
+}
