@@ -221,7 +221,7 @@ typedef struct {
   int32_t p0; /* gemv: lanes per row (16/32/64)   gemv_mfma: waves per workgroup   tiled: tile M */
   int32_t p1; /* gemv: rows per lane-group        gemv_mfma: iterations in flight  tiled: tile N */
   int32_t p2; /* gemv: waves per workgroup        gemv_mfma: K-split waves (0 = all)  tiled: tile K */
-  int32_t p3; /* gemv: K-split waves (LDS combine) tiled: waves M */
+  int32_t p3; /* gemv: K-split waves (LDS combine) gemv_mfma: K slices across workgroups (0/1 = none)  tiled: waves M */
   int32_t p4; /* gemv: chunks in flight (2/4/8)    tiled: waves N */
   int32_t p5;
   int32_t p6;

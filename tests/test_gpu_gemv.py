@@ -97,6 +97,57 @@ def test_every_candidate_config_gives_the_same_answer(be):
         assert rel_l2(got, want) <= 2e-6, c.as_tuple()
 
 
+@pytest.mark.parametrize("fmt,n,k,g", [
+    ("int4-grouped", 4096, 12288, 32), ("int4-grouped", 1000, 4096, 64),
+    ("int8-grouped", 520, 4096, 128), ("int8-row", 1031, 2304, 0),
+])
+@pytest.mark.parametrize("m", [5, 8, 13, 16])
+def test_matrix_core_kernel_with_k_slices_across_workgroups(be, fmt, n, k, g, m):
+    """Slices of K on different workgroups, combined by the last arriver: same
+    answer for every slice count, bit-identical on repeated launches (the sum
+    runs in slice order whoever arrives last), counters back at zero each time."""
+    rng = np.random.default_rng(n + k + m)
+    packed, scales, deq = make_weight(fmt, n, k, g, rng)
+    x = make_x(m, k, "f16", rng)
+    bias = rng.standard_normal(n).astype(np.float32)
+    want = O.linear(x.astype(np.float32), deq, bias, "silu", threads=8)
+    w = be.createQuantizedWeight(packed, scales, n, k, T.resolveWeightFormat(fmt_name(fmt, g), "f32"))
+    xt = be.ops.tensorFromArray(x, [m, k], "f16")
+    bt = be.ops.tensorFromArray(bias, [n], "f32")
+    ran = 0
+    for ks in (2, 4, 8, 16):
+        for waves, unroll, kw in ((8, 2, 8), (4, 1, 1), (8, 4, 2)):
+            c = L.KernelConfig.of(1, waves, unroll, kw, ks)
+            if c.as_tuple() not in [d.as_tuple() for d in be.candidates(w, "f16", m, "f32")] and ks != 16:
+                continue
+            try:
+                first = None
+                for _ in range(3):
+                    y = be.linear(xt, w, bt, "silu", fused=True, config=c)
+                    got = y.numpy()
+                    y.destroy()
+                    if first is None:
+                        first = got
+                    assert np.array_equal(got, first), c.as_tuple()
+            except L.TlhipError as e:
+                assert "not applicable" in str(e), str(e)
+                continue
+            ran += 1
+            assert rel_l2(first, want) <= 5e-6, (c.as_tuple(), rel_l2(first, want))
+    assert ran >= 3
+
+
+def test_k_slices_reject_what_the_workspace_cannot_hold(be):
+    rng = np.random.default_rng(5)
+    n, k, m = 256, 1024, 8
+    packed, scales, _ = make_weight("int4-grouped", n, k, 32, rng)
+    w = be.createQuantizedWeight(packed, scales, n, k, T.resolveWeightFormat("int4-32", "f32"))
+    xt = be.ops.tensorFromArray(make_x(m, k, "f16", rng), [m, k], "f16")
+    for ks in (3, 16, 32):   # not a power of two / does not divide K/128 = 8 / too many
+        with pytest.raises(L.TlhipError, match="config not applicable"):
+            be.linear(xt, w, config=L.KernelConfig.of(1, 8, 2, 8, ks))
+
+
 @pytest.mark.parametrize("fmt,g,xdt", [("int8-grouped", 64, "f32"), ("int8-row", 0, "f16"), ("int4-grouped", 64, "f32")])
 def test_candidates_other_formats(be, fmt, g, xdt):
     rng = np.random.default_rng(43)

@@ -71,6 +71,15 @@ int launch_gemv_mfma(const Problem& p, const tlhip_kernel_config_t& c, hipStream
 bool gemm_config_applicable(const Problem& p, const tlhip_kernel_config_t& c, const char** why);
 int launch_gemm(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t stream);
 
+// Device scratch for kernels that combine partial results of several workgroups:
+// `kSplitWorkspaceFloats` floats plus `kSplitCounters` arrival counters that are
+// zero whenever no launch is in flight.  One per stream, so launches on different
+// streams never share it; created on the stream's first use, which must not
+// happen while the stream is being captured.
+constexpr size_t kSplitWorkspaceFloats = 4u << 20;  // 16 MiB
+constexpr int kSplitCounters = 1 << 16;
+int split_workspace(hipStream_t stream, float** workspace, int** counters);
+
 // Counters.
 void count_gemv_dispatch();
 void count_gemm_dispatch();

@@ -69,13 +69,14 @@ tlhip_kernel_config_t gemv_cfg(int lpr, int r, int waves, int kw, int unroll) {
   return c;
 }
 
-tlhip_kernel_config_t mfma_cfg(int waves, int unroll, int kw) {
+tlhip_kernel_config_t mfma_cfg(int waves, int unroll, int kw, int ks = 1) {
   tlhip_kernel_config_t c;
   memset(&c, 0, sizeof c);
   c.variant = VARIANT_GEMV_MFMA;
   c.p0 = waves;
   c.p1 = unroll;
   c.p2 = kw;
+  c.p3 = ks;
   return c;
 }
 
@@ -114,8 +115,11 @@ tlhip_kernel_config_t default_config(const Problem& p) {
   // five or more activation rows: the matrix-core kernel streams the weights once
   // (below that the VALU kernel with its rows held in registers measures faster)
   if (p.m >= 5 && p.m <= 16) {
-    tlhip_kernel_config_t c = mfma_cfg(8, 2, p.n >= 32768 ? 1 : 8);
-    if (gemv_mfma_config_applicable(p, c, nullptr)) return c;
+    // the fewest K slices across workgroups whose activations fit LDS (measured best)
+    for (int ks = 1; ks <= 16; ks *= 2) {
+      tlhip_kernel_config_t c = mfma_cfg(8, 2, p.n >= 32768 ? 1 : (ks > 1 ? 4 : 8), ks);
+      if (gemv_mfma_config_applicable(p, c, nullptr)) return c;
+    }
   }
   // lanes per row: every lane busy for short rows; all chunks of a row in flight at once
   int lpr = 64;
@@ -145,11 +149,12 @@ std::vector<tlhip_kernel_config_t> candidates(const Problem& p) {
   if (p.m <= 16) {
     for (int waves : {4, 8})
       for (int unroll : {1, 2, 4})
-        for (int kw : {1, 2, 4, 8}) {
-          if (kw > waves) continue;
-          tlhip_kernel_config_t c = mfma_cfg(waves, unroll, kw);
-          if (gemv_mfma_config_applicable(p, c, nullptr)) out.push_back(c);
-        }
+        for (int kw : {1, 2, 4, 8})
+          for (int ks : {1, 2, 4, 8}) {
+            if (kw > waves) continue;
+            tlhip_kernel_config_t c = mfma_cfg(waves, unroll, kw, ks);
+            if (gemv_mfma_config_applicable(p, c, nullptr)) out.push_back(c);
+          }
   }
   if (p.x_dtype == TLHIP_F16 && p.m >= 16) {
     static const int tiles[][5] = {

@@ -34,14 +34,19 @@ struct MfmaArgs {
   const void* scales;
   const _Float16* x;
   void* y;
+  float* workspace;   // split-K partial tiles: [(row block * ks + slice) * 256]
+  int* counters;      // split-K arrival counters, one per row block; zero between launches
   int64_t n;
   int k;
   int m;
   int nchunks;        // 16-byte chunks per weight row
   int cpg_shift;      // log2(chunks per scale group), grouped formats
   int groups_per_row;
-  int iters;          // wave iterations over K: 4 chunks each
-  int kw;             // waves that split K for one 16-row block (power of two)
+  int ks;             // K slices handled by different workgroups (1 = none, power of two)
+  int ks_shift;
+  int slice_iters;    // wave iterations (4 chunks each) per K slice
+  int iters;          // wave iterations over all of K
+  int kw;             // waves that split a slice for one 16-row block (power of two)
   int kw_shift;
   int blocks_per_wg;  // 16-row blocks a workgroup works on at a time = waves / kw
   int nsteps;         // batches (U iterations each) per row block per wave
@@ -121,10 +126,21 @@ __global__ __launch_bounds__(512) void gemv_mfma_kernel(const MfmaArgs a) {
   const int g = lane >> 4;    // k sub-block
   const int mrows = a.m;
   const int ml = nl < mrows ? nl : mrows - 1;  // rows beyond M alias the last row; never stored
-  const int k_units = a.k >> 3;        // 16-byte units per activation row
-  const int row_units = k_units + 1;   // padded LDS row stride
+
+  // A workgroup keeps ONE K slice (all of K when ks == 1) of the activations in
+  // LDS and walks row-block groups with a grid stride; the ks workgroups of
+  // consecutive blockIdx take the ks slices of the same row-block groups.
+  const int slice = blockIdx.x & (a.ks - 1);
+  const int wg_stride = gridDim.x >> a.ks_shift;
+  int wgb = blockIdx.x >> a.ks_shift;
+  const int it_begin = slice * a.slice_iters;
+  const int last_local = a.slice_iters - 1;  // slices are equal: ks divides the iterations
+  constexpr int UNITS_PER_ITER = FMT == TLHIP_FMT_INT4_GROUPED ? 16 : 8;  // 16-byte x units per iteration
+  const int slice_units = a.slice_iters * UNITS_PER_ITER;  // resident x units per row
+  const int row_units = slice_units + 1;                    // padded LDS row stride
+  const int ku0 = it_begin * UNITS_PER_ITER;                // first resident unit
+  const int k_units = a.k >> 3;                             // units per activation row in memory
   float* partial = (float*)(lds + (size_t)row_units * mrows);
-  const int last_iter = a.iters - 1;
 
   // Raw loaded values only (no conversion at issue time, see gemv.hip).
   struct Batch {
@@ -132,14 +148,14 @@ __global__ __launch_bounds__(512) void gemv_mfma_kernel(const MfmaArgs a) {
     uint16_t s[U][STEPS];
   };
 
-  auto load_batch = [&](Batch& b, int wgb, int step) {
-    const int rb = min(wgb * a.blocks_per_wg + bw_idx, a.nblocks - 1);
+  auto load_batch = [&](Batch& b, int wb, int step) {
+    const int rb = min(wb * a.blocks_per_wg + bw_idx, a.nblocks - 1);
     const int64_t row = min((int64_t)rb * 16 + nl, a.n - 1);
     const u32x4* wrow = a.packed + row * a.nchunks;
     const uint16_t* srow = (const uint16_t*)a.scales + row * a.groups_per_row;
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const int it = min(kw_idx + (step * U + u) * a.kw, last_iter);
+      const int it = it_begin + min(kw_idx + (step * U + u) * a.kw, last_local);
       b.w[u] = __builtin_nontemporal_load(wrow + it * 4 + g);
       if (GROUPED) {
 #pragma unroll
@@ -157,10 +173,9 @@ __global__ __launch_bounds__(512) void gemv_mfma_kernel(const MfmaArgs a) {
   auto compute_batch = [&](const Batch& b, int step) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const int it_raw = kw_idx + (step * U + u) * a.kw;
-      const bool valid = it_raw <= last_iter;  // wave-uniform
-      const int it = min(it_raw, last_iter);
-      const int tl = it * STEPS;
+      const int it_raw = kw_idx + (step * U + u) * a.kw;  // local to the slice
+      const bool valid = it_raw <= last_local;             // wave-uniform
+      const int tl = min(it_raw, last_local) * STEPS;
       uint32_t w0 = b.w[u].x, w1 = b.w[u].y, w2 = b.w[u].z, w3 = b.w[u].w;
       half8_t bw[STEPS];
       if (FMT == TLHIP_FMT_INT4_GROUPED) {
@@ -200,9 +215,10 @@ __global__ __launch_bounds__(512) void gemv_mfma_kernel(const MfmaArgs a) {
     }
   };
 
-  // Combine the K parts (through LDS when kw > 1), apply the epilogue, store.
-  auto finish = [&](int wgb) {
-    const int rb = wgb * a.blocks_per_wg + bw_idx;
+  // Combine the K parts of the workgroup (through LDS when kw > 1) and of the
+  // other workgroups (through the workspace when ks > 1), apply the epilogue, store.
+  auto finish = [&](int wb) {
+    const int rb = wb * a.blocks_per_wg + bw_idx;
     if (a.kw > 1) {
       lds_barrier();  // the previous round's readers are done with `partial`
 #pragma unroll
@@ -217,7 +233,40 @@ __global__ __launch_bounds__(512) void gemv_mfma_kernel(const MfmaArgs a) {
         }
       }
     }
-    if (kw_idx == 0 && rb < a.nblocks) {
+    bool owner = kw_idx == 0 && rb < a.nblocks;  // wave-uniform
+    if (owner && a.ks > 1) {
+      // Publish this slice's tile; the workgroup that arrives last for the row
+      // block adds the ks tiles in slice order (so the sum does not depend on
+      // who is last), resets the counter for the next launch and stores.
+      // Tiles and counters move with device-scope atomic accesses only: those
+      // are coherent between the L2 caches of the chip by themselves, and a
+      // device-scope fence (a write-back and invalidate of a whole L2 per row
+      // block) measured 3x slower for the whole kernel.  Order: tile stores,
+      // wait until the memory system has acknowledged them, then the counter.
+      float* mine = a.workspace + ((size_t)rb * a.ks + slice) * 256;
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        __hip_atomic_store(mine + (4 * g + r) * 16 + nl, acc[r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+      __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): every store of this wave is acknowledged
+      int old = 0;
+      if (lane == 0) old = __hip_atomic_fetch_add(a.counters + rb, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      old = __shfl(old, 0);
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+      owner = old == a.ks - 1;
+      if (owner) {
+        const float* tiles = a.workspace + (size_t)rb * a.ks * 256;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          float s = 0.f;
+          for (int sl = 0; sl < a.ks; ++sl)
+            s += __hip_atomic_load(tiles + sl * 256 + (4 * g + r) * 16 + nl, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          acc[r] = s;
+        }
+        if (lane == 0) __hip_atomic_store(a.counters + rb, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+    if (owner) {
       const int64_t orow = (int64_t)rb * 16 + nl;
       if (orow < a.n) {
         float rs = a.scale_mul * a.alpha;
@@ -237,16 +286,17 @@ __global__ __launch_bounds__(512) void gemv_mfma_kernel(const MfmaArgs a) {
 
   // Activations first (they return first), then the first weight batch, then
   // the LDS store.  Row by row, consecutive threads on consecutive 16-byte units.
-  const u32x4* xg = (const u32x4*)a.x;
-  int wgb = blockIdx.x, step = 0;
+  const u32x4* xg = (const u32x4*)a.x + ku0;
+  const int res_units = slice_units;
+  int step = 0;
   Batch cur;
-  if (k_units <= (int)blockDim.x && mrows <= 4) {
+  if (res_units <= (int)blockDim.x && mrows <= 4) {
     u32x4 xr[4];
-    const int ku = min(tid, k_units - 1);
+    const int ku = min(tid, res_units - 1);
 #pragma unroll
     for (int m = 0; m < 4; ++m) xr[m] = xg[(size_t)min(m, mrows - 1) * k_units + ku];
     load_batch(cur, wgb, 0);
-    if (tid < k_units) {
+    if (tid < res_units) {
 #pragma unroll
       for (int m = 0; m < 4; ++m) {
         if (m < mrows) {
@@ -259,16 +309,16 @@ __global__ __launch_bounds__(512) void gemv_mfma_kernel(const MfmaArgs a) {
   } else {
     load_batch(cur, wgb, 0);
     // 8 rows at a time: 8 loads in flight per thread, then 8 LDS stores
-    for (int ku0 = 0; ku0 < k_units; ku0 += blockDim.x) {
-      const int kuv = ku0 + tid;
-      const int ku = min(kuv, k_units - 1);
+    for (int kb = 0; kb < res_units; kb += blockDim.x) {
+      const int kuv = kb + tid;
+      const int ku = min(kuv, res_units - 1);
       for (int m0 = 0; m0 < mrows; m0 += 8) {
         u32x4 xr[8];
 #pragma unroll
         for (int i = 0; i < 8; ++i) xr[i] = xg[(size_t)min(m0 + i, mrows - 1) * k_units + ku];
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-          if (m0 + i < mrows && kuv < k_units) {
+          if (m0 + i < mrows && kuv < res_units) {
             u32x4 v = xr[i];
             if (FMT == TLHIP_FMT_INT4_GROUPED) v = permute_x_for_int4(v);
             lds[(m0 + i) * row_units + ku] = v;
@@ -284,12 +334,12 @@ __global__ __launch_bounds__(512) void gemv_mfma_kernel(const MfmaArgs a) {
   // the steady-state loop is unconditional: a load under a branch makes the wait
   // counters at the join assume it was NOT issued, and the consumer of the other
   // set would then wait for the load just issued.
-  const int rounds = (a.nwgblocks - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;
+  const int rounds = (a.nwgblocks - wgb + wg_stride - 1) / wg_stride;
   const int total = rounds * a.nsteps;
   auto advance = [&](int& b, int& st) {
     if (++st == a.nsteps) {
       st = 0;
-      b += gridDim.x;
+      b += wg_stride;
     }
   };
   auto consume = [&](const Batch& b, int wb, int st) {
@@ -335,7 +385,9 @@ bool gemv_mfma_config_applicable(const Problem& p, const tlhip_kernel_config_t& 
       "group size must be a multiple of 32 (int4) or 64 (int8)",
       "iterations in flight must be 1, 2 or 4",
       "K-split waves must be a power of two that divides the waves per workgroup",
-      "activations (M x K f16) do not fit LDS",
+      "activations (M x K/slices f16) do not fit LDS",
+      "K slices must be a power of two (1..16) that divides K/128 (int4) or K/64 (int8)",
+      "K slices need more partial-tile workspace or counters than the library holds",
   };
   auto fail = [&](int i) {
     if (why) *why = reasons[i];
@@ -352,7 +404,14 @@ bool gemv_mfma_config_applicable(const Problem& p, const tlhip_kernel_config_t& 
   if (c.p1 != 1 && c.p1 != 2 && c.p1 != 4) return fail(6);
   const int kw = c.p2 == 0 ? c.p0 : c.p2;
   if (kw < 1 || (kw & (kw - 1)) != 0 || c.p0 % kw != 0) return fail(7);
-  if ((size_t)p.m * (p.k * 2 + 16) + (size_t)c.p0 * 1024 > kXLdsBudget) return fail(8);
+  const int ks = c.p3 < 1 ? 1 : c.p3;
+  const int64_t iters = p.k / kper;
+  if (ks > 16 || (ks & (ks - 1)) != 0 || iters % ks != 0) return fail(9);
+  if ((size_t)p.m * (p.k / ks * 2 + 16) + (size_t)c.p0 * 1024 > kXLdsBudget) return fail(8);
+  if (ks > 1) {
+    const int64_t nblocks = (p.n + 15) / 16;
+    if (nblocks > kSplitCounters || (size_t)nblocks * ks * 256 > kSplitWorkspaceFloats) return fail(10);
+  }
   return true;
 }
 
@@ -391,10 +450,19 @@ int launch_gemv_mfma(const Problem& p, const tlhip_kernel_config_t& c, hipStream
   a.cpg_shift = p.format == TLHIP_FMT_INT8_ROW ? 0 : __builtin_ctz((unsigned)(p.group_size / cw));
   a.groups_per_row = p.format == TLHIP_FMT_INT8_ROW ? 0 : (int)(p.k / p.group_size);
   a.iters = a.nchunks / 4;
+  a.ks = c.p3 < 1 ? 1 : c.p3;
+  a.ks_shift = __builtin_ctz((unsigned)a.ks);
+  a.slice_iters = a.iters / a.ks;
   a.kw = c.p2 == 0 ? waves : c.p2;
   a.kw_shift = __builtin_ctz((unsigned)a.kw);
   a.blocks_per_wg = waves / a.kw;
-  a.nsteps = (a.iters + a.kw * unroll - 1) / (a.kw * unroll);
+  a.nsteps = (a.slice_iters + a.kw * unroll - 1) / (a.kw * unroll);
+  a.workspace = nullptr;
+  a.counters = nullptr;
+  if (a.ks > 1) {
+    const int rc = split_workspace(stream, &a.workspace, &a.counters);
+    if (rc) return rc;
+  }
   a.nblocks = (int)((p.n + 15) / 16);
   a.nwgblocks = (a.nblocks + a.blocks_per_wg - 1) / a.blocks_per_wg;
   a.alpha = p.alpha;
@@ -402,14 +470,17 @@ int launch_gemv_mfma(const Problem& p, const tlhip_kernel_config_t& c, hipStream
   a.y_dtype = p.y_dtype;
   a.epi = p.epi;
   const size_t partial_bytes = (size_t)waves * 256 * sizeof(float);
-  const size_t lds_bytes = (size_t)a.m * (p.k * 2 + 16) + partial_bytes;
+  const size_t lds_bytes = (size_t)a.m * (p.k / a.ks * 2 + 16) + partial_bytes;
   const int threads = waves * 64;
   const int cus = device_cu_count();
   int per_cu = 2048 / threads;
   const int by_lds = (int)((160 * 1024) / lds_bytes);
   if (by_lds < per_cu) per_cu = by_lds < 1 ? 1 : by_lds;
-  int grid = a.nwgblocks < cus * per_cu ? a.nwgblocks : cus * per_cu;
-  if (grid < 1) grid = 1;
+  // resident workgroups only, in whole sets of ks; never more sets than row-block groups
+  int sets = cus * per_cu / a.ks;
+  if (sets > a.nwgblocks) sets = a.nwgblocks;
+  if (sets < 1) sets = 1;
+  const int grid = sets * a.ks;
   int rc;
   switch (p.format) {
     case TLHIP_FMT_INT4_GROUPED: rc = launch_mfma_u<TLHIP_FMT_INT4_GROUPED>(unroll, a, grid, threads, lds_bytes, stream); break;

@@ -7,6 +7,7 @@
 #include <cstring>
 #include <mutex>
 #include <string>
+#include <unordered_map>
 
 #include "common.h"
 
@@ -39,6 +40,59 @@ void clear_error() { g_error[0] = '\0'; }
 bool is_initialised() { return g_init; }
 
 hipStream_t resolve_stream(tlhip_stream_t s) { return s ? static_cast<hipStream_t>(s) : g_stream; }
+
+namespace {
+struct SplitWorkspace {
+  float* workspace;
+  int* counters;
+};
+std::mutex g_ws_mutex;
+std::unordered_map<hipStream_t, SplitWorkspace> g_workspaces;
+
+void free_workspaces() {
+  std::lock_guard<std::mutex> lock(g_ws_mutex);
+  for (auto& kv : g_workspaces) {
+    (void)hipFree(kv.second.workspace);
+    (void)hipFree(kv.second.counters);
+  }
+  g_workspaces.clear();
+}
+
+void free_workspace_of(hipStream_t stream) {
+  std::lock_guard<std::mutex> lock(g_ws_mutex);
+  auto it = g_workspaces.find(stream);
+  if (it == g_workspaces.end()) return;
+  (void)hipFree(it->second.workspace);
+  (void)hipFree(it->second.counters);
+  g_workspaces.erase(it);
+}
+}  // namespace
+
+int split_workspace(hipStream_t stream, float** workspace, int** counters) {
+  std::lock_guard<std::mutex> lock(g_ws_mutex);
+  auto it = g_workspaces.find(stream);
+  if (it == g_workspaces.end()) {
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    TLHIP_CHECK_HIP(hipStreamIsCapturing(stream, &status));
+    if (status != hipStreamCaptureStatusNone)
+      return set_error(TLHIP_ERR_STATE,
+                       "split-K workspace of this stream does not exist yet and cannot be created during "
+                       "capture: run the same call once on this stream before capturing");
+    SplitWorkspace w{nullptr, nullptr};
+    TLHIP_CHECK_HIP(hipMalloc((void**)&w.workspace, kSplitWorkspaceFloats * sizeof(float)));
+    hipError_t e = hipMalloc((void**)&w.counters, kSplitCounters * sizeof(int));
+    if (e == hipSuccess) e = hipMemset(w.counters, 0, kSplitCounters * sizeof(int));
+    if (e != hipSuccess) {
+      (void)hipFree(w.workspace);
+      if (w.counters) (void)hipFree(w.counters);
+      return set_error(TLHIP_ERR_DEVICE, "split-K counters: %s", hipGetErrorString(e));
+    }
+    it = g_workspaces.emplace(stream, w).first;
+  }
+  *workspace = it->second.workspace;
+  *counters = it->second.counters;
+  return TLHIP_OK;
+}
 
 int device_cu_count() { return g_init ? g_props.multiProcessorCount : 0; }
 
@@ -87,6 +141,7 @@ int tlhip_shutdown(void) {
   std::lock_guard<std::mutex> lock(g_mutex);
   if (!g_init) return TLHIP_OK;
   (void)hipStreamSynchronize(g_stream);
+  free_workspaces();
   (void)hipStreamDestroy(g_stream);
   g_stream = nullptr;
   g_init = false;
@@ -181,6 +236,8 @@ int tlhip_stream_create(tlhip_stream_t* out) {
 int tlhip_stream_destroy(tlhip_stream_t stream) {
   TLHIP_REQUIRE_INIT();
   if (!stream) return TLHIP_OK;
+  TLHIP_CHECK_HIP(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
+  free_workspace_of(static_cast<hipStream_t>(stream));
   TLHIP_CHECK_HIP(hipStreamDestroy(static_cast<hipStream_t>(stream)));
   return TLHIP_OK;
 }
