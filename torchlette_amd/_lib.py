@@ -13,7 +13,8 @@ import ctypes as C
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libtlhip.so")
+# TLHIP_LIBRARY names another build of the same library (e.g. one under test).
+LIB_PATH = os.environ.get("TLHIP_LIBRARY") or os.path.join(_HERE, "libtlhip.so")
 
 FMT_INT8_GROUPED, FMT_INT8_ROW, FMT_INT4_GROUPED = 0, 1, 2
 F32, F16 = 0, 1

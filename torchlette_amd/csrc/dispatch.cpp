@@ -116,10 +116,11 @@ tlhip_kernel_config_t default_config(const Problem& p) {
   // (below that the VALU kernel with its rows held in registers measures faster)
   if (p.m >= 5 && p.m <= 16) {
     // the fewest K slices across workgroups whose activations fit LDS (measured best)
-    for (int ks = 1; ks <= 16; ks *= 2) {
-      tlhip_kernel_config_t c = mfma_cfg(8, 2, p.n >= 32768 ? 1 : (ks > 1 ? 4 : 8), ks);
-      if (gemv_mfma_config_applicable(p, c, nullptr)) return c;
-    }
+    for (int ks = 1; ks <= 16; ks *= 2)
+      for (int unroll : {2, 1}) {
+        tlhip_kernel_config_t c = mfma_cfg(8, unroll, p.n >= 32768 ? 1 : (ks > 1 ? 4 : 8), ks);
+        if (gemv_mfma_config_applicable(p, c, nullptr)) return c;
+      }
   }
   // lanes per row: every lane busy for short rows; all chunks of a row in flight at once
   int lpr = 64;

@@ -49,7 +49,7 @@ struct MfmaArgs {
   int kw;             // waves that split a slice for one 16-row block (power of two)
   int kw_shift;
   int blocks_per_wg;  // 16-row blocks a workgroup works on at a time = waves / kw
-  int nsteps;         // batches (U iterations each) per row block per wave
+  int nsteps;         // batches (U consecutive iterations each) per row block per wave
   int nblocks;        // 16-row blocks
   int nwgblocks;      // ceil(nblocks / blocks_per_wg)
   float alpha;
@@ -110,7 +110,7 @@ __device__ __forceinline__ int x_unit(int t, int g, int m, int row_units) {
   return m * row_units + ku;
 }
 
-template <int FMT, int U>
+template <int FMT, int U, bool WIDE>
 __global__ __launch_bounds__(512) void gemv_mfma_kernel(const MfmaArgs a) {
   using Tr = MfmaTraits<FMT>;
   constexpr int STEPS = Tr::STEPS;
@@ -134,7 +134,6 @@ __global__ __launch_bounds__(512) void gemv_mfma_kernel(const MfmaArgs a) {
   const int wg_stride = gridDim.x >> a.ks_shift;
   int wgb = blockIdx.x >> a.ks_shift;
   const int it_begin = slice * a.slice_iters;
-  const int last_local = a.slice_iters - 1;  // slices are equal: ks divides the iterations
   constexpr int UNITS_PER_ITER = FMT == TLHIP_FMT_INT4_GROUPED ? 16 : 8;  // 16-byte x units per iteration
   const int slice_units = a.slice_iters * UNITS_PER_ITER;  // resident x units per row
   const int row_units = slice_units + 1;                    // padded LDS row stride
@@ -142,28 +141,48 @@ __global__ __launch_bounds__(512) void gemv_mfma_kernel(const MfmaArgs a) {
   const int k_units = a.k >> 3;                             // units per activation row in memory
   float* partial = (float*)(lds + (size_t)row_units * mrows);
 
-  // Raw loaded values only (no conversion at issue time, see gemv.hip).
+  // A wave's batch = U consecutive iterations; batch `kw_idx + step * kw` of the
+  // slice.  Raw loaded values only (no conversion at issue time, see gemv.hip).
+  // Scales: a separate 2-byte load per MFMA step made the kernel 2.5x slower
+  // than the weight stream alone (five memory instructions per kilobyte of
+  // weights), so with one scale per 32 weights (WIDE) the 4*U scales of a
+  // batch, contiguous in memory, come as U 8-byte or U/2 16-byte loads.
+  constexpr int NS = FMT == TLHIP_FMT_INT4_GROUPED ? 4 : 1;  // distinct scales per iteration at most
   struct Batch {
     u32x4 w[U];
-    uint16_t s[U][STEPS];
+    uint16_t s[U][NS];      // !WIDE
+    uint32_t sv[2 * U];     // WIDE: scale 4u+s in half (s & 1) of word 2u + s/2
   };
+  const int nbatches = a.slice_iters / U;  // U divides the iterations of a slice
 
   auto load_batch = [&](Batch& b, int wb, int step) {
     const int rb = min(wb * a.blocks_per_wg + bw_idx, a.nblocks - 1);
     const int64_t row = min((int64_t)rb * 16 + nl, a.n - 1);
     const u32x4* wrow = a.packed + row * a.nchunks;
     const uint16_t* srow = (const uint16_t*)a.scales + row * a.groups_per_row;
+    const int itb = it_begin + min(kw_idx + step * a.kw, nbatches - 1) * U;
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int it = it_begin + min(kw_idx + (step * U + u) * a.kw, last_local);
-      b.w[u] = __builtin_nontemporal_load(wrow + it * 4 + g);
-      if (GROUPED) {
+    for (int u = 0; u < U; ++u) b.w[u] = __builtin_nontemporal_load(wrow + (itb + u) * 4 + g);
+    if (WIDE) {
+      if (U == 1) {
+        const uint2 v = *(const uint2*)(srow + itb * 4);
+        b.sv[0] = v.x;
+        b.sv[1] = v.y;
+      } else {
 #pragma unroll
-        for (int s = 0; s < STEPS; ++s) {
-          // int4: step s is chunk 4*it+s; int8: both steps lie in chunks 4*it .. 4*it+3
-          const int chunk = FMT == TLHIP_FMT_INT4_GROUPED ? it * 4 + s : it * 4;
-          b.s[u][s] = srow[chunk >> a.cpg_shift];
+        for (int h = 0; h < U / 2; ++h) {
+          const u32x4 v = *(const u32x4*)(srow + itb * 4 + h * 8);  // 16-byte aligned: K % 256 == 0
+          b.sv[4 * h + 0] = v.x;
+          b.sv[4 * h + 1] = v.y;
+          b.sv[4 * h + 2] = v.z;
+          b.sv[4 * h + 3] = v.w;
         }
+      }
+    } else if (GROUPED) {
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+#pragma unroll
+        for (int s = 0; s < NS; ++s) b.s[u][s] = srow[((itb + u) * 4 + s) >> a.cpg_shift];
       }
     }
   };
@@ -171,11 +190,12 @@ __global__ __launch_bounds__(512) void gemv_mfma_kernel(const MfmaArgs a) {
   float4_t acc = {0.f, 0.f, 0.f, 0.f};
 
   auto compute_batch = [&](const Batch& b, int step) {
+    const int bidx = kw_idx + step * a.kw;
+    const bool valid = bidx < nbatches;  // wave-uniform
+    const int tlb = min(bidx, nbatches - 1) * U * STEPS;
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const int it_raw = kw_idx + (step * U + u) * a.kw;  // local to the slice
-      const bool valid = it_raw <= last_local;             // wave-uniform
-      const int tl = min(it_raw, last_local) * STEPS;
+      const int tl = tlb + u * STEPS;
       uint32_t w0 = b.w[u].x, w1 = b.w[u].y, w2 = b.w[u].z, w3 = b.w[u].w;
       half8_t bw[STEPS];
       if (FMT == TLHIP_FMT_INT4_GROUPED) {
@@ -197,20 +217,46 @@ __global__ __launch_bounds__(512) void gemv_mfma_kernel(const MfmaArgs a) {
           bw[s] = join8(h);
         }
       }
-      float4_t d[STEPS];
+      if (!GROUPED) {
+        // one scale per row, applied at the end: accumulate in the matrix core
+        if (valid) {
 #pragma unroll
-      for (int s = 0; s < STEPS; ++s) {
-        const u32x4 xa = lds[x_unit<FMT>(tl + s, g, ml, row_units)];
-        const float4_t zero = {0.f, 0.f, 0.f, 0.f};
-        d[s] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, xa), bw[s], zero, 0, 0, 0);
-      }
+          for (int s = 0; s < STEPS; ++s) {
+            const u32x4 xa = lds[x_unit<FMT>(tl + s, g, ml, row_units)];
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, xa), bw[s], acc, 0, 0, 0);
+          }
+        }
+      } else if (FMT == TLHIP_FMT_INT8_GROUPED) {
+        // both steps of an iteration lie in one scale group
+        const u32x4 xa0 = lds[x_unit<FMT>(tl, g, ml, row_units)];
+        const u32x4 xa1 = lds[x_unit<FMT>(tl + 1, g, ml, row_units)];
+        float4_t d = {0.f, 0.f, 0.f, 0.f};
+        d = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, xa0), bw[0], d, 0, 0, 0);
+        d = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, xa1), bw[1], d, 0, 0, 0);
+        const float sc = valid ? half_bits_to_float(b.s[u][0]) : 0.f;
 #pragma unroll
-      for (int s = 0; s < STEPS; ++s) {
-        const float sc = valid ? (GROUPED ? half_bits_to_float(b.s[u][s]) : 1.f) : 0.f;
-        acc[0] = fmaf(sc, d[s][0], acc[0]);
-        acc[1] = fmaf(sc, d[s][1], acc[1]);
-        acc[2] = fmaf(sc, d[s][2], acc[2]);
-        acc[3] = fmaf(sc, d[s][3], acc[3]);
+        for (int r = 0; r < 4; ++r) acc[r] = fmaf(sc, d[r], acc[r]);
+      } else {
+        float4_t d[STEPS];
+#pragma unroll
+        for (int s = 0; s < STEPS; ++s) {
+          const u32x4 xa = lds[x_unit<FMT>(tl + s, g, ml, row_units)];
+          const float4_t zero = {0.f, 0.f, 0.f, 0.f};
+          d[s] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, xa), bw[s], zero, 0, 0, 0);
+        }
+#pragma unroll
+        for (int s = 0; s < STEPS; ++s) {
+          uint16_t bits;
+          if (WIDE) {
+            const uint32_t wd = b.sv[2 * u + (s >> 1)];
+            bits = (uint16_t)((s & 1) ? (wd >> 16) : (wd & 0xffffu));
+          } else {
+            bits = b.s[u][s];
+          }
+          const float sc = valid ? half_bits_to_float(bits) : 0.f;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) acc[r] = fmaf(sc, d[s][r], acc[r]);
+        }
       }
     }
   };
@@ -388,6 +434,7 @@ bool gemv_mfma_config_applicable(const Problem& p, const tlhip_kernel_config_t& 
       "activations (M x K/slices f16) do not fit LDS",
       "K slices must be a power of two (1..16) that divides K/128 (int4) or K/64 (int8)",
       "K slices need more partial-tile workspace or counters than the library holds",
+      "iterations in flight must divide the 128-weight (int4) or 64-weight (int8) steps of a K slice",
   };
   auto fail = [&](int i) {
     if (why) *why = reasons[i];
@@ -408,6 +455,7 @@ bool gemv_mfma_config_applicable(const Problem& p, const tlhip_kernel_config_t& 
   const int64_t iters = p.k / kper;
   if (ks > 16 || (ks & (ks - 1)) != 0 || iters % ks != 0) return fail(9);
   if ((size_t)p.m * (p.k / ks * 2 + 16) + (size_t)c.p0 * 1024 > kXLdsBudget) return fail(8);
+  if ((iters / ks) % c.p1 != 0) return fail(11);
   if (ks > 1) {
     const int64_t nblocks = (p.n + 15) / 16;
     if (nblocks > kSplitCounters || (size_t)nblocks * ks * 256 > kSplitWorkspaceFloats) return fail(10);
@@ -415,13 +463,13 @@ bool gemv_mfma_config_applicable(const Problem& p, const tlhip_kernel_config_t& 
   return true;
 }
 
-template <int FMT>
+template <int FMT, bool WIDE>
 static int launch_mfma_u(int unroll, const MfmaArgs& a, int grid, int threads, size_t lds_bytes, hipStream_t stream) {
   const void* fn;
   switch (unroll) {
-    case 1: fn = (const void*)gemv_mfma_kernel<FMT, 1>; break;
-    case 2: fn = (const void*)gemv_mfma_kernel<FMT, 2>; break;
-    default: fn = (const void*)gemv_mfma_kernel<FMT, 4>; break;
+    case 1: fn = (const void*)gemv_mfma_kernel<FMT, 1, WIDE>; break;
+    case 2: fn = (const void*)gemv_mfma_kernel<FMT, 2, WIDE>; break;
+    default: fn = (const void*)gemv_mfma_kernel<FMT, 4, WIDE>; break;
   }
   if (lds_bytes > 64 * 1024)
     TLHIP_CHECK_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
@@ -456,7 +504,8 @@ int launch_gemv_mfma(const Problem& p, const tlhip_kernel_config_t& c, hipStream
   a.kw = c.p2 == 0 ? waves : c.p2;
   a.kw_shift = __builtin_ctz((unsigned)a.kw);
   a.blocks_per_wg = waves / a.kw;
-  a.nsteps = (a.slice_iters + a.kw * unroll - 1) / (a.kw * unroll);
+  const int nbatches = a.slice_iters / unroll;
+  a.nsteps = (nbatches + a.kw - 1) / a.kw;
   a.workspace = nullptr;
   a.counters = nullptr;
   if (a.ks > 1) {
@@ -483,9 +532,15 @@ int launch_gemv_mfma(const Problem& p, const tlhip_kernel_config_t& c, hipStream
   const int grid = sets * a.ks;
   int rc;
   switch (p.format) {
-    case TLHIP_FMT_INT4_GROUPED: rc = launch_mfma_u<TLHIP_FMT_INT4_GROUPED>(unroll, a, grid, threads, lds_bytes, stream); break;
-    case TLHIP_FMT_INT8_GROUPED: rc = launch_mfma_u<TLHIP_FMT_INT8_GROUPED>(unroll, a, grid, threads, lds_bytes, stream); break;
-    default: rc = launch_mfma_u<TLHIP_FMT_INT8_ROW>(unroll, a, grid, threads, lds_bytes, stream); break;
+    case TLHIP_FMT_INT4_GROUPED:
+      // one scale per 16-byte chunk and 16-byte aligned scale vectors: wide scale loads
+      if (p.group_size == 32 && (unroll == 1 || p.k % 256 == 0))
+        rc = launch_mfma_u<TLHIP_FMT_INT4_GROUPED, true>(unroll, a, grid, threads, lds_bytes, stream);
+      else
+        rc = launch_mfma_u<TLHIP_FMT_INT4_GROUPED, false>(unroll, a, grid, threads, lds_bytes, stream);
+      break;
+    case TLHIP_FMT_INT8_GROUPED: rc = launch_mfma_u<TLHIP_FMT_INT8_GROUPED, false>(unroll, a, grid, threads, lds_bytes, stream); break;
+    default: rc = launch_mfma_u<TLHIP_FMT_INT8_ROW, false>(unroll, a, grid, threads, lds_bytes, stream); break;
   }
   if (rc) return rc;
   TLHIP_CHECK_HIP(hipGetLastError());
