@@ -148,9 +148,9 @@ std::vector<tlhip_kernel_config_t> candidates(const Problem& p) {
             }
   }
   if (p.m <= 16) {
-    for (int waves : {4, 8})
+    for (int waves : {4, 8, 16})
       for (int unroll : {1, 2, 4})
-        for (int kw : {1, 2, 4, 8})
+        for (int kw : {1, 2, 4, 8, 16})
           for (int ks : {1, 2, 4, 8}) {
             if (kw > waves) continue;
             tlhip_kernel_config_t c = mfma_cfg(waves, unroll, kw, ks);

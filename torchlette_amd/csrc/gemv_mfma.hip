@@ -110,8 +110,8 @@ __device__ __forceinline__ int x_unit(int t, int g, int m, int row_units) {
   return m * row_units + ku;
 }
 
-template <int FMT, int U, bool WIDE>
-__global__ __launch_bounds__(512) void gemv_mfma_kernel(const MfmaArgs a) {
+template <int FMT, int U, bool WIDE, int MAXT>
+__global__ __launch_bounds__(MAXT) void gemv_mfma_kernel(const MfmaArgs a) {
   using Tr = MfmaTraits<FMT>;
   constexpr int STEPS = Tr::STEPS;
   constexpr bool GROUPED = (FMT != TLHIP_FMT_INT8_ROW);
@@ -419,12 +419,12 @@ __global__ __launch_bounds__(512) void gemv_mfma_kernel(const MfmaArgs a) {
 
 }  // namespace
 
-static constexpr size_t kXLdsBudget = 144 * 1024;
+static constexpr size_t kXLdsBudget = 160 * 1024;
 
 bool gemv_mfma_config_applicable(const Problem& p, const tlhip_kernel_config_t& c, const char** why) {
   static const char* reasons[] = {
       "not the gemv_mfma variant",
-      "waves per workgroup must be 4 or 8",
+      "waves per workgroup must be 4, 8 or 16 (16: at most two iterations in flight)",
       "activations must be f16",
       "M must be 1..16",
       "K must be a multiple of 128 (int4) or 64 (int8)",
@@ -441,7 +441,8 @@ bool gemv_mfma_config_applicable(const Problem& p, const tlhip_kernel_config_t& 
     return false;
   };
   if (c.variant != VARIANT_GEMV_MFMA) return fail(0);
-  if (c.p0 != 4 && c.p0 != 8) return fail(1);
+  if (c.p0 != 4 && c.p0 != 8 && c.p0 != 16) return fail(1);
+  if (c.p0 == 16 && c.p1 > 2) return fail(1);
   if (p.x_dtype != TLHIP_F16) return fail(2);
   if (p.m < 1 || p.m > 16) return fail(3);
   const int kper = p.format == TLHIP_FMT_INT4_GROUPED ? 128 : 64;
@@ -465,11 +466,16 @@ bool gemv_mfma_config_applicable(const Problem& p, const tlhip_kernel_config_t& 
 
 template <int FMT, bool WIDE>
 static int launch_mfma_u(int unroll, const MfmaArgs& a, int grid, int threads, size_t lds_bytes, hipStream_t stream) {
+  // 16 waves leave 128 registers per lane: enough for one or two iterations in flight
   const void* fn;
-  switch (unroll) {
-    case 1: fn = (const void*)gemv_mfma_kernel<FMT, 1, WIDE>; break;
-    case 2: fn = (const void*)gemv_mfma_kernel<FMT, 2, WIDE>; break;
-    default: fn = (const void*)gemv_mfma_kernel<FMT, 4, WIDE>; break;
+  if (threads > 512) {
+    fn = unroll == 1 ? (const void*)gemv_mfma_kernel<FMT, 1, WIDE, 1024> : (const void*)gemv_mfma_kernel<FMT, 2, WIDE, 1024>;
+  } else {
+    switch (unroll) {
+      case 1: fn = (const void*)gemv_mfma_kernel<FMT, 1, WIDE, 512>; break;
+      case 2: fn = (const void*)gemv_mfma_kernel<FMT, 2, WIDE, 512>; break;
+      default: fn = (const void*)gemv_mfma_kernel<FMT, 4, WIDE, 512>; break;
+    }
   }
   if (lds_bytes > 64 * 1024)
     TLHIP_CHECK_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
