@@ -215,7 +215,10 @@ int tlhip_hbm_read_probe(const void* ptr, size_t bytes, void* sink4, tlhip_strea
  * dispatch.ts:60-207, 405-578) ---- */
 
 /* A launch configuration.  variant 0 = "gemv" (VALU dot), 1 = "gemv_mfma"
- * (skinny MFMA), 2 = "tiled" (prefill MFMA GEMM).  Unused fields are 0. */
+ * (skinny MFMA), 2 = "tiled" (prefill MFMA GEMM, both operands through LDS),
+ * 3 = "tiled_direct" (prefill MFMA GEMM for int4, weights dequantised in
+ * registers; fields as "tiled" with tile K 128 and 2x4 or 4x2 waves).
+ * Unused fields are 0. */
 typedef struct {
   int32_t variant;
   int32_t p0; /* gemv: lanes per row (16/32/64)   gemv_mfma: waves per workgroup   tiled: tile M */

@@ -53,6 +53,44 @@ def test_every_tile_config_ragged_shapes(be, fmt, g, bm, bn):
     assert rel_l2(got, want) <= REL_L2_TOL, rel_l2(got, want)
 
 
+DIRECT_TILES = [(256, 256, 2, 4), (256, 128, 2, 4), (128, 256, 2, 4), (256, 128, 4, 2), (128, 128, 2, 2), (256, 256, 2, 2)]
+
+
+@pytest.mark.parametrize("bm,bn,wm,wn", DIRECT_TILES)
+@pytest.mark.parametrize("g,m,n,k", [(32, 300, 333, 256), (128, 300, 333, 384), (32, 520, 777, 1152), (64, 64, 256, 128)])
+def test_direct_weight_operand_gemm_every_tile_ragged_shapes(be, g, m, n, k, bm, bn, wm, wn):
+    """The int4 GEMM whose weights are dequantised in registers (no LDS for W):
+    ragged M and N, odd and even numbers of 128-k steps, bias + activation fused."""
+    rng = np.random.default_rng(bm + bn + wm + g + k)
+    packed, scales, deq = make_weight("int4-grouped", n, k, g, rng)
+    x = make_x(m, k, "f16", rng, std=0.5)
+    bias = rng.standard_normal(n).astype(np.float32)
+    cfg = L.KernelConfig.of(3, bm, bn, 128, wm, wn)
+    before = T.getQuantGemmDispatchCount()
+    got = run(be, "int4-grouped", packed, scales, n, k, g, x, "f32", bias=bias, act="gelu", config=cfg)
+    assert T.getQuantGemmDispatchCount() == before + 1
+    want = O.linear(x.astype(np.float32), deq, bias, "gelu", threads=8)
+    assert got.shape == (m, n) and got.dtype == np.float32
+    assert rel_l2(got, want) <= REL_L2_TOL, rel_l2(got, want)
+    # and against the LDS-staged GEMM: same roundings of the weights, f32 accumulate
+    other = run(be, "int4-grouped", packed, scales, n, k, g, x, "f32", bias=bias, act="gelu", config=tiled(128, 128))
+    assert rel_l2(got, other) <= 2e-6
+
+
+def test_direct_gemm_rejects_what_it_does_not_cover(be):
+    rng = np.random.default_rng(3)
+    x = be.ops.tensorFromArray(make_x(32, 192, "f16", rng), [32, 192], "f16")
+    packed, scales, _ = make_weight("int4-grouped", 64, 192, 32, rng)
+    w = be.createQuantizedWeight(packed, scales, 64, 192, T.resolveWeightFormat("int4-32", "f32"))
+    with pytest.raises(L.TlhipError, match="K must be a multiple of 128"):
+        be.linear(x, w, config=L.KernelConfig.of(3, 256, 256, 128, 2, 4))
+    packed8, scales8, _ = make_weight("int8-row", 64, 256, 0, rng)
+    w8 = be.createQuantizedWeight(packed8, scales8, 64, 256, T.resolveWeightFormat("int8-row", "f32"))
+    x8 = be.ops.tensorFromArray(make_x(32, 256, "f16", rng), [32, 256], "f16")
+    with pytest.raises(L.TlhipError, match="int4-grouped"):
+        be.linear(x8, w8, config=L.KernelConfig.of(3, 256, 256, 128, 2, 4))
+
+
 @pytest.mark.parametrize("m,n,k", [(17, 128, 64), (64, 64, 128), (100, 512, 1024), (1000, 256, 2048), (33, 1000, 4096)])
 def test_default_route_for_m_above_16_is_the_gemm(be, m, n, k):
     rng = np.random.default_rng(m + n + k)

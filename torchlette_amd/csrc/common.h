@@ -70,6 +70,8 @@ bool gemv_mfma_config_applicable(const Problem& p, const tlhip_kernel_config_t& 
 int launch_gemv_mfma(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t stream);
 bool gemm_config_applicable(const Problem& p, const tlhip_kernel_config_t& c, const char** why);
 int launch_gemm(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t stream);
+bool gemm_direct_config_applicable(const Problem& p, const tlhip_kernel_config_t& c, const char** why);
+int launch_gemm_direct(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t stream);
 
 // Device scratch for kernels that combine partial results of several workgroups:
 // `kSplitWorkspaceFloats` floats plus `kSplitCounters` arrival counters that are
@@ -86,6 +88,6 @@ void count_gemm_dispatch();
 void count_dequant_dispatch();
 void count_autotune_run();
 
-enum { VARIANT_GEMV = 0, VARIANT_GEMV_MFMA = 1, VARIANT_TILED = 2 };
+enum { VARIANT_GEMV = 0, VARIANT_GEMV_MFMA = 1, VARIANT_TILED = 2, VARIANT_TILED_DIRECT = 3 };
 
 }  // namespace tlhip

@@ -92,7 +92,14 @@ tlhip_kernel_config_t tiled_cfg(int tm, int tn, int tk, int wm, int wn) {
   return c;
 }
 
+tlhip_kernel_config_t direct_cfg(int tm, int tn, int wm, int wn) {
+  tlhip_kernel_config_t c = tiled_cfg(tm, tn, 128, wm, wn);
+  c.variant = VARIANT_TILED_DIRECT;
+  return c;
+}
+
 bool config_applicable(const Problem& p, const tlhip_kernel_config_t& c, const char** why) {
+  if (c.variant == VARIANT_TILED_DIRECT) return gemm_direct_config_applicable(p, c, why);
   if (c.variant == VARIANT_TILED) return gemm_config_applicable(p, c, why);
   if (c.variant == VARIANT_GEMV_MFMA) return gemv_mfma_config_applicable(p, c, why);
   return gemv_config_applicable(p, c, why);
@@ -166,6 +173,11 @@ std::vector<tlhip_kernel_config_t> candidates(const Problem& p) {
       tlhip_kernel_config_t c = tiled_cfg(t[0], t[1], t[2], t[3], t[4]);
       if (gemm_config_applicable(p, c, nullptr)) out.push_back(c);
     }
+    static const int direct[][4] = {{256, 256, 2, 4}, {256, 128, 2, 4}, {128, 256, 2, 4}, {256, 128, 4, 2}, {128, 128, 2, 2}, {256, 256, 2, 2}};
+    for (auto& t : direct) {
+      tlhip_kernel_config_t c = direct_cfg(t[0], t[1], t[2], t[3]);
+      if (gemm_direct_config_applicable(p, c, nullptr)) out.push_back(c);
+    }
   }
   return out;
 }
@@ -180,6 +192,7 @@ tlhip_kernel_config_t select_config(const Problem& p) {
 }
 
 int run_config(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t stream) {
+  if (c.variant == VARIANT_TILED_DIRECT) return launch_gemm_direct(p, c, stream);
   if (c.variant == VARIANT_TILED) return launch_gemm(p, c, stream);
   if (c.variant == VARIANT_GEMV_MFMA) return launch_gemv_mfma(p, c, stream);
   return launch_gemv(p, c, stream);
@@ -338,7 +351,7 @@ int tlhip_gemv(const tlhip_qweight_t* w, const void* x, int x_dtype, int64_t m, 
   if (rc) return rc;
   if (m > 16) return set_error(TLHIP_ERR_INVALID, "gemv: M=%lld above 16; use tlhip_gemm_prefill", (long long)m);
   tlhip_kernel_config_t c = select_config(p);
-  if (c.variant == VARIANT_TILED) c = default_config(p);
+  if (c.variant == VARIANT_TILED || c.variant == VARIANT_TILED_DIRECT) c = default_config(p);
   return run_config(p, c, resolve_stream(stream));
 }
 
@@ -350,17 +363,17 @@ int tlhip_gemm_prefill(const tlhip_qweight_t* w, const void* x, int x_dtype, int
   if (rc) return rc;
   if (x_dtype != TLHIP_F16) return set_error(TLHIP_ERR_INVALID, "gemm_prefill: activations must be f16");
   tlhip_kernel_config_t c = select_config(p);
-  if (c.variant != VARIANT_TILED) {
+  if (c.variant != VARIANT_TILED && c.variant != VARIANT_TILED_DIRECT) {
     c = tiled_cfg(p.m >= 128 ? 128 : 64, 128, 64, 2, 2);
     const char* why = nullptr;
     if (!gemm_config_applicable(p, c, &why))
       return set_error(TLHIP_ERR_INVALID, "gemm_prefill: shape not supported: %s", why ? why : "?");
   }
-  return launch_gemm(p, c, resolve_stream(stream));
+  return run_config(p, c, resolve_stream(stream));
 }
 
 static int matmul_with(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t stream) {
-  if (c.variant == VARIANT_TILED) return launch_gemm(p, c, stream);
+  if (c.variant == VARIANT_TILED || c.variant == VARIANT_TILED_DIRECT) return run_config(p, c, stream);
   if (p.m <= 16) return run_config(p, c, stream);
   // f32 activations (or a shape the tiled kernel rejects) above 16 rows: GEMV
   // passes of 16 rows.  Declared, slow: every pass streams the weights again.

@@ -1,0 +1,117 @@
+// Pieces shared by the two prefill GEMM kernels: the workgroup -> tile map and
+// the per-wave epilogue.
+#pragma once
+#include "device_utils.h"
+
+namespace tlhip {
+
+// Workgroup ids are dealt round-robin to the 8 XCDs (each with its own L2), and
+// the workgroups of one XCD start in id order.  A run of 2^sb_shift (at most 32 =
+// the CUs of an XCD) consecutive workgroups of an XCD takes one "super-block" of
+// 2^gm_shift x 2^gn_shift tiles, so the tiles that run together on an XCD share
+// their X row blocks and W column blocks through that XCD's L2: the L2 fill per
+// K step is (GM * BM + GN * BN) rows instead of (32 * BM + BN).
+struct TileMap {
+  int tiles_m, tiles_n;
+  int gm_shift, gn_shift;  // super-block = 2^gm_shift x 2^gn_shift tiles
+  int sbm;                 // super-blocks along M
+  int nsb;                 // super-blocks in all
+};
+
+inline TileMap make_tile_map(int tiles_m, int tiles_n, int* grid) {
+  TileMap t;
+  t.tiles_m = tiles_m;
+  t.tiles_n = tiles_n;
+  const long total = (long)tiles_m * tiles_n;
+  // as large as 32 tiles, but at least 16 super-blocks so that every XCD gets work
+  int s_shift = 5;
+  while (s_shift > 0 && (total >> s_shift) < 16) --s_shift;
+  int gm_shift = 0;
+  while (gm_shift < 3 && gm_shift < s_shift && (2 << gm_shift) <= tiles_m) ++gm_shift;
+  t.gm_shift = gm_shift;
+  t.gn_shift = s_shift - gm_shift;
+  const int gm = 1 << t.gm_shift, gn = 1 << t.gn_shift;
+  t.sbm = (tiles_m + gm - 1) / gm;
+  const int sbn = (tiles_n + gn - 1) / gn;
+  t.nsb = t.sbm * sbn;
+  *grid = ((t.nsb + 7) / 8) * 8 << s_shift;
+  return t;
+}
+
+// false: this workgroup has no tile (padding of the last super-blocks).
+__device__ __forceinline__ bool tile_of(const TileMap& t, int id, int& tm, int& tn) {
+  const int s_shift = t.gm_shift + t.gn_shift;
+  const int xcd = id & 7, local = id >> 3;
+  const int sb = (local >> s_shift) * 8 + xcd;
+  const int in = local & ((1 << s_shift) - 1);
+  const int sb_n = sb / t.sbm, sb_m = sb - sb_n * t.sbm;
+  tm = (sb_m << t.gm_shift) + (in & ((1 << t.gm_shift) - 1));
+  tn = (sb_n << t.gn_shift) + (in >> t.gm_shift);
+  return sb < t.nsb && tm < t.tiles_m && tn < t.tiles_n;
+}
+
+struct OutArgs {
+  void* y;
+  int y_dtype;
+  int vec_ok;  // N % 8 == 0 and y 16-byte aligned: rows can be stored 8 columns at a time
+  int m, n;
+  float alpha;
+  DevEpilogue epi;
+};
+
+// Epilogue of one 32-row block of a wave: TN accumulator tiles of
+// v_mfma_f32_32x32x16 side by side (32 x 32*TN outputs).  The accumulator layout
+// (lane l: column l%32, rows 8*(r/4) + 4*(l/32) + r%4) would give 64-byte row
+// pieces per store; instead the block goes through a private LDS patch and every
+// lane then owns 8 consecutive columns of one row: acc*alpha -> ops in order
+// (bias indexed by n, unary) -> cast, stored as one 16-byte (f16) or two 16-byte
+// (f32) pieces, whole 128-byte lines per row for f16 and TN = 2.
+// `patch` holds 32 * (32*TN + 4) floats and belongs to this wave alone.
+template <int TN>
+__device__ __forceinline__ void wave_epilogue(float* patch, const float16_t (&acc)[TN], int lane, int row0,
+                                              int col0, const OutArgs& o) {
+  constexpr int PW = TN * 32 + 4;
+  constexpr int LPR = TN * 4;     // lanes per row, 8 columns each
+  constexpr int RPP = 64 / LPR;   // rows per pass
+  const int lrow = lane & 31, lk = lane >> 5;
+#pragma unroll
+  for (int j = 0; j < TN; ++j)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) patch[(8 * (r >> 2) + 4 * lk + (r & 3)) * PW + j * 32 + lrow] = acc[j][r];
+  __builtin_amdgcn_s_waitcnt(0xc07f);  // this wave's LDS writes have landed (lgkmcnt(0))
+  const int rr0 = lane / LPR, cc = (lane % LPR) * 8;
+  const int col = col0 + cc;
+  const bool vec = o.vec_ok && col + 8 <= o.n;
+#pragma unroll 1
+  for (int p = 0; p < 32 / RPP; ++p) {
+    const int rr = p * RPP + rr0;
+    const int row = row0 + rr;
+    const float4_t a = *(const float4_t*)(patch + rr * PW + cc);
+    const float4_t b = *(const float4_t*)(patch + rr * PW + cc + 4);
+    float v[8] = {a[0], a[1], a[2], a[3], b[0], b[1], b[2], b[3]};
+    if (row < o.m) {
+      if (vec) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = apply_epilogue(o.epi, v[e] * o.alpha, col + e);
+        const int64_t idx = (int64_t)row * o.n + col;
+        if (o.y_dtype == TLHIP_F16) {
+          half8_t h;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) h[e] = (_Float16)v[e];
+          *(half8_t*)((_Float16*)o.y + idx) = h;
+        } else {
+          float* dst = (float*)o.y + idx;
+          *(float4_t*)dst = (float4_t){v[0], v[1], v[2], v[3]};
+          *(float4_t*)(dst + 4) = (float4_t){v[4], v[5], v[6], v[7]};
+        }
+      } else {
+        for (int e = 0; e < 8; ++e)
+          if (col + e < o.n)
+            store_out(o.y, o.y_dtype, (int64_t)row * o.n + col + e, apply_epilogue(o.epi, v[e] * o.alpha, col + e));
+      }
+    }
+  }
+  __builtin_amdgcn_s_waitcnt(0xc07f);  // reads done before the patch is overwritten
+}
+
+}  // namespace tlhip
