@@ -45,6 +45,11 @@ def test_every_tile_config_ragged_shapes(be, fmt, g, bm, bn):
     m, n, k = 300, 333, 256          # neither M nor N a multiple of any tile
     packed, scales, deq = make_weight(fmt, n, k, g, rng)
     x = make_x(m, k, "f16", rng, std=0.5)
+    if (bm, bn) == (256, 256) and fmt != "int4-grouped":
+        # not built: the int8 dequantisation would spill registers at this tile
+        with pytest.raises(L.TlhipError, match="config not applicable"):
+            run(be, fmt, packed, scales, n, k, g, x, "f32", config=tiled(bm, bn))
+        return
     before = T.getQuantGemmDispatchCount()
     got = run(be, fmt, packed, scales, n, k, g, x, "f32", config=tiled(bm, bn))
     assert T.getQuantGemmDispatchCount() == before + 1

@@ -86,16 +86,25 @@ __device__ __forceinline__ void store_out(void* y, int y_dtype, int64_t idx, flo
 // (0x6400) gives the f16 value 1024+q+8 (or 1024+16*(q+8) for a nibble at bit
 // 4), from which q is recovered exactly by one packed add or fma.
 // Output order: pairs (k0,k4) (k1,k5) (k2,k6) (k3,k7).
+// (a & mask) | orv as the single instruction it is.  Left to itself the compiler
+// emits a separate AND and OR for half of the uses (a VOP3 instruction takes no
+// 32-bit literal, and it prefers literals to keeping the constants in registers).
+__device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t mask, uint32_t orv) {
+  uint32_t d;
+  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(d) : "v"(a), "s"(mask), "v"(orv));
+  return d;
+}
+
 __device__ __forceinline__ void unpack_int4_word(uint32_t w, half2_t out[4]) {
   const uint32_t t = w ^ 0x88888888u;
   const uint32_t lo = t, hi = t >> 8;
   const half2_t sub_lo = {(_Float16)-1032.f, (_Float16)-1032.f};  // -(1024 + 8)
   const half2_t mul_hi = {(_Float16)0.0625f, (_Float16)0.0625f};  // 1/16
   const half2_t sub_hi = {(_Float16)-72.f, (_Float16)-72.f};      // -(1024/16 + 8)
-  const uint32_t a0 = (lo & 0x000f000fu) | 0x64006400u;
-  const uint32_t a1 = (lo & 0x00f000f0u) | 0x64006400u;
-  const uint32_t a2 = (hi & 0x000f000fu) | 0x64006400u;
-  const uint32_t a3 = (hi & 0x00f000f0u) | 0x64006400u;
+  const uint32_t a0 = and_or(lo, 0x000f000fu, 0x64006400u);
+  const uint32_t a1 = and_or(lo, 0x00f000f0u, 0x64006400u);
+  const uint32_t a2 = and_or(hi, 0x000f000fu, 0x64006400u);
+  const uint32_t a3 = and_or(hi, 0x00f000f0u, 0x64006400u);
   out[0] = __builtin_bit_cast(half2_t, a0) + sub_lo;
   out[1] = __builtin_bit_cast(half2_t, a1) * mul_hi + sub_hi;
   out[2] = __builtin_bit_cast(half2_t, a2) + sub_lo;

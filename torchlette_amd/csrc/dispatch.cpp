@@ -98,6 +98,7 @@ tlhip_kernel_config_t direct_cfg(int tm, int tn, int wm, int wn) {
   return c;
 }
 
+
 bool config_applicable(const Problem& p, const tlhip_kernel_config_t& c, const char** why) {
   if (c.variant == VARIANT_TILED_DIRECT) return gemm_direct_config_applicable(p, c, why);
   if (c.variant == VARIANT_TILED) return gemm_config_applicable(p, c, why);
@@ -110,8 +111,15 @@ tlhip_kernel_config_t default_config(const Problem& p) {
   const int cw = p.format == TLHIP_FMT_INT4_GROUPED ? 32 : 16;
   const int64_t nchunks = p.k / cw;
   if (p.m > 16 && p.x_dtype == TLHIP_F16) {
-    // largest tile that still gives every CU a workgroup
     const int cus = device_cu_count() > 0 ? device_cu_count() : 256;
+    // int4: the kernel that keeps the weights packed up to the operand registers;
+    // 256 x 256 tiles once they fill the chip twice over, else 256 x 128
+    {
+      const int64_t t256 = ((p.m + 255) / 256) * ((p.n + 255) / 256);
+      tlhip_kernel_config_t c = t256 >= 2 * cus ? direct_cfg(256, 256, 2, 4) : direct_cfg(256, 128, 2, 4);
+      if (gemm_direct_config_applicable(p, c, nullptr)) return c;
+    }
+    // largest tile that still gives every CU a workgroup
     static const int tiles[][2] = {{256, 256}, {256, 128}, {128, 128}, {64, 128}};
     for (auto& t : tiles) {
       const int64_t wgs = ((p.m + t[0] - 1) / t[0]) * ((p.n + t[1] - 1) / t[1]);

@@ -1,24 +1,33 @@
-// Prefill GEMM over packed int4 weights, second form: the weight operand never
-// touches LDS.  Y[M,N] = epilogue(alpha * X[M,K] * W[N,K]^T); same contract and
-// reference route as gemm_prefill.hip (src/backend/webgpu/ops/matmul-ops.ts:163-181;
+// Prefill GEMM over packed int4 weights, second form: the weights stay PACKED
+// until they are in the operand registers.  Y[M,N] = epilogue(alpha * X[M,K] *
+// W[N,K]^T); same contract and reference route as gemm_prefill.hip
+// (src/backend/webgpu/ops/matmul-ops.ts:163-181;
 // src/schedule/matmul-skeleton.ts:738-966).
 //
-// Why a second form: with both operands staged through LDS a 4-wave tile moves
-// about 1 KB of LDS traffic per MFMA and the kernel is bound by LDS, not by the
-// matrix cores.  Here
+// Why a second form: with the dequantised f16 weights staged through LDS a tile
+// moves about 1 KB of LDS traffic per MFMA and the kernel is bound by LDS, not
+// by the matrix cores.  Here, per 128-k step of a BM x BN tile,
+//   * the packed weights (BN rows x 64 bytes) go global -> registers -> LDS as
+//     they are, 16 bytes per lane with four consecutive lanes on one row, so the
+//     global loads are coalesced (a lane loading its own MFMA operand row made
+//     64 scattered 16-byte requests per instruction and cost a quarter of the
+//     kernel's time); LDS holds them with the chunk position XOR-swizzled by
+//     the row so that the operand reads spread over all banks;
 //   * a lane of the B operand of v_mfma_f32_32x32x16_f16 (weight row n, k half
-//     lk) loads ITS packed weights straight from global memory — 32 contiguous
-//     bytes (two 16-byte chunks = 64 weights) per 128-k step, plus the two group
-//     scales — and dequantises them in registers, one 32-bit word (8 weights,
-//     one MFMA) at a time: exact integers in f16, times the scale, one rounding;
+//     lk) reads ITS two 16-byte chunks (64 weights) from LDS and dequantises them
+//     in registers, one 32-bit word (8 weights, one MFMA) at a time: exact
+//     integers in f16, times the group scale (loaded by the lane itself, 4
+//     bytes per step), one rounding.  LDS traffic for W is a quarter of what
+//     dequantised f16 would be;
 //   * the k order inside a step is chosen to fit that: MFMA (c, w) of a step
 //     covers k = 64*lk + 32*c + 8*w + (0..7) for lane half lk, and the A operand
 //     reads the activations of exactly those k from LDS;
-//   * only X goes through LDS (global -> registers -> LDS in two halves per step,
-//     double buffered, one LDS-only barrier per 128-k step), written with the
-//     (0,4,1,5,2,6,3,7) order the int4 unpack produces;
-//   * 8 waves (2 per SIMD) per workgroup, so one wave's dequantisation and LDS
-//     reads overlap the other's MFMAs.
+//   * X goes global -> registers -> LDS in parts spread over the step, written
+//     with the (0,4,1,5,2,6,3,7) order the int4 unpack produces, rows padded to
+//     272 bytes, double buffered; the W buffer is single (a second LDS-only
+//     barrier in the middle of the step frees it), which keeps a 256 x 256 tile
+//     within the 160 KB of LDS;
+//   * 8 waves (2 per SIMD) per workgroup.
 // MFMA-bound by design: per MFMA a wave reads 1 KB / TN from LDS and spends
 // 14 / TM VALU instructions on dequantisation.
 #include "gemm_common.h"
@@ -27,7 +36,7 @@ namespace tlhip {
 namespace {
 
 constexpr int DK = 128;            // k per step
-constexpr int DROW_UNITS = 17;     // LDS row: 128 f16 = 16 units + 1 unit of padding
+constexpr int DROW_UNITS = 17;     // LDS row of X: 128 f16 = 16 units + 1 unit of padding
 
 struct DirectArgs {
   const uint8_t* packed;  // row stride K/2 bytes
@@ -50,9 +59,11 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_direct_kernel(const DirectA
   constexpr int THREADS = WM * WN * 64;
   constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
   constexpr int X_LOADS = BM * 16 / THREADS;  // 16-byte units of the X tile per thread per step
-  static_assert(BM * 16 % THREADS == 0, "X tile must divide over the threads");
-  constexpr int STAGE_UNITS = BM * DROW_UNITS;
-  extern __shared__ u32x4 lds[];
+  constexpr int W_LOADS = BN * 4 / THREADS;   // 16-byte chunks of the W tile per thread per step
+  static_assert(BM * 16 % THREADS == 0 && BN * 4 % THREADS == 0, "tiles must divide over the threads");
+  constexpr int X_UNITS = BM * DROW_UNITS;
+  extern __shared__ u32x4 lds[];  // X buffer 0, X buffer 1, W buffer
+  u32x4* const lds_w = lds + 2 * X_UNITS;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -64,57 +75,70 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_direct_kernel(const DirectA
   if (!tile_of(a.map, blockIdx.x, tm_idx, tn_idx)) return;  // padding of the tile map (whole workgroup)
   const int m0 = tm_idx * BM, n0 = tn_idx * BN;
 
-  // The lane's weight rows: 64 bytes of a row per step, this lane takes bytes 32*lk .. 32*lk+31.
-  const uint8_t* wptr[TN];
+  // ---- W: global -> registers -> LDS, packed --------------------------------
+  // chunk q = tid + i*THREADS of the tile: row q/4, chunk q%4 of the step's 64 bytes
+  u32x4 wr[W_LOADS];
+  auto load_w = [&](int step) {
+    const int st = min(step, a.ksteps - 1);  // past the end: a harmless reload of the last step
+#pragma unroll
+    for (int i = 0; i < W_LOADS; ++i) {
+      const int q = tid + i * THREADS;
+      const int row = min(n0 + (q >> 2), a.n - 1);
+      wr[i] = *(const u32x4*)(a.packed + (size_t)row * a.w_row_bytes + (size_t)st * 64 + (q & 3) * 16);
+    }
+  };
+  auto store_w = [&]() {
+    u32x4* ws = lds_w;
+#pragma unroll
+    for (int i = 0; i < W_LOADS; ++i) {
+      const int q = tid + i * THREADS;
+      const int r = q >> 2;
+      ws[r * 4 + ((q & 3) ^ ((r >> 2) & 3))] = wr[i];
+    }
+  };
+  // The lane's scales: raw bits, two stages (this step, next step).
   const uint16_t* sptr[TN];
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
     const int row = min(n0 + (wn * TN + j) * 32 + lrow, a.n - 1);
-    wptr[j] = a.packed + (size_t)row * a.w_row_bytes + lk * 32;
     sptr[j] = a.scales + (size_t)row * a.groups_per_row;
   }
-
-  // Raw loaded values only; nothing is converted at issue time.
-  struct BStage {
-    u32x4 w[TN][2];
+  struct Scales {
     uint32_t s[TN][2];  // G32: s[j][0] holds both scales; else one 16-bit scale each
   };
-  auto load_b = [&](int step, BStage& b) {
-    const int st = min(step, a.ksteps - 1);  // past the end: a harmless reload of the last step
+  auto load_s = [&](int step, Scales& sc) {
+    const int st = min(step, a.ksteps - 1);
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
-      const u32x4* src = (const u32x4*)(wptr[j] + (size_t)st * 64);
-      b.w[j][0] = src[0];
-      b.w[j][1] = src[1];
       if (G32) {
-        b.s[j][0] = *(const uint32_t*)(sptr[j] + st * 4 + lk * 2);
+        sc.s[j][0] = *(const uint32_t*)(sptr[j] + st * 4 + lk * 2);
       } else {
         const int ch = st * 4 + lk * 2;
-        b.s[j][0] = sptr[j][ch >> a.cpg_shift];
-        b.s[j][1] = sptr[j][(ch + 1) >> a.cpg_shift];
+        sc.s[j][0] = sptr[j][ch >> a.cpg_shift];
+        sc.s[j][1] = sptr[j][(ch + 1) >> a.cpg_shift];
       }
     }
   };
-  // X goes through registers in two halves (units i < XH, then the rest), each
-  // loaded before one half of the step's MFMAs and stored to LDS after it: half
-  // the staging registers, and the loads still have a half step to arrive.
-  constexpr int XH = X_LOADS / 2;
-  static_assert(X_LOADS % 2 == 0, "X tile units per thread must be even");
+
+  // ---- X: global -> registers -> LDS in NXP parts per step ---------------------
+  constexpr int NXP = X_LOADS >= 4 ? 4 : 2;
+  constexpr int XH = X_LOADS / NXP;
+  static_assert(X_LOADS % NXP == 0, "X tile units per thread must divide into the staging parts");
   u32x4 xr[XH];
-  auto load_x = [&](int step, int half) {
+  auto load_x = [&](int step, int part) {
     const int k0 = min(step, a.ksteps - 1) * DK;
 #pragma unroll
     for (int i = 0; i < XH; ++i) {
-      const int u = tid + (half * XH + i) * THREADS;
+      const int u = tid + (part * XH + i) * THREADS;
       const int row = min(m0 + (u >> 4), a.m - 1);
       xr[i] = *(const u32x4*)(a.x + (size_t)row * a.k + k0 + (u & 15) * 8);
     }
   };
-  auto store_x = [&](int buf, int half) {
-    u32x4* xs = lds + buf * STAGE_UNITS;
+  auto store_x = [&](int buf, int part) {
+    u32x4* xs = lds + buf * X_UNITS;
 #pragma unroll
     for (int i = 0; i < XH; ++i) {
-      const int u = tid + (half * XH + i) * THREADS;
+      const int u = tid + (part * XH + i) * THREADS;
       xs[(u >> 4) * DROW_UNITS + (u & 15)] = permute_x_for_int4(xr[i]);
     }
   };
@@ -127,21 +151,30 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_direct_kernel(const DirectA
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  // One step = 8 MFMA groups kk = 4*c + w.  They are software pipelined by hand:
-  // while the MFMAs of group kk run, the A operands of group kk+1 are read from
-  // LDS and its B operands dequantised, into the other of two operand sets; the
-  // B operands of the NEXT step's first group are prepared during the last
-  // group, before the barrier.  An MFMA occupies the matrix pipe for 8 passes and
-  // the wave can issue 7 other instructions meanwhile, so written in this order
-  // the dequantisation and the LDS reads hide under the MFMAs of the same wave.
-  auto dequant = [&](const BStage& b, int kk, half8_t (&bf)[TN]) {
+  // ---- operands ------------------------------------------------------------------
+  // One step = 8 MFMA groups kk = 4*c + w, software pipelined by hand.  While the
+  // MFMAs of group kk run, the B operands of group kk+1 are dequantised into the
+  // other of two operand sets, and each A operand is re-read from LDS for group
+  // kk+1 as soon as its last MFMA of group kk has been issued: an MFMA occupies
+  // the matrix pipe for 8 passes and the wave can issue 7 other instructions
+  // meanwhile, so the dequantisation and the LDS reads hide under the MFMAs.
+  u32x4 bw[TN][2];  // the lane's packed chunks c = 0, 1 of the step
+  auto read_w = [&](int c) {
+    const u32x4* ws = lds_w;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int r = (wn * TN + j) * 32 + lrow;
+      bw[j][c] = ws[r * 4 + ((lk * 2 + c) ^ ((r >> 2) & 3))];
+    }
+  };
+  auto dequant = [&](const Scales& sc, int kk, half8_t (&bf)[TN]) {
     const int c = kk >> 2, w = kk & 3;
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
-      const uint32_t bits = G32 ? (c ? (b.s[j][0] >> 16) : (b.s[j][0] & 0xffffu)) : b.s[j][c];
+      const uint32_t bits = G32 ? (c ? (sc.s[j][0] >> 16) : (sc.s[j][0] & 0xffffu)) : sc.s[j][c];
       const _Float16 sh = __builtin_bit_cast(_Float16, (uint16_t)bits);
       const half2_t s2 = {sh, sh};
-      const u32x4 chunk = b.w[j][c];
+      const u32x4 chunk = bw[j][c];
       const uint32_t word = w == 0 ? chunk.x : (w == 1 ? chunk.y : (w == 2 ? chunk.z : chunk.w));
       half2_t h[4];
       unpack_int4_word(word, h);
@@ -152,65 +185,91 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_direct_kernel(const DirectA
       bf[j] = v;
     }
   };
-  auto read_a = [&](int buf, int kk, half8_t (&af)[TM]) {
-    const u32x4* xs = lds + buf * STAGE_UNITS + (wm * TM * 32 + lrow) * DROW_UNITS + lk * 8 + kk;
-#pragma unroll
-    for (int i = 0; i < TM; ++i) af[i] = __builtin_bit_cast(half8_t, xs[i * 32 * DROW_UNITS]);
+  half8_t af[TM];
+  auto read_a = [&](int buf, int kk, int i) {
+    const u32x4* xs = lds + buf * X_UNITS + (wm * TM * 32 + lrow) * DROW_UNITS + lk * 8 + kk;
+    af[i] = __builtin_bit_cast(half8_t, xs[i * 32 * DROW_UNITS]);
   };
-  auto mfmas = [&](const half8_t (&af)[TM], const half8_t (&bf)[TN]) {
+  // MFMAs of one group; `next` >= 0: re-read each A operand for group `next`
+  auto group = [&](int buf, const half8_t (&bf)[TN], int next) {
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
+    for (int i = 0; i < TM; ++i) {
 #pragma unroll
       for (int j = 0; j < TN; ++j)
         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
+      if (next >= 0) read_a(buf, next, i);
+    }
   };
 
-  // Two weight stages ping-pong (no copies, no dynamic indexing); X of step s+1 is
-  // loaded to registers while step s computes and goes to the other LDS buffer.
-  // Every load is unconditional (clamped past the end).
-  BStage b0, b1;
-  half8_t afA[TM], afB[TM], bfA[TN], bfB[TN];
-  load_x(0, 0);
-  load_b(0, b0);
-  load_b(1, b1);
-  store_x(0, 0);
-  load_x(0, 1);
-  store_x(0, 1);
-  dequant(b0, 0, bfA);
+  // ---- pipeline -----------------------------------------------------------------
+  // X and W of step s+1 are loaded to registers while step s computes and go to
+  // the other LDS buffers before the barrier that ends the step; the scales are
+  // one more step ahead.  Every load is unconditional (clamped past the end).
+  Scales s0, s1;
+  half8_t bfA[TN], bfB[TN];
+  load_s(0, s0);
+  load_s(1, s1);
+  load_w(0);
+#pragma unroll
+  for (int p = 0; p < NXP; ++p) {
+    load_x(0, p);
+    store_x(0, p);
+  }
+  store_w();
   lds_barrier();
-  // The scheduling fences keep the compiler from sinking the X loads to their
-  // use (the LDS store), which would expose their latency.
-  auto step = [&](int s, BStage& b, const BStage& bnext) {
+  // The scheduling fences keep the compiler from sinking the global loads to
+  // their use (the LDS store), which would expose their latency.
+  auto step = [&](int s, Scales& sc) {
     const int buf = s & 1;
+    load_w(s + 1);
     load_x(s + 1, 0);
-    read_a(buf, 0, afA);
+    read_w(0);
+    read_w(1);
+#pragma unroll
+    for (int i = 0; i < TM; ++i) read_a(buf, 0, i);
+    dequant(sc, 0, bfA);
     __builtin_amdgcn_sched_barrier(0);
-    read_a(buf, 1, afB); dequant(b, 1, bfB); mfmas(afA, bfA);
-    read_a(buf, 2, afA); dequant(b, 2, bfA); mfmas(afB, bfB);
-    read_a(buf, 3, afB); dequant(b, 3, bfB); mfmas(afA, bfA);
-    read_a(buf, 4, afA); dequant(b, 4, bfA); mfmas(afB, bfB);
+    dequant(sc, 1, bfB); group(buf, bfA, 1);
+    dequant(sc, 2, bfA); group(buf, bfB, 2);
+    if (NXP == 4) {
+      __builtin_amdgcn_sched_barrier(0);
+      store_x(buf ^ 1, 0);
+      load_x(s + 1, 1);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    dequant(sc, 3, bfB); group(buf, bfA, 3);
+    dequant(sc, 4, bfA); group(buf, bfB, 4);
     __builtin_amdgcn_sched_barrier(0);
-    store_x(buf ^ 1, 0);
-    load_x(s + 1, 1);
+    store_x(buf ^ 1, NXP == 4 ? 1 : 0);
+    load_x(s + 1, NXP == 4 ? 2 : 1);
+    // the single W buffer: every wave took its chunks of this step at the top of
+    // the step; the barrier makes that certain before the next step's go in
+    lds_barrier();
+    store_w();
     __builtin_amdgcn_sched_barrier(0);
-    read_a(buf, 5, afB); dequant(b, 5, bfB); mfmas(afA, bfA);
-    read_a(buf, 6, afA); dequant(b, 6, bfA); mfmas(afB, bfB);
-    read_a(buf, 7, afB); dequant(b, 7, bfB); mfmas(afA, bfA);
-    dequant(bnext, 0, bfA); mfmas(afB, bfB);
+    dequant(sc, 5, bfB); group(buf, bfA, 5);
+    dequant(sc, 6, bfA); group(buf, bfB, 6);
+    if (NXP == 4) {
+      __builtin_amdgcn_sched_barrier(0);
+      store_x(buf ^ 1, 2);
+      load_x(s + 1, 3);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    dequant(sc, 7, bfB); group(buf, bfA, 7);
+    group(buf, bfB, -1);
     __builtin_amdgcn_sched_barrier(0);
-    load_b(s + 2, b);
-    store_x(buf ^ 1, 1);
+    load_s(s + 2, sc);
+    store_x(buf ^ 1, NXP - 1);
     lds_barrier();
   };
   // Whole pairs in the loop and the odd step after it: a step under a branch
-  // inside the loop would make the wait counters at the loop head assume that the
-  // stage consumed next was refilled one step ago, and stall on it.
+  // inside the loop would make the wait counters at the loop head pessimistic.
   int s = 0;
   for (; s + 1 < a.ksteps; s += 2) {
-    step(s, b0, b1);
-    step(s + 1, b1, b0);
+    step(s, s0);
+    step(s + 1, s1);
   }
-  if (s < a.ksteps) step(s, b0, b1);
+  if (s < a.ksteps) step(s, s0);
 
   // Epilogue: one 32-row block of the wave at a time through a private LDS patch
   // (the staging buffers are free after the last barrier).
@@ -225,7 +284,7 @@ int launch_direct_tile(const DirectArgs& a, bool g32, hipStream_t stream) {
   constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
   const void* fn = g32 ? (const void*)gemm_direct_kernel<WM, WN, TM, TN, true>
                        : (const void*)gemm_direct_kernel<WM, WN, TM, TN, false>;
-  size_t lds_bytes = (size_t)2 * BM * DROW_UNITS * 16;
+  size_t lds_bytes = (size_t)(2 * BM * DROW_UNITS + BN * 4) * 16;
   const size_t patch_bytes = (size_t)WM * WN * 32 * (TN * 32 + 4) * sizeof(float);
   if (lds_bytes < patch_bytes) lds_bytes = patch_bytes;
   if (lds_bytes > 64 * 1024)

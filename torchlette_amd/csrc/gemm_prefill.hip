@@ -22,7 +22,7 @@
 // traffic only, not for the global loads in flight).
 // Epilogue: acc*alpha -> ops in order (bias indexed by n, unary) -> cast, the
 // order of applyBlockEpilogue (matmul-skeleton.ts:916-966).
-#include "device_utils.h"
+#include "gemm_common.h"
 
 namespace tlhip {
 namespace {
@@ -35,17 +35,14 @@ struct GemmArgs {
   const uint8_t* packed;  // bytes; row stride row_bytes
   const void* scales;
   const _Float16* x;
-  void* y;
   int m, n, k;
   int w_row_bytes;        // K/2 (int4) or K (int8)
   int cpg_shift;          // log2(16-byte chunks per scale group)
   int groups_per_row;
   int ksteps;
-  int tiles_m, tiles_n;
-  float alpha;
   float scale_mul;
-  int y_dtype;
-  DevEpilogue epi;
+  TileMap map;
+  OutArgs out;
 };
 
 // Unpack one 16-byte chunk to f16 values already multiplied by the scale.
@@ -120,21 +117,8 @@ __global__ __launch_bounds__(256) void gemm_prefill_kernel(const GemmArgs a) {
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
-  // XCD-aware tile order: consecutive workgroup ids are dealt round-robin to the
-  // 8 XCDs, each with its own L2.  When the column blocks divide by 8, XCD x
-  // owns the column blocks congruent to x and walks the row blocks of each in
-  // turn, so a packed W block is fetched into one L2 only.
-  const int tile = blockIdx.x;
-  int tn_idx, tm_idx;
-  if ((a.tiles_n & 7) == 0) {
-    const int xcd = tile & 7, local = tile >> 3;
-    const int q = local / a.tiles_m;
-    tn_idx = q * 8 + xcd;
-    tm_idx = local - q * a.tiles_m;
-  } else {
-    tn_idx = tile / a.tiles_m;
-    tm_idx = tile - tn_idx * a.tiles_m;
-  }
+  int tm_idx, tn_idx;
+  if (!tile_of(a.map, blockIdx.x, tm_idx, tn_idx)) return;  // padding of the tile map (whole workgroup)
   const int m0 = tm_idx * BM, n0 = tn_idx * BN;
 
   // ---- global -> register staging -------------------------------------
@@ -238,52 +222,38 @@ __global__ __launch_bounds__(256) void gemm_prefill_kernel(const GemmArgs a) {
   }
 
   // ---- epilogue -----------------------------------------------------------
-  // 32x32 accumulator layout: lane l holds column l%32 and rows
-  // 8*(r/4) + 4*(l/32) + r%4 for r = 0..15.  Each tile goes through a private
-  // 32 x 33 f32 patch of LDS (the staging buffers are free now): registers are
-  // written with static indices, and a short rolled loop reads the patch back,
-  // applies the epilogue and stores.  Applying the epilogue straight from the
-  // registers would need 16 x TM x TN inlined copies of it; the compiler then
-  // stops unrolling and the accumulators fall into scratch memory.
-  float* patch = (float*)lds + wave * (32 * 33);
+  // One 32-row block of the wave at a time through a private LDS patch (the
+  // staging buffers are free now); see wave_epilogue.  Applying the epilogue
+  // straight from the accumulator registers would need 16 x TM x TN inlined
+  // copies of it; the compiler then stops unrolling and the accumulators fall
+  // into scratch memory.
+  float* patch = (float*)lds + wave * (32 * (TN * 32 + 4));
 #pragma unroll
-  for (int j = 0; j < TN; ++j) {
-#pragma unroll
-    for (int i = 0; i < TM; ++i) {
-#pragma unroll
-      for (int r = 0; r < 16; ++r) patch[(8 * (r >> 2) + 4 * lk + (r & 3)) * 33 + lrow] = acc[i][j][r];
-      __builtin_amdgcn_s_waitcnt(0xc07f);  // this wave's LDS writes have landed (lgkmcnt(0))
-      const int64_t col = n0 + wn * (BN / 2) + j * 32 + lrow;
-      const int row0 = m0 + wm * (BM / 2) + i * 32 + lk;
-#pragma unroll 1
-      for (int it = 0; it < 16; ++it) {
-        const int row = row0 + 2 * it;
-        const float v = patch[(2 * it + lk) * 33 + lrow];
-        if (row < a.m && col < a.n)
-          store_out(a.y, a.y_dtype, (int64_t)row * a.n + col, apply_epilogue(a.epi, v * a.alpha, col));
-      }
-      __builtin_amdgcn_s_waitcnt(0xc07f);  // reads done before the patch is overwritten
-    }
-  }
+  for (int i = 0; i < TM; ++i)
+    wave_epilogue<TN>(patch, acc[i], lane, m0 + wm * (BM / 2) + i * 32, n0 + wn * (BN / 2), a.out);
 }
 
 template <int FMT, int BM, int BN>
 int launch_tile(const GemmArgs& a, hipStream_t stream) {
   const void* fn = (const void*)gemm_prefill_kernel<FMT, BM, BN>;
-  const size_t lds_bytes = (size_t)2 * (BM + BN) * ROW_BYTES;
+  size_t lds_bytes = (size_t)2 * (BM + BN) * ROW_BYTES;
+  const size_t patch_bytes = (size_t)4 * 32 * (BN / 64 * 32 + 4) * sizeof(float);
+  if (lds_bytes < patch_bytes) lds_bytes = patch_bytes;
   if (lds_bytes > 64 * 1024)
     TLHIP_CHECK_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
   GemmArgs b = a;
-  b.tiles_m = (a.m + BM - 1) / BM;
-  b.tiles_n = (a.n + BN - 1) / BN;
+  int grid = 0;
+  b.map = make_tile_map((a.m + BM - 1) / BM, (a.n + BN - 1) / BN, &grid);
   void* args[] = {(void*)&b};
-  TLHIP_CHECK_HIP(hipLaunchKernel(fn, dim3(b.tiles_m * b.tiles_n), dim3(256), args, lds_bytes, stream));
+  TLHIP_CHECK_HIP(hipLaunchKernel(fn, dim3(grid), dim3(256), args, lds_bytes, stream));
   return TLHIP_OK;
 }
 
 template <int FMT>
 int launch_fmt(int bm, int bn, const GemmArgs& a, hipStream_t stream) {
-  if (bm == 256 && bn == 256) return launch_tile<FMT, 256, 256>(a, stream);
+  if constexpr (FMT == TLHIP_FMT_INT4_GROUPED) {
+    if (bm == 256 && bn == 256) return launch_tile<FMT, 256, 256>(a, stream);
+  }
   if (bm == 128 && bn == 256) return launch_tile<FMT, 128, 256>(a, stream);
   if (bm == 256 && bn == 128) return launch_tile<FMT, 256, 128>(a, stream);
   if (bm == 128 && bn == 128) return launch_tile<FMT, 128, 128>(a, stream);
@@ -299,7 +269,7 @@ bool gemm_config_applicable(const Problem& p, const tlhip_kernel_config_t& c, co
       "activations must be f16",
       "K must be a multiple of 64",
       "group size must be a multiple of 32 (int4) or 16 (int8)",
-      "tile must be one of 256x256, 128x256, 256x128, 128x128, 64x128 with tile K 64 and 2x2 waves",
+      "tile must be one of 256x256 (int4 only), 128x256, 256x128, 128x128, 64x128 with tile K 64 and 2x2 waves",
   };
   auto fail = [&](int i) {
     if (why) *why = reasons[i];
@@ -314,6 +284,8 @@ bool gemm_config_applicable(const Problem& p, const tlhip_kernel_config_t& c, co
   const bool ok = (bm == 256 && bn == 256) || (bm == 128 && bn == 256) || (bm == 256 && bn == 128) ||
                   (bm == 128 && bn == 128) || (bm == 64 && bn == 128);
   if (!ok || c.p2 != 64 || c.p3 != 2 || c.p4 != 2) return fail(4);
+  // the int8 dequantisation needs more registers: its 256 x 256 instance would spill
+  if (bm == 256 && bn == 256 && p.format != TLHIP_FMT_INT4_GROUPED) return fail(4);
   return true;
 }
 
@@ -327,7 +299,6 @@ int launch_gemm(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t st
   a.packed = (const uint8_t*)p.packed;
   a.scales = p.scales;
   a.x = (const _Float16*)p.x;
-  a.y = p.y;
   a.m = (int)p.m;
   a.n = (int)p.n;
   a.k = (int)p.k;
@@ -335,11 +306,14 @@ int launch_gemm(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t st
   a.cpg_shift = p.format == TLHIP_FMT_INT8_ROW ? 0 : __builtin_ctz((unsigned)(p.group_size / cw));
   a.groups_per_row = p.format == TLHIP_FMT_INT8_ROW ? 0 : (int)(p.k / p.group_size);
   a.ksteps = (int)(p.k / BK);
-  a.tiles_m = a.tiles_n = 0;
-  a.alpha = p.alpha;
   a.scale_mul = p.format == TLHIP_FMT_INT8_GROUPED ? (1.0f / 127.0f) : 1.0f;
-  a.y_dtype = p.y_dtype;
-  a.epi = p.epi;
+  a.out.y = p.y;
+  a.out.y_dtype = p.y_dtype;
+  a.out.vec_ok = (p.n % 8 == 0) && ((uintptr_t)p.y % 16 == 0);
+  a.out.m = (int)p.m;
+  a.out.n = (int)p.n;
+  a.out.alpha = p.alpha;
+  a.out.epi = p.epi;
   int rc;
   switch (p.format) {
     case TLHIP_FMT_INT4_GROUPED: rc = launch_fmt<TLHIP_FMT_INT4_GROUPED>(c.p0, c.p1, a, stream); break;
