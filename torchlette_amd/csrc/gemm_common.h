@@ -82,6 +82,23 @@ __device__ __forceinline__ void wave_epilogue(float* patch, const float16_t (&ac
   const int rr0 = lane / LPR, cc = (lane % LPR) * 8;
   const int col = col0 + cc;
   const bool vec = o.vec_ok && col + 8 <= o.n;
+  // The common chain, [bias] then [unary], keeps the lane's 8 bias values in
+  // registers across the passes (the column does not change) and runs no loop
+  // over the ops per element.
+  const int n_ops = o.epi.n_ops;
+  const bool has_bias = n_ops >= 1 && o.epi.kind[0] == TLHIP_EPI_BIAS;
+  const int un_at = has_bias ? 1 : 0;
+  const bool simple = n_ops <= un_at + 1 && (n_ops == un_at || o.epi.kind[un_at] == TLHIP_EPI_UNARY);
+  const int unary = (simple && n_ops > un_at) ? o.epi.unary[un_at] : TLHIP_UNARY_NONE;
+  float bias[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    bias[e] = 0.f;
+    if (simple && has_bias && col + e < o.n) {
+      if (o.epi.input_dtype[0] == TLHIP_F16) bias[e] = (float)((const _Float16*)o.epi.input[0])[col + e];
+      else bias[e] = ((const float*)o.epi.input[0])[col + e];
+    }
+  }
 #pragma unroll 1
   for (int p = 0; p < 32 / RPP; ++p) {
     const int rr = p * RPP + rr0;
@@ -90,9 +107,14 @@ __device__ __forceinline__ void wave_epilogue(float* patch, const float16_t (&ac
     const float4_t b = *(const float4_t*)(patch + rr * PW + cc + 4);
     float v[8] = {a[0], a[1], a[2], a[3], b[0], b[1], b[2], b[3]};
     if (row < o.m) {
-      if (vec) {
+      if (simple) {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) v[e] = apply_epilogue(o.epi, v[e] * o.alpha, col + e);
+        for (int e = 0; e < 8; ++e) v[e] = apply_unary(unary, v[e] * o.alpha + bias[e]);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = apply_epilogue(o.epi, v[e] * o.alpha, min(col + e, o.n - 1));
+      }
+      if (vec) {
         const int64_t idx = (int64_t)row * o.n + col;
         if (o.y_dtype == TLHIP_F16) {
           half8_t h;
@@ -105,9 +127,9 @@ __device__ __forceinline__ void wave_epilogue(float* patch, const float16_t (&ac
           *(float4_t*)(dst + 4) = (float4_t){v[4], v[5], v[6], v[7]};
         }
       } else {
+#pragma unroll
         for (int e = 0; e < 8; ++e)
-          if (col + e < o.n)
-            store_out(o.y, o.y_dtype, (int64_t)row * o.n + col + e, apply_epilogue(o.epi, v[e] * o.alpha, col + e));
+          if (col + e < o.n) store_out(o.y, o.y_dtype, (int64_t)row * o.n + col + e, v[e]);
       }
     }
   }
