@@ -205,6 +205,11 @@ def main() -> int:
     ap.add_argument("--no-autotune", action="store_true", help="use the heuristic kernel choices")
     ap.add_argument("--autotune", action="store_true",
                     help="re-tune every case (weights rotating through HBM) even if a tuning cache file exists")
+    ap.add_argument("--traffic-probe", action="store_true",
+                    help="for a counter run under rocprofv3 --pmc: 20 launches of the step's slowest call, then "
+                         "three device-to-device copies of 256 MiB (the known size the counters are scaled by), and exit")
+    ap.add_argument("--traffic-file", default=os.path.join(ROOT, "torchlette_amd", "tuning", "mi355x_traffic.json"),
+                    help="measured HBM bytes per launch (from the counter runs), keyed by call; fills roofline.traffic")
     ap.add_argument("--tuning-cache", default=os.path.join(ROOT, "torchlette_amd", "tuning", "mi355x.json"),
                     help="JSON tuning cache to import before the run and to write after --autotune")
     args = ap.parse_args()
@@ -247,6 +252,24 @@ def main() -> int:
                           "config": list(cfg.as_tuple()), "kernel": kernel_name_of(cfg)})
     step_bytes = sum(c["bytes"] for c in cases)
 
+    if args.traffic_probe:
+        for c in cases:
+            c["us"] = B.median_time(c["call"], 50, batches=3)
+        dom = max(cases, key=lambda c: c["us"])
+        be.synchronize()
+        for _ in range(20):
+            dom["call"]()
+        be.synchronize()
+        nbytes = 256 << 20
+        src, dst = be._alloc([nbytes // 4], "f32"), be._alloc([nbytes // 4], "f32")
+        for _ in range(3):
+            L.call("tlhip_memcpy_d2d", dst.ptr, src.ptr, nbytes, None)
+        be.synchronize()
+        print(json.dumps({"traffic_probe": {"m": dom["m"], "n": dom["n"], "k": dom["k"], "kernel": dom["kernel"],
+                                            "config": dom["config"], "algorithmic_bytes": dom["bytes"],
+                                            "launches": 20, "copy_bytes": nbytes, "copies": 3}}))
+        return 0
+
     def step():
         for c in cases:
             c["call"]()
@@ -266,8 +289,14 @@ def main() -> int:
         c["gbps"] = c["bytes"] / c["us"] / 1e3
     dominant = max(cases, key=lambda c: c["us"])
     dom_us = B.median_time(dominant["call"], 500, batches=7)
+    # HBM bytes per launch measured with FETCH_SIZE / WRITE_SIZE counter runs of --traffic-probe
+    traffic = None
+    if os.path.exists(args.traffic_file):
+        rec = json.load(open(args.traffic_file)).get(f'{dominant["m"]}_{dominant["n"]}_{dominant["k"]}_int4-g32')
+        if rec and rec.get("config") == dominant["config"]:
+            traffic = rec["traffic_bytes"]
     roofline = {"bound": "hbm", "achieved": dominant["bytes"] / dom_us / 1e3, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                "frac": dominant["bytes"] / dom_us / 1e3 / HBM_PEAK_GBPS, "traffic": None,
+                "frac": dominant["bytes"] / dom_us / 1e3 / HBM_PEAK_GBPS, "traffic": traffic,
                 "kernel": dominant["kernel"], "launch_us": dom_us, "bytes_per_launch": dominant["bytes"],
                 "shape": {"m": dominant["m"], "n": dominant["n"], "k": dominant["k"]}}
 
