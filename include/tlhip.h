@@ -161,6 +161,14 @@ float tlhip_f16_bits_to_f32(uint16_t bits);
 int tlhip_quantize_int8_grouped(const float* host_weight, int64_t n, int64_t k, int64_t group_size,
                                 uint32_t* host_packed, uint16_t* host_scales);
 
+/* The same quantizer on the device, for weights already resident in HBM
+ * (quantize-at-load, examples/qwen3/loader.ts:228-254): `weight` f32 [n,k],
+ * `packed` u32 [n,k/4], `scales` u16 [n,k/group_size], all device pointers.
+ * Bit-identical to tlhip_quantize_int8_grouped.  group_size must also be a
+ * multiple of 4 here. */
+int tlhip_quantize_int8_grouped_device(const float* weight, int64_t n, int64_t k, int64_t group_size,
+                                       uint32_t* packed, uint16_t* scales, tlhip_stream_t stream);
+
 /* ---- compute ---- */
 
 /* Explicit dequantisation to f32 [N,K], bit-exact against dequantizeToF32

@@ -95,6 +95,7 @@ SIGNATURES = {
     "tlhip_graph_destroy": (_i, [_vp]),
     "tlhip_f32_to_f16_bits": (C.c_uint16, [_f]),
     "tlhip_f16_bits_to_f32": (_f, [C.c_uint16]),
+    "tlhip_quantize_int8_grouped_device": (_i, [_vp, _i64, _i64, _i64, _vp, _vp, _vp]),
     "tlhip_quantize_int8_grouped": (_i, [_vp, _i64, _i64, _i64, _vp, _vp]),
     "tlhip_dequant": (_i, [_QW, _vp, _vp]),
     "tlhip_gemv": (_i, [_QW, _vp, _i, _i64, _vp, _i, _f, _EP, _vp]),

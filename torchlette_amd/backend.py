@@ -359,6 +359,30 @@ class HipBackend:
         self._state.extend([packedT, scalesT, logical])
         return logical
 
+    def quantizeLinearWeightOnDevice(self, weight: HipTensor, groupSize: int = 64,
+                                     elementType: str = "f32") -> HipTensor:
+        """quantizeLinearWeight (quantize.ts:77-131) for a weight that is already
+        on the device (quantize-at-load, examples/qwen3/loader.ts:228-254): f32
+        [N,K] in, the logical packed [N,K] weight with ``format`` and ``scales``
+        out, bit-identical to the host quantizer followed by
+        ``createQuantizedWeight``."""
+        if weight.dtype != "f32" or len(weight.shape) != 2 or not weight.isContiguous:
+            raise ValueError("quantizeLinearWeightOnDevice: weight must be a contiguous f32 [N,K] tensor")
+        n, k = weight.shape
+        if k % 4 != 0:
+            raise ValueError(f"quantizeLinearWeight: K={k} must be divisible by 4")
+        if groupSize <= 0 or k % groupSize != 0:
+            raise ValueError(f"quantizeLinearWeight: K={k} must be divisible by groupSize={groupSize}")
+        packedT = self._alloc([n, k // 4], "u32")
+        scalesT = self._alloc([n * (k // groupSize)], "f16")
+        L.call("tlhip_quantize_int8_grouped_device", weight.ptr, n, k, groupSize, packedT.ptr, scalesT.ptr,
+               self.stream)
+        fmt = StorageFormat(elementType, QuantPacking("int8-grouped", groupSize))
+        logical = HipTensor(self, [n, k], elementType, packedT.ptr, packedT.nbytes, False, [k, 1], fmt,
+                            scalesT, packedT)
+        self._state.extend([packedT, scalesT, logical])
+        return logical
+
     def dequantizeToF32(self, w: HipTensor) -> HipTensor:
         """Explicit dequant of a packed weight to f32 [N,K] on the device
         (quantize.ts:138-156; matmul/dispatch.ts:949-1037)."""
