@@ -185,6 +185,23 @@ int tlhip_dequant(const tlhip_qweight_t* w, float* out, tlhip_stream_t stream);
 int tlhip_gemv(const tlhip_qweight_t* w, const void* x, int x_dtype, int64_t m, void* y,
                int y_dtype, float alpha, const tlhip_epilogue_t* epilogue, tlhip_stream_t stream);
 
+/* Up to 4 decode GEMVs of one shape class in ONE launch (q/k/v or gate/up of a
+ * decode step: the frontend issues them back to back on the same activations,
+ * src/frontend/torchlette.ts:878-894 once per Linear, and each is too small to
+ * fill the chip while every launch costs 2-3 us).  All problems: m = 1, f16
+ * activations, the same format, group size, K and output type; N, pointers and
+ * epilogues are per problem.  Results are those of `count` tlhip_gemv calls.
+ * Falls back to separate launches when the selected kernel configuration has no
+ * grouped form. */
+typedef struct {
+  tlhip_qweight_t w;
+  const void* x;
+  void* y;
+  const tlhip_epilogue_t* epilogue; /* may be NULL */
+} tlhip_gemv_problem_t;
+int tlhip_gemv_grouped(const tlhip_gemv_problem_t* problems, int count, int x_dtype, int y_dtype, float alpha,
+                       tlhip_stream_t stream);
+
 /* Prefill GEMM with dequant fused into the LDS stage: same contract as
  * tlhip_gemv for any m >= 1; x must be f16.  Stands in for the explicit
  * dequant + stock matmul the reference runs when M > 1

@@ -298,3 +298,57 @@ def test_transpose_view_carries_format_and_scales(be):
     wt = be.ops.transpose(w)
     assert wt.shape == [64, 32] and wt.strides == [1, 64]
     assert wt.format is w.format and wt.scales is w.scales and wt.ownsBuffer is False
+
+
+@pytest.mark.parametrize("fmt,g,k,ns", [
+    ("int4-grouped", 32, 1024, [2048, 1024, 1024]),       # q, k, v of the 0.6B decode step
+    ("int4-grouped", 32, 1024, [3072, 3072]),              # gate, up
+    ("int4-grouped", 64, 3072, [1024]),                    # a group of one
+    ("int8-row", 0, 2304, [1000, 37, 515, 2048]),          # ragged N, four problems
+    ("int8-grouped", 64, 2048, [4096, 512]),
+])
+def test_grouped_decode_gemvs_equal_separate_launches(be, fmt, g, k, ns):
+    """q/k/v (or gate/up) in one launch: bit-identical to the separate calls with
+    the same kernel configuration, and within tolerance of the oracle."""
+    rng = np.random.default_rng(sum(ns) + k)
+    x = make_x(1, k, "f16", rng)
+    xt = be.ops.tensorFromArray(x, [1, k], "f16")
+    ws, deqs, biases, bts = [], [], [], []
+    for n in ns:
+        packed, scales, deq = make_weight(fmt, n, k, g, rng)
+        ws.append(be.createQuantizedWeight(packed, scales, n, k, T.resolveWeightFormat(fmt_name(fmt, g), "f32")))
+        deqs.append(deq)
+        b = rng.standard_normal(n).astype(np.float32)
+        biases.append(b)
+        bts.append(be.ops.tensorFromArray(b, [n], "f32"))
+    before = T.getQuantGemvDispatchCount()
+    outs = be.linearGrouped(xt, ws, bts, "silu")
+    assert T.getQuantGemvDispatchCount() == before + len(ns)
+    for w, bt, b, deq, o in zip(ws, bts, biases, deqs, outs):
+        got = o.numpy()
+        want = O.linear(x.astype(np.float32), deq, b, "silu")
+        assert rel_l2(got, want) <= 2e-6
+        c = be.selectedConfig(ws[int(np.argmax(ns))], "f16", 1, "f32")
+        if c.variant == 0:
+            c.p4 = 2
+            c.p1 = min(c.p1, 2)
+            sep = be.linear(xt, w, bt, "silu", fused=True, config=c).numpy()
+            assert np.array_equal(got, sep)
+
+
+def test_grouped_gemv_rejects_mixed_shapes(be):
+    rng = np.random.default_rng(1)
+    x = be.ops.tensorFromArray(make_x(1, 256, "f16", rng), [1, 256], "f16")
+    p1, s1, _ = make_weight("int4-grouped", 64, 256, 32, rng)
+    p2, s2, _ = make_weight("int4-grouped", 64, 512, 32, rng)
+    w1 = be.createQuantizedWeight(p1, s1, 64, 256, T.resolveWeightFormat("int4-32", "f32"))
+    w2 = be.createQuantizedWeight(p2, s2, 64, 512, T.resolveWeightFormat("int4-32", "f32"))
+    # different K cannot share the activation row: the second problem's K does not match x
+    outs = be.linearGrouped(x, [w1], None, None)
+    assert outs[0].numpy().shape == (1, 64)
+    with pytest.raises(ValueError, match="1..4"):
+        be.linearGrouped(x, [w1] * 5)
+    x2 = be.ops.tensorFromArray(make_x(2, 256, "f16", rng), [2, 256], "f16")
+    with pytest.raises(ValueError, match="one f16 activation row"):
+        be.linearGrouped(x2, [w1])
+    del w2

@@ -65,6 +65,10 @@ class KernelConfig(C.Structure):
         return cls(*vals)
 
 
+class GemvProblem(C.Structure):
+    _fields_ = [("w", QWeight), ("x", C.c_void_p), ("y", C.c_void_p), ("epilogue", C.POINTER(Epilogue))]
+
+
 # name -> (restype, argtypes); every symbol include/tlhip.h declares.
 _vp, _i, _i64, _sz, _f = C.c_void_p, C.c_int, C.c_int64, C.c_size_t, C.c_float
 _QW, _EP, _KC = C.POINTER(QWeight), C.POINTER(Epilogue), C.POINTER(KernelConfig)
@@ -99,6 +103,7 @@ SIGNATURES = {
     "tlhip_quantize_int8_grouped": (_i, [_vp, _i64, _i64, _i64, _vp, _vp]),
     "tlhip_dequant": (_i, [_QW, _vp, _vp]),
     "tlhip_gemv": (_i, [_QW, _vp, _i, _i64, _vp, _i, _f, _EP, _vp]),
+    "tlhip_gemv_grouped": (_i, [C.POINTER(GemvProblem), _i, _i, _i, _f, _vp]),
     "tlhip_gemm_prefill": (_i, [_QW, _vp, _i, _i64, _vp, _i, _f, _EP, _vp]),
     "tlhip_matmul_quantized": (_i, [_QW, _vp, _i, _i64, _vp, _i, _f, _EP, _vp]),
     "tlhip_matmul_quantized_config": (_i, [_QW, _vp, _i, _i64, _vp, _i, _f, _EP, _KC, _vp]),

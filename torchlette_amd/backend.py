@@ -475,6 +475,32 @@ class HipBackend:
             y = y2
         return y
 
+    def linearGrouped(self, input: HipTensor, weights: Sequence[HipTensor],
+                      biases: Optional[Sequence[Optional[HipTensor]]] = None,
+                      activation: Optional[str] = None) -> List[HipTensor]:
+        """Up to four decode Linears on the same activation row (q/k/v, or gate/up)
+        in one launch: the results of ``[linear(input, w, b, activation, fused=True)
+        for w, b in zip(weights, biases)]``.  M = 1 and f16 activations."""
+        if not 1 <= len(weights) <= 4:
+            raise ValueError("linearGrouped: a group holds 1..4 weights")
+        biases = list(biases) if biases is not None else [None] * len(weights)
+        qws = [self._qweight(w, transposed=False) for w in weights]
+        m = input.size // qws[0].k
+        if m != 1 or input.dtype != "f16":
+            raise ValueError("linearGrouped: one f16 activation row")
+        out_dtype = "f16" if all(w.format.elementType == "f16" for w in weights) else "f32"
+        outs = [self._alloc(list(input.shape[:-1]) + [qw.n], out_dtype) for qw in qws]
+        eps = [self.makeEpilogue(b, activation) for b in biases]
+        probs = (L.GemvProblem * len(weights))()
+        for i, (qw, o, ep) in enumerate(zip(qws, outs, eps)):
+            probs[i].w = qw
+            probs[i].x = input.ptr
+            probs[i].y = o.ptr
+            probs[i].epilogue = C.pointer(ep) if ep is not None else None
+        L.call("tlhip_gemv_grouped", probs, len(weights), _DT_CODE[input.dtype], _DT_CODE[out_dtype], 1.0,
+               self.stream)
+        return outs
+
     # tuning + counters -----------------------------------------------------
     def pretuneMatmulShapes(self, shapes: Sequence[Sequence[int]]) -> None:
         flat = (C.c_int64 * (3 * len(shapes)))(*[int(v) for s in shapes for v in s])

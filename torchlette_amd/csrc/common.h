@@ -66,6 +66,8 @@ int validate_weight(const tlhip_qweight_t* w, const char* who);
 int launch_dequant(const tlhip_qweight_t& w, float* out, hipStream_t stream);
 bool gemv_config_applicable(const Problem& p, const tlhip_kernel_config_t& c, const char** why);
 int launch_gemv(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t stream);
+bool gemv_group_compatible(const Problem* ps, int count, const tlhip_kernel_config_t& c, const char** why);
+int launch_gemv_grouped(const Problem* ps, int count, const tlhip_kernel_config_t& c, hipStream_t stream);
 bool gemv_mfma_config_applicable(const Problem& p, const tlhip_kernel_config_t& c, const char** why);
 int launch_gemv_mfma(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t stream);
 bool gemm_config_applicable(const Problem& p, const tlhip_kernel_config_t& c, const char** why);

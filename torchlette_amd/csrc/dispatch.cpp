@@ -351,6 +351,8 @@ int tlhip_dequant(const tlhip_qweight_t* w, float* out, tlhip_stream_t stream) {
   return launch_dequant(*w, out, resolve_stream(stream));
 }
 
+static int matmul_with(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t stream);
+
 int tlhip_gemv(const tlhip_qweight_t* w, const void* x, int x_dtype, int64_t m, void* y, int y_dtype,
                float alpha, const tlhip_epilogue_t* epilogue, tlhip_stream_t stream) {
   TLHIP_REQUIRE_INIT();
@@ -361,6 +363,36 @@ int tlhip_gemv(const tlhip_qweight_t* w, const void* x, int x_dtype, int64_t m, 
   tlhip_kernel_config_t c = select_config(p);
   if (c.variant == VARIANT_TILED || c.variant == VARIANT_TILED_DIRECT) c = default_config(p);
   return run_config(p, c, resolve_stream(stream));
+}
+
+int tlhip_gemv_grouped(const tlhip_gemv_problem_t* problems, int count, int x_dtype, int y_dtype, float alpha,
+                       tlhip_stream_t stream) {
+  TLHIP_REQUIRE_INIT();
+  if (count < 0 || (count > 0 && !problems)) return set_error(TLHIP_ERR_INVALID, "gemv_grouped: bad problem list");
+  if (count > 4) return set_error(TLHIP_ERR_INVALID, "gemv_grouped: a group holds at most 4 problems, got %d", count);
+  Problem ps[4];
+  for (int i = 0; i < count; ++i) {
+    int rc = make_problem(&problems[i].w, problems[i].x, x_dtype, 1, problems[i].y, y_dtype, alpha,
+                          problems[i].epilogue, &ps[i], "gemv_grouped");
+    if (rc) return rc;
+  }
+  if (count == 0) return TLHIP_OK;
+  hipStream_t s = resolve_stream(stream);
+  // the configuration of the largest problem, in its grouped form when there is one
+  int big = 0;
+  for (int i = 1; i < count; ++i)
+    if (ps[i].n > ps[big].n) big = i;
+  tlhip_kernel_config_t c = select_config(ps[big]);
+  if (c.variant == VARIANT_GEMV) {
+    c.p4 = 2;
+    if (c.p1 > 2) c.p1 = 2;
+    if (gemv_group_compatible(ps, count, c, nullptr)) return launch_gemv_grouped(ps, count, c, s);
+  }
+  for (int i = 0; i < count; ++i) {
+    int rc = matmul_with(ps[i], select_config(ps[i]), s);
+    if (rc) return rc;
+  }
+  return TLHIP_OK;
 }
 
 int tlhip_gemm_prefill(const tlhip_qweight_t* w, const void* x, int x_dtype, int64_t m, void* y, int y_dtype,

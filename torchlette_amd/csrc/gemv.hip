@@ -170,8 +170,11 @@ struct ChunkDot<TLHIP_FMT_INT4_GROUPED, float> {
 // overlaps the staging, the arithmetic and the reductions.  The hot path has no
 // per-lane branches: out-of-range chunks load a clamped address and contribute
 // zero through their scale (or a select).
+// `bid` / `nblk`: this workgroup's index among, and the number of, the workgroups
+// that work on this problem (the whole grid for a single launch; a slice of it
+// when several problems share one launch).
 template <int FMT, typename XT, int MT, int R, int U>
-__global__ __launch_bounds__(512) void gemv_kernel(const GemvArgs a) {
+__device__ __forceinline__ void gemv_body(const GemvArgs& a, const int bid, const int nblk) {
   using Dot = ChunkDot<FMT, XT>;
   constexpr int NQ = Dot::NQ;
   constexpr bool GROUPED = (FMT != TLHIP_FMT_INT8_ROW);
@@ -306,7 +309,7 @@ __global__ __launch_bounds__(512) void gemv_kernel(const GemvArgs a) {
 
   const int step_chunks = cstride * U;
   const int nsteps = a.nsteps;
-  int rb = blockIdx.x, step = 0;
+  int rb = bid, step = 0;
   Batch cur;
   // Order of issue matters: loads return in order, so the (few) activation
   // loads go first, then the first weight batch; the LDS store then waits for
@@ -379,12 +382,12 @@ __global__ __launch_bounds__(512) void gemv_kernel(const GemvArgs a) {
   // the steady-state loop is unconditional: a load under a branch makes the wait
   // counters at the join assume it was NOT issued, and the consumer of the other
   // set would then wait for the load just issued.
-  const int rounds = (a.nblocks - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;
+  const int rounds = (a.nblocks - bid + nblk - 1) / nblk;
   const int total = rounds * nsteps;
   auto advance = [&](int& r, int& st) {
     if (++st == nsteps) {
       st = 0;
-      r += gridDim.x;
+      r += nblk;
     }
   };
   auto consume = [&](const Batch& b, int r, int st) {
@@ -418,6 +421,32 @@ __global__ __launch_bounds__(512) void gemv_kernel(const GemvArgs a) {
   } else if (total - j == 1) {
     consume(cur, rb, step);
   }
+}
+
+template <int FMT, typename XT, int MT, int R, int U>
+__global__ __launch_bounds__(512) void gemv_kernel(const GemvArgs a) {
+  gemv_body<FMT, XT, MT, R, U>(a, blockIdx.x, gridDim.x);
+}
+
+// Several problems of one shape class (same format, K, activation type, rows and
+// kernel configuration; N, pointers and epilogues differ) in ONE launch: a decode
+// step issues q/k/v or gate/up on the same activations, each far too small to
+// fill the chip, and every launch costs 2-3 us.  Workgroups
+// [first[i], first[i+1]) work on problem i.
+constexpr int kMaxGroup = 4;
+struct GroupedGemvArgs {
+  int count;
+  int first[kMaxGroup + 1];
+  GemvArgs p[kMaxGroup];
+};
+
+template <int FMT, typename XT, int MT, int R, int U>
+__global__ __launch_bounds__(512) void gemv_grouped_kernel(const GroupedGemvArgs g) {
+  int i = 0;
+#pragma unroll
+  for (int j = 1; j < kMaxGroup; ++j)
+    if (j < g.count && (int)blockIdx.x >= g.first[j]) i = j;
+  gemv_body<FMT, XT, MT, R, U>(g.p[i], (int)blockIdx.x - g.first[i], g.first[i + 1] - g.first[i]);
 }
 
 constexpr int kLdsBudget = 128 * 1024;
@@ -498,15 +527,58 @@ bool gemv_config_applicable(const Problem& p, const tlhip_kernel_config_t& c, co
   return true;
 }
 
+// Kernel arguments and launch geometry of one pass (rows m0 .. m0+mrows of x).
+static void fill_args(const Problem& p, const tlhip_kernel_config_t& c, int64_t m0, int mrows, GemvArgs& a, int& mt,
+                      int& threads, int& grid, size_t& lds_bytes) {
+  const int cw = chunk_weights(p.format);
+  const int xbytes = p.x_dtype == TLHIP_F16 ? 2 : 4;
+  const int ybytes = p.y_dtype == TLHIP_F16 ? 2 : 4;
+  mt = mrows == 1 ? 1 : (mrows == 2 ? 2 : 4);
+  a.packed = (const u32x4*)p.packed;
+  a.scales = p.scales;
+  a.x = (const char*)p.x + m0 * p.k * xbytes;
+  a.y = (char*)p.y + m0 * p.n * ybytes;
+  a.n = p.n;
+  a.k = (int)p.k;
+  a.m = mrows;
+  a.nchunks = (int)(p.k / cw);
+  a.cpg_shift = p.format == TLHIP_FMT_INT8_ROW ? 0 : __builtin_ctz((unsigned)(p.group_size / cw));
+  a.groups_per_row = p.format == TLHIP_FMT_INT8_ROW ? 0 : (int)(p.k / p.group_size);
+  a.lpr = c.p0;
+  a.lpr_shift = __builtin_ctz((unsigned)c.p0);
+  a.kw = c.p3;
+  a.kw_shift = __builtin_ctz((unsigned)c.p3);
+  const int r = c.p1, waves = c.p2, unroll = c.p4 == 0 ? 2 : c.p4;
+  a.nsteps = (a.nchunks + a.lpr * a.kw * unroll - 1) / (a.lpr * a.kw * unroll);
+  a.rows_per_wave = (64 / a.lpr) * r;
+  a.rows_per_wg = (waves / a.kw) * a.rows_per_wave;
+  a.nblocks = (int)((p.n + a.rows_per_wg - 1) / a.rows_per_wg);
+  a.alpha = p.alpha;
+  a.scale_mul = p.format == TLHIP_FMT_INT8_GROUPED ? (1.0f / 127.0f) : 1.0f;
+  a.y_dtype = p.y_dtype;
+  a.epi = p.epi;
+  // LDS: staged x (mt rows) + split-K partials
+  const int chunk_x_bytes = cw * xbytes;
+  const size_t partial_bytes = a.kw > 1 ? (size_t)a.kw * a.rows_per_wg * mt * sizeof(float) : 0;
+  lds_bytes = (size_t)mt * chunk_x_bytes * a.nchunks + partial_bytes;
+  threads = waves * 64;
+  const int cus = device_cu_count();
+  // resident workgroups per CU: bounded by 2048 lanes and by LDS
+  int per_cu = 2048 / threads;
+  const int by_lds = (int)((160 * 1024) / (lds_bytes ? lds_bytes : 1));
+  if (by_lds < per_cu) per_cu = by_lds < 1 ? 1 : by_lds;
+  if (per_cu < 1) per_cu = 1;
+  grid = a.nblocks < cus * per_cu ? a.nblocks : cus * per_cu;
+  if (grid < 1) grid = 1;
+}
+
 // One launch handles at most 4 activation rows; larger M is issued as passes of
 // 4 rows (each pass streams the weights again — the MFMA variant avoids that).
 int launch_gemv(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t stream) {
   const char* why = nullptr;
   if (!gemv_config_applicable(p, c, &why)) return set_error(TLHIP_ERR_INVALID, "gemv: config not applicable: %s", why);
   if (p.n == 0 || p.m == 0) return TLHIP_OK;
-  const int cw = chunk_weights(p.format);
   const int xbytes = p.x_dtype == TLHIP_F16 ? 2 : 4;
-  const int ybytes = p.y_dtype == TLHIP_F16 ? 2 : 4;
 
   // activation rows per pass: as many (4, 2 or 1) as fit LDS next to the partials
   int pass = 4;
@@ -516,44 +588,11 @@ int launch_gemv(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t st
 
   for (int64_t m0 = 0; m0 < p.m; m0 += pass) {
     const int mrows = (int)(p.m - m0 < pass ? p.m - m0 : pass);
-    const int mt = mrows == 1 ? 1 : (mrows == 2 ? 2 : 4);
     GemvArgs a;
-    a.packed = (const u32x4*)p.packed;
-    a.scales = p.scales;
-    a.x = (const char*)p.x + m0 * p.k * xbytes;
-    a.y = (char*)p.y + m0 * p.n * ybytes;
-    a.n = p.n;
-    a.k = (int)p.k;
-    a.m = mrows;
-    a.nchunks = (int)(p.k / cw);
-    a.cpg_shift = p.format == TLHIP_FMT_INT8_ROW ? 0 : __builtin_ctz((unsigned)(p.group_size / cw));
-    a.groups_per_row = p.format == TLHIP_FMT_INT8_ROW ? 0 : (int)(p.k / p.group_size);
-    a.lpr = c.p0;
-    a.lpr_shift = __builtin_ctz((unsigned)c.p0);
-    a.kw = c.p3;
-    a.kw_shift = __builtin_ctz((unsigned)c.p3);
-    const int r = c.p1, waves = c.p2, unroll = c.p4 == 0 ? 2 : c.p4;
-    a.nsteps = (a.nchunks + a.lpr * a.kw * unroll - 1) / (a.lpr * a.kw * unroll);
-    a.rows_per_wave = (64 / a.lpr) * r;
-    a.rows_per_wg = (waves / a.kw) * a.rows_per_wave;
-    a.nblocks = (int)((p.n + a.rows_per_wg - 1) / a.rows_per_wg);
-    a.alpha = p.alpha;
-    a.scale_mul = p.format == TLHIP_FMT_INT8_GROUPED ? (1.0f / 127.0f) : 1.0f;
-    a.y_dtype = p.y_dtype;
-    a.epi = p.epi;
-    // LDS: staged x (mt rows) + split-K partials
-    const int chunk_x_bytes = cw * xbytes;
-    const size_t partial_bytes = a.kw > 1 ? (size_t)a.kw * a.rows_per_wg * mt * sizeof(float) : 0;
-    const size_t lds_bytes = (size_t)mt * chunk_x_bytes * a.nchunks + partial_bytes;
-    const int threads = waves * 64;
-    const int cus = device_cu_count();
-    // resident workgroups per CU: bounded by 2048 lanes and by LDS
-    int per_cu = 2048 / threads;
-    const int by_lds = (int)((160 * 1024) / (lds_bytes ? lds_bytes : 1));
-    if (by_lds < per_cu) per_cu = by_lds < 1 ? 1 : by_lds;
-    if (per_cu < 1) per_cu = 1;
-    int grid = a.nblocks < cus * per_cu ? a.nblocks : cus * per_cu;
-    if (grid < 1) grid = 1;
+    int mt, threads, grid;
+    size_t lds_bytes;
+    fill_args(p, c, m0, mrows, a, mt, threads, grid, lds_bytes);
+    const int r = c.p1, unroll = c.p4 == 0 ? 2 : c.p4;
     int rc;
     switch (p.format) {
       case TLHIP_FMT_INT4_GROUPED:
@@ -570,6 +609,100 @@ int launch_gemv(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t st
     TLHIP_CHECK_HIP(hipGetLastError());
   }
   count_gemv_dispatch();
+  return TLHIP_OK;
+}
+
+// Grouped launch: see gemv_grouped_kernel.  M = 1, f16 activations, and (rows per
+// lane group, chunks in flight) = (1,2) or (2,2) are built.
+bool gemv_group_compatible(const Problem* ps, int count, const tlhip_kernel_config_t& c, const char** why) {
+  static const char* reasons[] = {
+      "a group holds 1..4 problems",
+      "grouped launches are built for M = 1 and f16 activations",
+      "all problems of a group must share format, group size, K and output type",
+      "grouped launches are built for (rows per lane group, chunks in flight) = (1,2) or (2,2)",
+  };
+  auto fail = [&](int i) {
+    if (why) *why = reasons[i];
+    return false;
+  };
+  if (count < 1 || count > kMaxGroup) return fail(0);
+  for (int i = 0; i < count; ++i) {
+    if (ps[i].m != 1 || ps[i].x_dtype != TLHIP_F16) return fail(1);
+    if (ps[i].format != ps[0].format || ps[i].group_size != ps[0].group_size || ps[i].k != ps[0].k ||
+        ps[i].y_dtype != ps[0].y_dtype)
+      return fail(2);
+    if (!gemv_config_applicable(ps[i], c, why)) return false;
+  }
+  const int u = c.p4 == 0 ? 2 : c.p4;
+  if (u != 2 || (c.p1 != 1 && c.p1 != 2)) return fail(3);
+  return true;
+}
+
+template <int FMT, int R>
+static int launch_grouped_t(const GroupedGemvArgs& g, int threads, size_t lds_bytes, hipStream_t stream) {
+  const void* fn = (const void*)gemv_grouped_kernel<FMT, _Float16, 1, R, 2>;
+  if (lds_bytes > 64 * 1024)
+    TLHIP_CHECK_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+  void* args[] = {(void*)&g};
+  TLHIP_CHECK_HIP(hipLaunchKernel(fn, dim3(g.first[g.count]), dim3(threads), args, lds_bytes, stream));
+  return TLHIP_OK;
+}
+
+int launch_gemv_grouped(const Problem* ps, int count, const tlhip_kernel_config_t& c, hipStream_t stream) {
+  const char* why = nullptr;
+  if (!gemv_group_compatible(ps, count, c, &why))
+    return set_error(TLHIP_ERR_INVALID, "gemv_grouped: %s", why ? why : "?");
+  GroupedGemvArgs g;
+  g.count = 0;
+  g.first[0] = 0;
+  int threads = 0;
+  size_t lds_bytes = 0;
+  // every problem gets the workgroups it would get alone, scaled down together if
+  // the sum exceeds what is resident at once
+  int grids[kMaxGroup], total = 0, resident = 0;
+  for (int i = 0; i < count; ++i) {
+    if (ps[i].n == 0) continue;
+    int mt, grid;
+    size_t lds;
+    fill_args(ps[i], c, 0, 1, g.p[g.count], mt, threads, grid, lds);
+    lds_bytes = lds > lds_bytes ? lds : lds_bytes;
+    const int cus = device_cu_count();
+    int per_cu = 2048 / threads;
+    const int by_lds = (int)((160 * 1024) / (lds ? lds : 1));
+    if (by_lds < per_cu) per_cu = by_lds < 1 ? 1 : by_lds;
+    resident = cus * per_cu;
+    grids[g.count] = grid;
+    total += grid;
+    ++g.count;
+  }
+  if (g.count == 0) return TLHIP_OK;
+  for (int i = 0; i < g.count; ++i) {
+    int grid = grids[i];
+    if (total > resident) {
+      grid = (int)((int64_t)grid * resident / total);
+      if (grid < 1) grid = 1;
+    }
+    g.first[i + 1] = g.first[i] + grid;
+  }
+  int rc;
+  const int r = c.p1;
+  switch (ps[0].format) {
+    case TLHIP_FMT_INT4_GROUPED:
+      rc = r == 1 ? launch_grouped_t<TLHIP_FMT_INT4_GROUPED, 1>(g, threads, lds_bytes, stream)
+                  : launch_grouped_t<TLHIP_FMT_INT4_GROUPED, 2>(g, threads, lds_bytes, stream);
+      break;
+    case TLHIP_FMT_INT8_GROUPED:
+      rc = r == 1 ? launch_grouped_t<TLHIP_FMT_INT8_GROUPED, 1>(g, threads, lds_bytes, stream)
+                  : launch_grouped_t<TLHIP_FMT_INT8_GROUPED, 2>(g, threads, lds_bytes, stream);
+      break;
+    default:
+      rc = r == 1 ? launch_grouped_t<TLHIP_FMT_INT8_ROW, 1>(g, threads, lds_bytes, stream)
+                  : launch_grouped_t<TLHIP_FMT_INT8_ROW, 2>(g, threads, lds_bytes, stream);
+      break;
+  }
+  if (rc) return rc;
+  TLHIP_CHECK_HIP(hipGetLastError());
+  for (int i = 0; i < g.count; ++i) count_gemv_dispatch();
   return TLHIP_OK;
 }
 
