@@ -261,26 +261,11 @@ __global__ __launch_bounds__(MAXT) void gemv_mfma_kernel(const MfmaArgs a) {
     }
   };
 
-  // Combine the K parts of the workgroup (through LDS when kw > 1) and of the
-  // other workgroups (through the workspace when ks > 1), apply the epilogue, store.
-  auto finish = [&](int wb) {
-    const int rb = wb * a.blocks_per_wg + bw_idx;
-    if (a.kw > 1) {
-      lds_barrier();  // the previous round's readers are done with `partial`
-#pragma unroll
-      for (int r = 0; r < 4; ++r) partial[(wave * 16 + (4 * g + r)) * 16 + nl] = acc[r];
-      lds_barrier();
-      if (kw_idx == 0) {
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          float s = 0.f;
-          for (int w = 0; w < a.kw; ++w) s += partial[((wave + w) * 16 + (4 * g + r)) * 16 + nl];
-          acc[r] = s;
-        }
-      }
-    }
-    bool owner = kw_idx == 0 && rb < a.nblocks;  // wave-uniform
-    if (owner && a.ks > 1) {
+  // One finished 16 x 16 tile (all of this workgroup's K): combine with the other
+  // workgroups' K slices when ks > 1, apply the epilogue, store.
+  auto emit = [&](int rb, float4_t t) {
+    bool owner = true;  // wave-uniform
+    if (a.ks > 1) {
       // Publish this slice's tile; the workgroup that arrives last for the row
       // block adds the ks tiles in slice order (so the sum does not depend on
       // who is last), resets the counter for the next launch and stores.
@@ -292,7 +277,7 @@ __global__ __launch_bounds__(MAXT) void gemv_mfma_kernel(const MfmaArgs a) {
       float* mine = a.workspace + ((size_t)rb * a.ks + slice) * 256;
 #pragma unroll
       for (int r = 0; r < 4; ++r)
-        __hip_atomic_store(mine + (4 * g + r) * 16 + nl, acc[r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(mine + (4 * g + r) * 16 + nl, t[r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
       __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): every store of this wave is acknowledged
       int old = 0;
@@ -304,10 +289,10 @@ __global__ __launch_bounds__(MAXT) void gemv_mfma_kernel(const MfmaArgs a) {
         const float* tiles = a.workspace + (size_t)rb * a.ks * 256;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          float s = 0.f;
+          float sum = 0.f;
           for (int sl = 0; sl < a.ks; ++sl)
-            s += __hip_atomic_load(tiles + sl * 256 + (4 * g + r) * 16 + nl, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          acc[r] = s;
+            sum += __hip_atomic_load(tiles + sl * 256 + (4 * g + r) * 16 + nl, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          t[r] = sum;
         }
         if (lane == 0) __hip_atomic_store(a.counters + rb, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
@@ -321,12 +306,31 @@ __global__ __launch_bounds__(MAXT) void gemv_mfma_kernel(const MfmaArgs a) {
         for (int r = 0; r < 4; ++r) {
           const int m = 4 * g + r;
           if (m < mrows) {
-            const float v = apply_epilogue(a.epi, acc[r] * rs, orow);
+            const float v = apply_epilogue(a.epi, t[r] * rs, orow);
             store_out(a.y, a.y_dtype, (int64_t)m * a.n + orow, v);
           }
         }
       }
     }
+  };
+
+  // End of a row block for this wave.  kw == 1: the wave owns the block, emit it.
+  // kw > 1: park the wave's partial tile in LDS slot (round, wave) and go on; the
+  // kw tiles of every block are combined after the main loop, behind ONE barrier.
+  // (A combine per row block cost two barriers, i.e. two waits for the slowest
+  // wave's memory latency, and with K slices one drain of the load pipeline, per
+  // block: 3 us of a 12 us kernel, 6 us with four K slices.)
+  int round = 0;
+  auto finish = [&](int wb) {
+    if (a.kw == 1) {
+      const int rb = wb * a.blocks_per_wg + bw_idx;
+      if (rb < a.nblocks) emit(rb, acc);
+    } else {
+      float* tile = partial + (size_t)(round * (int)(blockDim.x >> 6) + wave) * 256;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) tile[(4 * g + r) * 16 + nl] = acc[r];
+    }
+    ++round;
     acc = (float4_t){0.f, 0.f, 0.f, 0.f};
   };
 
@@ -415,11 +419,62 @@ __global__ __launch_bounds__(MAXT) void gemv_mfma_kernel(const MfmaArgs a) {
   } else if (total - j == 1) {
     consume(cur, wgb, step);
   }
+
+  if (a.kw > 1) {
+    // the parked tiles: rounds x blocks_per_wg of them, dealt to the waves
+    lds_barrier();
+    const int waves = (int)(blockDim.x >> 6);
+    const int bshift = __builtin_ctz((unsigned)a.blocks_per_wg);
+    const int wgb0 = (int)(blockIdx.x >> a.ks_shift);
+    for (int t = wave; t < (rounds << bshift); t += waves) {
+      const int r = t >> bshift, b = t & (a.blocks_per_wg - 1);
+      const int rb = (wgb0 + r * wg_stride) * a.blocks_per_wg + b;
+      if (rb >= a.nblocks) continue;  // wave-uniform
+      const float* tiles = partial + (size_t)(r * waves + b * a.kw) * 256;
+      float4_t sum = {0.f, 0.f, 0.f, 0.f};
+      for (int w = 0; w < a.kw; ++w) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) sum[q] += tiles[w * 256 + (4 * g + q) * 16 + nl];
+      }
+      emit(rb, sum);
+    }
+  }
 }
 
 }  // namespace
 
 static constexpr size_t kXLdsBudget = 160 * 1024;
+
+// Grid and LDS of a launch.  With kw > 1 every workgroup parks one tile per
+// (round, wave) in LDS, so LDS grows with the rounds a workgroup walks, the rounds
+// shrink with the grid, and the grid is bounded by what LDS lets reside: take the
+// most workgroups per CU for which it closes.
+struct MfmaGeometry {
+  int grid;
+  size_t lds_bytes;
+};
+static bool mfma_geometry(int64_t n, int64_t k, int64_t m, int waves, int kw, int ks, MfmaGeometry* out) {
+  const int threads = waves * 64;
+  const int64_t nblocks = (n + 15) / 16;
+  const int blocks_per_wg = waves / kw;
+  const int64_t nwgblocks = (nblocks + blocks_per_wg - 1) / blocks_per_wg;
+  const size_t x_bytes = (size_t)m * (k / ks * 2 + 16);
+  const int cus = device_cu_count() > 0 ? device_cu_count() : 256;
+  for (int per_cu = 2048 / threads; per_cu >= 1; --per_cu) {
+    int64_t sets = (int64_t)cus * per_cu / ks;
+    if (sets > nwgblocks) sets = nwgblocks;
+    if (sets < 1) sets = 1;
+    const int64_t rounds = (nwgblocks + sets - 1) / sets;
+    const size_t parked = kw > 1 ? (size_t)rounds * waves * 1024 : 0;
+    const size_t lds = x_bytes + parked;
+    if (lds * per_cu <= kXLdsBudget) {
+      out->grid = (int)(sets * ks);
+      out->lds_bytes = lds;
+      return true;
+    }
+  }
+  return false;
+}
 
 bool gemv_mfma_config_applicable(const Problem& p, const tlhip_kernel_config_t& c, const char** why) {
   static const char* reasons[] = {
@@ -431,7 +486,7 @@ bool gemv_mfma_config_applicable(const Problem& p, const tlhip_kernel_config_t& 
       "group size must be a multiple of 32 (int4) or 64 (int8)",
       "iterations in flight must be 1, 2 or 4",
       "K-split waves must be a power of two that divides the waves per workgroup",
-      "activations (M x K/slices f16) do not fit LDS",
+      "activations (M x K/slices f16) plus one parked tile per round and wave do not fit LDS",
       "K slices must be a power of two (1..16) that divides K/128 (int4) or K/64 (int8)",
       "K slices need more partial-tile workspace or counters than the library holds",
       "iterations in flight must divide the 128-weight (int4) or 64-weight (int8) steps of a K slice",
@@ -455,7 +510,8 @@ bool gemv_mfma_config_applicable(const Problem& p, const tlhip_kernel_config_t& 
   const int ks = c.p3 < 1 ? 1 : c.p3;
   const int64_t iters = p.k / kper;
   if (ks > 16 || (ks & (ks - 1)) != 0 || iters % ks != 0) return fail(9);
-  if ((size_t)p.m * (p.k / ks * 2 + 16) + (size_t)c.p0 * 1024 > kXLdsBudget) return fail(8);
+  MfmaGeometry geo;
+  if (!mfma_geometry(p.n, p.k, p.m, c.p0, kw, ks, &geo)) return fail(8);
   if ((iters / ks) % c.p1 != 0) return fail(11);
   if (ks > 1) {
     const int64_t nblocks = (p.n + 15) / 16;
@@ -524,18 +580,12 @@ int launch_gemv_mfma(const Problem& p, const tlhip_kernel_config_t& c, hipStream
   a.scale_mul = p.format == TLHIP_FMT_INT8_GROUPED ? (1.0f / 127.0f) : 1.0f;
   a.y_dtype = p.y_dtype;
   a.epi = p.epi;
-  const size_t partial_bytes = (size_t)waves * 256 * sizeof(float);
-  const size_t lds_bytes = (size_t)a.m * (p.k / a.ks * 2 + 16) + partial_bytes;
+  MfmaGeometry geo;
+  if (!mfma_geometry(p.n, p.k, p.m, waves, a.kw, a.ks, &geo))
+    return set_error(TLHIP_ERR_INVALID, "gemv_mfma: launch geometry does not close");
+  const size_t lds_bytes = geo.lds_bytes;
   const int threads = waves * 64;
-  const int cus = device_cu_count();
-  int per_cu = 2048 / threads;
-  const int by_lds = (int)((160 * 1024) / lds_bytes);
-  if (by_lds < per_cu) per_cu = by_lds < 1 ? 1 : by_lds;
-  // resident workgroups only, in whole sets of ks; never more sets than row-block groups
-  int sets = cus * per_cu / a.ks;
-  if (sets > a.nwgblocks) sets = a.nwgblocks;
-  if (sets < 1) sets = 1;
-  const int grid = sets * a.ks;
+  const int grid = geo.grid;
   int rc;
   switch (p.format) {
     case TLHIP_FMT_INT4_GROUPED:
