@@ -352,3 +352,36 @@ def test_grouped_gemv_rejects_mixed_shapes(be):
     with pytest.raises(ValueError, match="one f16 activation row"):
         be.linearGrouped(x2, [w1])
     del w2
+
+
+def test_k_slices_are_stable_over_many_back_to_back_launches(be):
+    """The cross-workgroup combine relies on device-scope atomics for its tiles and
+    counters: 300 back-to-back launches over rotating weights (so nothing stays in
+    cache) must each reproduce, bit for bit, what the same weight gave the first time,
+    and the unsliced kernel's answer to f32 accumulation order."""
+    rng = np.random.default_rng(77)
+    n, k, m, g = 4096, 12288, 16, 32
+    x = make_x(m, k, "f16", rng)
+    xt = be.ops.tensorFromArray(x, [m, k], "f16")
+    ws = []
+    for _ in range(3):
+        packed = rng.integers(0, 2**32, n * k // 8, dtype=np.uint64).astype(np.uint32)
+        scales = rng.uniform(0.01, 0.05, n * k // g).astype(np.float16).view(np.uint16)
+        ws.append(be.createQuantizedWeight(packed, scales, n, k, T.resolveWeightFormat("int4-32", "f32")))
+    sliced = L.KernelConfig.of(1, 8, 2, 4, 4)
+    firsts = [None] * 3
+    outs = []
+    for it in range(300):
+        outs.append((it % 3, be.linear(xt, ws[it % 3], config=sliced)))
+        if len(outs) == 30 or it == 299:
+            for wi, y in outs:
+                got = y.numpy()
+                y.destroy()
+                if firsts[wi] is None:
+                    firsts[wi] = got
+                assert np.array_equal(got, firsts[wi]), it
+            outs = []
+    valu = L.KernelConfig.of(0, 32, 1, 8, 1, 2)
+    for wi in range(3):
+        ref = be.linear(xt, ws[wi], config=valu).numpy()
+        assert rel_l2(firsts[wi], ref) <= 2e-6
