@@ -301,7 +301,7 @@ def main() -> int:
                 "shape": {"m": dominant["m"], "n": dominant["n"], "k": dominant["k"]}}
 
     result = {
-        "metric": "quant-GEMV HBM GB/s (% peak) + us/decode-token for linears; prefill TFLOP/s",
+        "metric": "quant-GEMV HBM GB/s (% peak) + \u00b5s/decode-token for linears; prefill TFLOP/s",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(step_us / 1e3, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16 x int4 -> f32 accumulate", "data": "synthetic",
