@@ -347,6 +347,16 @@ def main() -> int:
                        "config": list(cfg.as_tuple())})
             out.destroy()
         details["lm_head_int8_row_256000x2304"] = lm
+        # the LM head's consumer: device top-k of the 256 000 logits (k = 64), 512 B read back
+        logits = be._alloc([256000], "f32")
+        tv, ti = be._alloc([64], "f32"), be._alloc([64], "i32")
+        L.call("tlhip_topk", logits.ptr, 0, 256000, 64, tv.ptr, ti.ptr, L.I32, None)  # first use allocates workspace
+
+        def topk_call():
+            L.call("tlhip_topk", logits.ptr, 0, 256000, 64, tv.ptr, ti.ptr, L.I32, None)
+        details["lm_head_topk64_of_256000"] = {"us": round(B.median_time(topk_call, 50), 2)}
+        for t in (logits, tv, ti):
+            t.destroy()
         us = B.probe_time(lm_pool, 256000 * 2304)
         details["read_only_probe"]["256000x2304"] = {"bytes": 256000 * 2304, "us": round(us, 2),
                                                      "gbps": round(256000 * 2304 / us / 1e3, 1)}

@@ -50,7 +50,7 @@ typedef enum {
 } tlhip_format_t;
 
 /* DType subset used on this path (src/backend/types.ts DType "f32" | "f16"). */
-typedef enum { TLHIP_F32 = 0, TLHIP_F16 = 1 } tlhip_dtype_t;
+typedef enum { TLHIP_F32 = 0, TLHIP_F16 = 1, TLHIP_I32 = 2 } tlhip_dtype_t;
 
 /* Unary epilogue ops: the GEMV epilogue vocabulary
  * (src/backend/webgpu/matmul/gemv.ts:135-143); formulas from
@@ -234,6 +234,16 @@ int tlhip_cast(const void* in, int in_dtype, void* out, int out_dtype, int64_t c
  * a GEMV launch of the same size, it gives the rate a single launch of that size
  * can reach at all.  `sink4` is 4 writable device bytes. */
 int tlhip_hbm_read_probe(const void* ptr, size_t bytes, void* sink4, tlhip_stream_t stream);
+
+/* Top-k of logits[offset .. offset+length) (f32, device): the k largest values in
+ * descending order, ties towards the smaller index, NaN below every number;
+ * out_values f32[k], out_indices [k] relative to `offset`, as TLHIP_I32 or (the
+ * packed form deviceTopK returns) TLHIP_F32; device pointers.  Fewer than k
+ * elements: the rest is (-3.4028234e38, -1).  The sampling
+ * prefilter readTopK / deviceTopK (src/backend/types.ts:632-634, 669-678;
+ * src/backend/webgpu/topk-kernel.ts): the consumer of the LM-head GEMV. */
+int tlhip_topk(const float* logits, int64_t offset, int64_t length, int k, float* out_values,
+               void* out_indices, int index_dtype, tlhip_stream_t stream);
 
 /* ---- kernel choice: variant registry + autotuner
  * (src/backend/webgpu/matmul/variants.ts:54-260; autotune.ts:48-547;

@@ -17,7 +17,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("TLHIP_LIBRARY") or os.path.join(_HERE, "libtlhip.so")
 
 FMT_INT8_GROUPED, FMT_INT8_ROW, FMT_INT4_GROUPED = 0, 1, 2
-F32, F16 = 0, 1
+F32, F16, I32 = 0, 1, 2
 UNARY = {"none": 0, "relu": 1, "silu": 2, "gelu": 3, "gelu_tanh": 3, "gelu_erf": 4,
          "sigmoid": 5, "tanh": 6}
 EPI_NONE, EPI_BIAS, EPI_UNARY = 0, 1, 2
@@ -110,6 +110,7 @@ SIGNATURES = {
     "tlhip_bias_add": (_i, [_vp, _i, _vp, _i, _vp, _i64, _i64, _vp]),
     "tlhip_unary": (_i, [_i, _vp, _i, _vp, _i64, _vp]),
     "tlhip_cast": (_i, [_vp, _i, _vp, _i, _i64, _vp]),
+    "tlhip_topk": (_i, [_vp, _i64, _i64, _i, _vp, _vp, _i, _vp]),
     "tlhip_hbm_read_probe": (_i, [_vp, _sz, _vp, _vp]),
     "tlhip_candidate_count": (_i, [_QW, _i, _i64, _i, C.POINTER(_i)]),
     "tlhip_candidate_get": (_i, [_QW, _i, _i64, _i, _i, _KC]),

@@ -383,6 +383,31 @@ class HipBackend:
         self._state.extend([packedT, scalesT, logical])
         return logical
 
+    def readTopK(self, a: HipTensor, k: int, offset: int = 0, length: Optional[int] = None):
+        """types.ts:669-678: the top-k (values descending, ties to the smaller index)
+        of a contiguous f32 tensor (or of [offset, offset+length) of it), selected on
+        the device; only 2k numbers are read back."""
+        if a.dtype != "f32" or not a.isContiguous:
+            raise ValueError("readTopK: a contiguous f32 tensor")
+        length = a.size - offset if length is None else length
+        if offset < 0 or length < 0 or offset + length > a.size:
+            raise ValueError("readTopK: range outside the tensor")
+        vals, idx = self._alloc([k], "f32"), self._alloc([k], "i32")
+        L.call("tlhip_topk", a.ptr, offset, length, k, vals.ptr, idx.ptr, L.I32, self.stream)
+        v, i = self._download(vals), self._download(idx)
+        vals.destroy()
+        idx.destroy()
+        return v, i
+
+    def deviceTopK(self, logits: HipTensor, k: int) -> HipTensor:
+        """types.ts:632-634: [.., V] -> packed [1, 2, k] on the device, row 0 the
+        values (descending), row 1 the token ids as f32."""
+        if logits.dtype != "f32" or not logits.isContiguous:
+            raise ValueError("deviceTopK: a contiguous f32 logits row")
+        out = self._alloc([1, 2, k], "f32")
+        L.call("tlhip_topk", logits.ptr, 0, logits.size, k, out.ptr, out.ptr + 4 * k, L.F32, self.stream)
+        return out
+
     def dequantizeToF32(self, w: HipTensor) -> HipTensor:
         """Explicit dequant of a packed weight to f32 [N,K] on the device
         (quantize.ts:138-156; matmul/dispatch.ts:949-1037)."""
