@@ -8,15 +8,15 @@
 // Every element becomes a 64-bit key, (order-preserving bits of the value) << 32 |
 // (0xffffffff - index), so that "larger key" is exactly "larger value, then smaller
 // index"; NaN maps below every number.  A workgroup sorts up to 4096 keys in LDS
-// (bitonic, descending) and keeps the first k; levels repeat (4096 -> k per
-// workgroup) until one workgroup holds the answer.  One level covers
-// 4096 * 4096 / k elements, i.e. 262 144 at k = 64.  HBM traffic: the row once.
+// (bitonic, descending) and keeps the first k; levels repeat (chunk -> k per
+// workgroup) until one workgroup holds the answer.  Chunks of 1024 keys for
+// k <= 256 (many small sorts, every CU busy: 250 + 16 + 1 workgroups for 256 000
+// logits at k = 64), of 4096 above.  HBM traffic: the row once.
 #include "device_utils.h"
 
 namespace tlhip {
 namespace {
 
-constexpr int kTopkChunk = 4096;
 constexpr float kTopkNegInf = -3.4028234e38f;  // the reference's filler for missing entries
 
 __device__ __forceinline__ uint64_t topk_key(float v, uint32_t index) {
@@ -35,15 +35,17 @@ __device__ __forceinline__ float topk_value(uint64_t key) {
 // FROM_FLOAT: keys are made from `logits[offset + i]` with index i; else read from `keys_in`.
 // The first `k` keys of the sorted chunk go to keys_out[block * k ..]; with `final`
 // they are decoded into values / indices instead.
-template <bool FROM_FLOAT>
-__global__ __launch_bounds__(256) void topk_level_kernel(const float* __restrict__ logits, int64_t offset,
+template <bool FROM_FLOAT, int kTopkChunk>
+__global__ __launch_bounds__(kTopkChunk / 4) void topk_level_kernel(const float* __restrict__ logits, int64_t offset,
                                                         const uint64_t* __restrict__ keys_in, int64_t count, int k,
                                                         uint64_t* __restrict__ keys_out, int final,
                                                         float* __restrict__ out_values,
                                                         void* __restrict__ out_indices, int index_dtype) {
   __shared__ uint64_t keys[kTopkChunk];
   const int64_t base = (int64_t)blockIdx.x * kTopkChunk;
-  for (int i = threadIdx.x; i < kTopkChunk; i += 256) {
+  constexpr int THREADS = kTopkChunk / 4;
+#pragma unroll
+  for (int i = threadIdx.x; i < kTopkChunk; i += THREADS) {
     const int64_t e = base + i;
     uint64_t key = 0;  // padding sorts last: the index part of a real key is at least 1
     if (e < count) key = FROM_FLOAT ? topk_key(logits[offset + e], (uint32_t)e) : keys_in[e];
@@ -53,20 +55,19 @@ __global__ __launch_bounds__(256) void topk_level_kernel(const float* __restrict
   // bitonic sort, descending
   for (int size = 2; size <= kTopkChunk; size <<= 1) {
     for (int stride = size >> 1; stride > 0; stride >>= 1) {
-      for (int t = threadIdx.x; t < kTopkChunk / 2; t += 256) {
-        const int lo = 2 * t - (t & (stride - 1));
-        const int hi = lo + stride;
-        const bool descending = (lo & size) == 0;
-        const uint64_t a = keys[lo], b = keys[hi];
-        if ((a < b) == descending) {
-          keys[lo] = b;
-          keys[hi] = a;
-        }
-      }
+      // two compare-exchanges per thread, both pairs read before either is written
+      const int t0 = threadIdx.x, t1 = threadIdx.x + THREADS;
+      const int lo0 = 2 * t0 - (t0 & (stride - 1)), lo1 = 2 * t1 - (t1 & (stride - 1));
+      const uint64_t a0 = keys[lo0], b0 = keys[lo0 + stride], a1 = keys[lo1], b1 = keys[lo1 + stride];
+      const bool swap0 = (a0 < b0) == ((lo0 & size) == 0), swap1 = (a1 < b1) == ((lo1 & size) == 0);
+      keys[lo0] = swap0 ? b0 : a0;
+      keys[lo0 + stride] = swap0 ? a0 : b0;
+      keys[lo1] = swap1 ? b1 : a1;
+      keys[lo1 + stride] = swap1 ? a1 : b1;
       __syncthreads();
     }
   }
-  for (int i = threadIdx.x; i < k; i += 256) {
+  for (int i = threadIdx.x; i < k; i += THREADS) {
     const uint64_t key = keys[i];
     if (final) {
       const bool real = key != 0;
@@ -97,8 +98,9 @@ extern "C" int tlhip_topk(const float* logits, int64_t offset, int64_t length, i
   hipStream_t s = resolve_stream(stream);
   // level 0 reads the floats; later levels read the keys the level before wrote
   // into the stream's workspace, alternating between its two halves
+  const int chunk = k <= 256 ? 1024 : 4096;
   int64_t count = length;
-  int64_t blocks = (count + kTopkChunk - 1) / kTopkChunk;
+  int64_t blocks = (count + chunk - 1) / chunk;
   if (blocks < 1) blocks = 1;
   float* ws = nullptr;
   int* counters = nullptr;
@@ -116,17 +118,25 @@ extern "C" int tlhip_topk(const float* logits, int64_t offset, int64_t length, i
   while (true) {
     const int final = blocks == 1;
     uint64_t* keys_out = final ? nullptr : bufs[level & 1];
-    if (level == 0)
-      hipLaunchKernelGGL(topk_level_kernel<true>, dim3((unsigned)blocks), dim3(256), 0, s, logits, offset, nullptr,
-                         count, k, keys_out, final, out_values, out_indices, index_dtype);
+    const dim3 grid((unsigned)blocks), threads(chunk / 4);
+    const int64_t zero = 0;
+    if (level == 0 && chunk == 1024)
+      hipLaunchKernelGGL((topk_level_kernel<true, 1024>), grid, threads, 0, s, logits, offset, nullptr, count, k,
+                         keys_out, final, out_values, out_indices, index_dtype);
+    else if (level == 0)
+      hipLaunchKernelGGL((topk_level_kernel<true, 4096>), grid, threads, 0, s, logits, offset, nullptr, count, k,
+                         keys_out, final, out_values, out_indices, index_dtype);
+    else if (chunk == 1024)
+      hipLaunchKernelGGL((topk_level_kernel<false, 1024>), grid, threads, 0, s, nullptr, zero, keys_in, count, k,
+                         keys_out, final, out_values, out_indices, index_dtype);
     else
-      hipLaunchKernelGGL(topk_level_kernel<false>, dim3((unsigned)blocks), dim3(256), 0, s, nullptr, (int64_t)0, keys_in,
-                         count, k, keys_out, final, out_values, out_indices, index_dtype);
+      hipLaunchKernelGGL((topk_level_kernel<false, 4096>), grid, threads, 0, s, nullptr, zero, keys_in, count, k,
+                         keys_out, final, out_values, out_indices, index_dtype);
     TLHIP_CHECK_HIP(hipGetLastError());
     if (final) break;
     keys_in = keys_out;
     count = blocks * k;
-    blocks = (count + kTopkChunk - 1) / kTopkChunk;
+    blocks = (count + chunk - 1) / chunk;
     ++level;
   }
   return TLHIP_OK;
