@@ -441,6 +441,61 @@ def main() -> int:
         L.call("tlhip_graph_end_capture", None, C.byref(graph))
         us_grouped_graph = B.median_time(replay, 5)
         L.call("tlhip_graph_destroy", graph)
+        # the same token with the producers of the Linears' inputs: RMSNorm in front of
+        # (q, k, v) and of (gate, up), silu(gate) * up in front of down.  Apart: 7
+        # launches per layer; fused into the GEMVs' activation staging: still 4.
+        nw = be.ops.tensorFromArray(np.ones(1024, np.float32), [1024], "f32")
+        xn = be._alloc([1, 1024], "f16")
+        act = be._alloc([1, 3072], "f16")
+        lib = L.load()
+        pro_norm = L.Prologue(L.PRO_RMSNORM, 0, 1e-6, 0, nw.ptr)
+        pro_gate = L.Prologue(L.PRO_GATED_MUL, L.UNARY["silu"], 0.0, 0, lout2["up"].ptr)
+
+        def chk(rc):
+            if rc:
+                L.check(rc)
+
+        def token_producers_apart():
+            for i in range(0, len(gcalls), 4):
+                (pq, nq), (po, no), (pg, ng), (pd, nd) = gcalls[i:i + 4]
+                chk(lib.tlhip_rmsnorm(lx[1024].ptr, L.F16, nw.ptr, xn.ptr, L.F16, 1, 1024, 1e-6, None))
+                chk(gfn(pq, nq, L.F16, L.F16, 1.0, None))
+                chk(gfn(po, no, L.F16, L.F16, 1.0, None))
+                chk(lib.tlhip_rmsnorm(lx[1024].ptr, L.F16, nw.ptr, xn.ptr, L.F16, 1, 1024, 1e-6, None))
+                chk(gfn(pg, ng, L.F16, L.F16, 1.0, None))
+                chk(lib.tlhip_gated_mul(L.UNARY["silu"], lout2["gate"].ptr, lout2["up"].ptr, L.F16, act.ptr, 3072, None))
+                chk(gfn(pd, nd, L.F16, L.F16, 1.0, None))
+
+        gpro = lib.tlhip_gemv_grouped_prologue
+        down_x = []
+        for i in range(3, len(gcalls), 4):
+            # the down projection reads the gate row; `up` arrives through the prologue
+            probs = (L.GemvProblem * 1)()
+            probs[0] = gcalls[i][0][0]
+            probs[0].x = lout2["gate"].ptr
+            down_x.append(probs)
+
+        def token_producers_fused():
+            for j, i in enumerate(range(0, len(gcalls), 4)):
+                (pq, nq), (po, no), (pg, ng), _ = gcalls[i:i + 4]
+                chk(gpro(pq, nq, C.byref(pro_norm), L.F16, L.F16, 1.0, None))
+                chk(gfn(po, no, L.F16, L.F16, 1.0, None))
+                chk(gpro(pg, ng, C.byref(pro_norm), L.F16, L.F16, 1.0, None))
+                chk(gpro(down_x[j], 1, C.byref(pro_gate), L.F16, L.F16, 1.0, None))
+
+        producer_us = {}
+        for name, fn in (("apart", token_producers_apart), ("fused", token_producers_fused)):
+            fn()
+            L.call("tlhip_graph_begin_capture", None)
+            fn()
+            L.call("tlhip_graph_end_capture", None, C.byref(graph))
+            producer_us[name] = B.median_time(replay, 5)
+            L.call("tlhip_graph_destroy", graph)
+        details["qwen3_0p6b_decode_token_with_producers"] = {
+            "what": "28 layers: rmsnorm -> (q,k,v), o, rmsnorm -> (gate,up), silu(gate)*up -> down; HIP graph",
+            "launches_apart": 28 * 7, "us_per_token_apart": round(producer_us["apart"], 1),
+            "launches_fused": 28 * 4, "us_per_token_fused": round(producer_us["fused"], 1)}
+
         details["qwen3_0p6b_decode_token"] = {
             "gemvs": len(calls), "bytes": token_bytes, "us_per_token_stream": round(us_stream, 1),
             "us_per_token_graph": round(us_graph, 1), "gbps_stream": round(token_bytes / us_stream / 1e3, 1),

@@ -33,6 +33,7 @@ extern "C" {
 #define TLHIP_ERR_INVALID 1 /* bad argument / unsupported combination */
 #define TLHIP_ERR_DEVICE 2  /* a HIP call failed */
 #define TLHIP_ERR_STATE 3   /* library not initialised */
+#define TLHIP_ERR_UNSUPPORTED 4 /* valid request that no built kernel covers; the caller has a fallback */
 
 typedef void* tlhip_stream_t;
 typedef void* tlhip_event_t;
@@ -228,6 +229,47 @@ int tlhip_bias_add(const void* in, int dtype, const void* bias, int bias_dtype, 
 int tlhip_unary(int op, const void* in, int dtype, void* out, int64_t count, tlhip_stream_t stream);
 int tlhip_cast(const void* in, int in_dtype, void* out, int out_dtype, int64_t count,
                tlhip_stream_t stream);
+
+/* The two steps that produce a decode Linear's input (the GEMV's x).
+ * rmsnorm: y[r,:] = x[r,:] * rsqrt(mean(x[r,:]^2) + eps) * weight, f32 arithmetic;
+ *   fusedRMSNormForward (src/backend/types.ts:635-640, the kernel in
+ *   src/backend/webgpu/rmsnorm-kernel.ts:31-66; CPU form
+ *   src/frontend/decomposed-ops.ts:221-233).  x [m,d] of x_dtype, weight f32 [d],
+ *   y [m,d] of y_dtype.
+ * gated_mul: out[i] = unary(gate[i]) * up[i], the MLP's `mul(act(gate), up)`
+ *   (packages/qwen3-browser/src/model.ts:357-361, gemma2-browser model.ts:411-415);
+ *   gate, up and out share `dtype`; f32 arithmetic, one rounding to `dtype`. */
+int tlhip_rmsnorm(const void* x, int x_dtype, const float* weight, void* y, int y_dtype, int64_t m,
+                  int64_t d, float eps, tlhip_stream_t stream);
+int tlhip_gated_mul(int unary, const void* gate, const void* up, int dtype, void* out, int64_t count,
+                    tlhip_stream_t stream);
+
+/* The same two steps fused into the decode GEMV that consumes them: the kernel
+ * stages f(x) instead of x in LDS, so the normalised / gated activations never
+ * travel through HBM and one launch per Linear disappears.
+ *   RMSNORM  : f(x)[m,k] = x[m,k] * rsqrt(mean_k x[m,:]^2 + eps) * operand[k]
+ *              (operand: f32 [K], the norm weight)
+ *   GATED_MUL: f(x)[m,k] = unary(x[m,k]) * operand[m,k]
+ *              (x is the gate, operand the up projection, [m,K] of x_dtype)
+ * With f16 activations f(x) is rounded to f16 once, as the unfused kernel's f16
+ * output would be.  Built into the VALU kernel only: m <= 4; for more rows the
+ * call returns TLHIP_ERR_UNSUPPORTED and the caller runs the two steps apart.
+ * tlhip_gemv_grouped_prologue: the same prologue for every problem of the group
+ * (q/k/v and gate/up share their input). */
+typedef enum { TLHIP_PRO_NONE = 0, TLHIP_PRO_RMSNORM = 1, TLHIP_PRO_GATED_MUL = 2 } tlhip_prologue_kind_t;
+typedef struct {
+  int32_t kind;        /* tlhip_prologue_kind_t */
+  int32_t unary;       /* tlhip_unary_t, GATED_MUL */
+  float eps;           /* RMSNORM */
+  int32_t reserved;
+  const void* operand; /* device; see above */
+} tlhip_prologue_t;
+int tlhip_gemv_prologue(const tlhip_qweight_t* w, const tlhip_prologue_t* prologue, const void* x, int x_dtype,
+                        int64_t m, void* y, int y_dtype, float alpha, const tlhip_epilogue_t* epilogue,
+                        tlhip_stream_t stream);
+int tlhip_gemv_grouped_prologue(const tlhip_gemv_problem_t* problems, int count,
+                                const tlhip_prologue_t* prologue, int x_dtype, int y_dtype, float alpha,
+                                tlhip_stream_t stream);
 
 /* Measuring stick for the decode GEMV (no counterpart in the reference): reads
  * `bytes` bytes at `ptr` once with 16-byte loads and discards them.  Timed like

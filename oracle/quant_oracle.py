@@ -66,6 +66,10 @@ def lib() -> ctypes.CDLL:
         L.ref_unary_scalar.restype = ctypes.c_double
         L.ref_unary_scalar.argtypes = [ci, ctypes.c_double]
         L.ref_max_threads.restype = ci
+        L.ref_mul.argtypes = [vp, vp, vp, i64]
+        L.ref_mul.restype = None
+        L.ref_rmsnorm.argtypes = [vp, vp, vp, i64, i64, ctypes.c_double]
+        L.ref_rmsnorm.restype = None
         for f in ("ref_f32_to_f16_bits_array", "ref_f16_bits_to_f32_array",
                   "ref_dequant_int8_grouped", "ref_dequant_int8_row", "ref_dequant_int4_grouped",
                   "ref_matmul_nt", "ref_matmul_strided", "ref_bias_add", "ref_unary"):
@@ -199,6 +203,32 @@ def unary(op: str, y) -> np.ndarray:
     y = np.array(y, np.float32, copy=True, order="C")
     lib().ref_unary(UNARY[op], _p(y), y.size)
     return y
+
+
+def mul(a, b) -> np.ndarray:
+    a = _c(a, np.float32)
+    b = _c(b, np.float32)
+    assert a.shape == b.shape
+    out = np.empty_like(a)
+    lib().ref_mul(_p(a), _p(b), _p(out), a.size)
+    return out
+
+
+def rmsnorm(x, weight, eps: float = 1e-6) -> np.ndarray:
+    """tensor.rmsnorm on the CPU backend (decomposed-ops.ts:221-233)."""
+    x = _c(x, np.float32)
+    weight = _c(weight, np.float32)
+    d = x.shape[-1]
+    assert weight.shape == (d,)
+    out = np.empty_like(x)
+    lib().ref_rmsnorm(_p(x), _p(weight), _p(out), x.size // d if d else 0, d, float(eps))
+    return out
+
+
+def gated(gate, up, act: str = "silu") -> np.ndarray:
+    """The MLP's `mul(act(gate), up)` as two CPU ops, each storing f32
+    (packages/qwen3-browser/src/model.ts:357-361; gemma2-browser model.ts:411-415)."""
+    return mul(unary(act, gate), up)
 
 
 def linear(x, w_dequant, bias=None, act: str = "none", threads: int = 1) -> np.ndarray:

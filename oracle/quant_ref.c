@@ -26,6 +26,10 @@
  *                            exp/tanh stand in for V8's Math.exp/Math.tanh
  *                            (both < 1 ulp in double; the last double bit is
  *                            "parity unpinned", far below the 1e-3 gate)
+ *   ref_rmsnorm              the rows and closed form of the reference's own test
+ *                            (test/nn-rmsnorm.spec.ts:10-41), unit RMS of the
+ *                            output, invariance under scaling of x, constant rows
+ *   ref_mul                  numpy float32 multiply (bit-exact)
  */
 #include <math.h>
 #include <stdint.h>
@@ -302,6 +306,39 @@ double ref_unary_scalar(int op, double x) {
 
 void ref_unary(int op, float* y, int64_t count) {
   for (int64_t i = 0; i < count; i++) y[i] = (float)ref_unary_scalar(op, (double)y[i]);
+}
+
+/* api.mul on the CPU backend: double product of two f32 values, one f32 store
+ * (numeric.ts binary loop; the product of two f32 is exact in double, so this is
+ * the IEEE f32 product). */
+void ref_mul(const float* a, const float* b, float* out, int64_t count) {
+  for (int64_t i = 0; i < count; i++) out[i] = (float)((double)a[i] * (double)b[i]);
+}
+
+/* rmsnorm(x, weight, eps) on the CPU backend, the decomposed forward of
+ * src/frontend/decomposed-ops.ts:221-233: five ops, each storing f32.
+ *   xSq    = mul(x, x)
+ *   meanSq = mean(xSq, dim=-1)   numeric.ts:1022-1057: the running sum lives in a
+ *            Float32Array cell, so every addition rounds to f32; then f32(sum / D)
+ *   t      = add(meanSq, eps)    eps is a double
+ *   inv    = rsqrt(t)            catalog.ts:96-97: 1 / sqrt(t)
+ *   y      = mul(mul(x, inv), weight) */
+void ref_rmsnorm(const float* x, const float* weight, float* y, int64_t m, int64_t d, double eps) {
+  for (int64_t r = 0; r < m; r++) {
+    const float* xr = x + r * d;
+    float sum = 0.0f;
+    for (int64_t i = 0; i < d; i++) {
+      const float sq = (float)((double)xr[i] * (double)xr[i]);
+      sum = (float)((double)sum + (double)sq);
+    }
+    const float mean = (float)((double)sum / (double)d);
+    const float t = (float)((double)mean + eps);
+    const float inv = (float)(1.0 / sqrt((double)t));
+    for (int64_t i = 0; i < d; i++) {
+      const float nrm = (float)((double)xr[i] * (double)inv);
+      y[r * d + i] = (float)((double)nrm * (double)weight[i]);
+    }
+  }
 }
 
 int ref_max_threads(void) {

@@ -65,6 +65,15 @@ class KernelConfig(C.Structure):
         return cls(*vals)
 
 
+class Prologue(C.Structure):
+    _fields_ = [("kind", C.c_int32), ("unary", C.c_int32), ("eps", C.c_float), ("reserved", C.c_int32),
+                ("operand", C.c_void_p)]
+
+
+PRO_NONE, PRO_RMSNORM, PRO_GATED_MUL = 0, 1, 2
+ERR_INVALID, ERR_DEVICE, ERR_STATE, ERR_UNSUPPORTED = 1, 2, 3, 4
+
+
 class GemvProblem(C.Structure):
     _fields_ = [("w", QWeight), ("x", C.c_void_p), ("y", C.c_void_p), ("epilogue", C.POINTER(Epilogue))]
 
@@ -104,6 +113,10 @@ SIGNATURES = {
     "tlhip_dequant": (_i, [_QW, _vp, _vp]),
     "tlhip_gemv": (_i, [_QW, _vp, _i, _i64, _vp, _i, _f, _EP, _vp]),
     "tlhip_gemv_grouped": (_i, [C.POINTER(GemvProblem), _i, _i, _i, _f, _vp]),
+    "tlhip_gemv_prologue": (_i, [_QW, C.POINTER(Prologue), _vp, _i, _i64, _vp, _i, _f, _EP, _vp]),
+    "tlhip_gemv_grouped_prologue": (_i, [C.POINTER(GemvProblem), _i, C.POINTER(Prologue), _i, _i, _f, _vp]),
+    "tlhip_rmsnorm": (_i, [_vp, _i, _vp, _vp, _i, _i64, _i64, _f, _vp]),
+    "tlhip_gated_mul": (_i, [_i, _vp, _vp, _i, _vp, _i64, _vp]),
     "tlhip_gemm_prefill": (_i, [_QW, _vp, _i, _i64, _vp, _i, _f, _EP, _vp]),
     "tlhip_matmul_quantized": (_i, [_QW, _vp, _i, _i64, _vp, _i, _f, _EP, _vp]),
     "tlhip_matmul_quantized_config": (_i, [_QW, _vp, _i, _i64, _vp, _i, _f, _EP, _KC, _vp]),

@@ -265,6 +265,37 @@ class _Ops:
         approximate = (options or {}).get("approximate", "tanh")
         return self._unary("gelu_tanh" if approximate == "tanh" else "gelu_erf", a)
 
+    def mul(self, a: HipTensor, b: HipTensor) -> HipTensor:
+        """Elementwise product of two tensors of one shape and dtype (the MLP's
+        `mul(act(gate), up)`, packages/qwen3-browser/src/model.ts:357-361)."""
+        return self.gatedMul(a, b, "none")
+
+    def gatedMul(self, gate: HipTensor, up: HipTensor, activation: str = "silu") -> HipTensor:
+        """`mul(activation(gate), up)` in one pass."""
+        if (gate.dtype not in _DT_CODE or gate.dtype != up.dtype or list(gate.shape) != list(up.shape)
+                or not gate.isContiguous or not up.isContiguous):
+            raise NotImplementedError("hip backend mul: two contiguous f32/f16 tensors of one shape")
+        act = "gelu_tanh" if activation == "gelu" else activation
+        out = self._b._alloc(gate.shape, gate.dtype)
+        L.call("tlhip_gated_mul", L.UNARY[act], gate.ptr, up.ptr, _DT_CODE[gate.dtype], out.ptr, gate.size,
+               self._b.stream)
+        return out
+
+    def fusedRMSNormForward(self, x: HipTensor, weight: HipTensor, config: dict,
+                            outDtype: Optional[str] = None) -> HipTensor:
+        """BackendOps.fusedRMSNormForward (src/backend/types.ts:635-640): x [N,D],
+        weight f32 [D], config {numRows, featureDim, eps}."""
+        rows, d, eps = int(config["numRows"]), int(config["featureDim"]), float(config["eps"])
+        if x.dtype not in _DT_CODE or weight.dtype != "f32" or not x.isContiguous:
+            raise NotImplementedError("hip backend rmsnorm: contiguous f32/f16 x, f32 weight")
+        if x.size != rows * d or weight.size != d:
+            raise ValueError("fusedRMSNormForward: shape mismatch")
+        out_dtype = outDtype or x.dtype
+        out = self._b._alloc(x.shape, out_dtype)
+        L.call("tlhip_rmsnorm", x.ptr, _DT_CODE[x.dtype], weight.ptr, out.ptr, _DT_CODE[out_dtype], rows, d, eps,
+               self._b.stream)
+        return out
+
     def cast(self, a: HipTensor, dtype: str) -> HipTensor:
         if a.dtype == dtype:
             return a
@@ -502,7 +533,7 @@ class HipBackend:
 
     def linearGrouped(self, input: HipTensor, weights: Sequence[HipTensor],
                       biases: Optional[Sequence[Optional[HipTensor]]] = None,
-                      activation: Optional[str] = None) -> List[HipTensor]:
+                      activation: Optional[str] = None, _prologue: Optional[L.Prologue] = None) -> List[HipTensor]:
         """Up to four decode Linears on the same activation row (q/k/v, or gate/up)
         in one launch: the results of ``[linear(input, w, b, activation, fused=True)
         for w, b in zip(weights, biases)]``.  M = 1 and f16 activations."""
@@ -522,9 +553,86 @@ class HipBackend:
             probs[i].x = input.ptr
             probs[i].y = o.ptr
             probs[i].epilogue = C.pointer(ep) if ep is not None else None
-        L.call("tlhip_gemv_grouped", probs, len(weights), _DT_CODE[input.dtype], _DT_CODE[out_dtype], 1.0,
-               self.stream)
+        if _prologue is not None:
+            L.call("tlhip_gemv_grouped_prologue", probs, len(weights), C.byref(_prologue), _DT_CODE[input.dtype],
+                   _DT_CODE[out_dtype], 1.0, self.stream)
+        else:
+            L.call("tlhip_gemv_grouped", probs, len(weights), _DT_CODE[input.dtype], _DT_CODE[out_dtype], 1.0,
+                   self.stream)
         return outs
+
+    # the producers of a decode Linear's input, fused into its GEMV ------------
+    def _prologue(self, kind: int, operand: HipTensor, activation: str = "none", eps: float = 0.0) -> L.Prologue:
+        act = "gelu_tanh" if activation == "gelu" else activation
+        return L.Prologue(kind, L.UNARY[act], eps, 0, operand.ptr)
+
+    # Every workgroup of the GEMV forms f(x) for itself, so the fused form costs M * K
+    # extra work per workgroup: measured on MI355X it beats the separate launch (about
+    # 3 us inside a HIP graph) for one or two activation rows and loses from three on.
+    fusedPrologueMaxRows = 2
+
+    def _linearWithPrologue(self, input: HipTensor, pro: L.Prologue, weight: HipTensor,
+                            bias: Optional[HipTensor], activation: Optional[str]) -> Optional[HipTensor]:
+        """One fused launch, or None when no built kernel covers the request (or the
+        separate launches are faster)."""
+        qw = self._qweight(weight, transposed=False)
+        if input.dtype not in _DT_CODE or not input.isContiguous or input.shape[-1] != qw.k:
+            raise ValueError("linear: activations must be contiguous [..., K] of f32/f16")
+        m = input.size // qw.k if qw.k else 0
+        if m > self.fusedPrologueMaxRows:
+            return None
+        out_dtype = "f16" if (input.dtype == "f16" and weight.format.elementType == "f16") else "f32"
+        out = self._alloc(list(input.shape[:-1]) + [qw.n], out_dtype)
+        ep = self.makeEpilogue(bias, activation)
+        rc = L.load().tlhip_gemv_prologue(C.byref(qw), C.byref(pro), input.ptr, _DT_CODE[input.dtype], m, out.ptr,
+                                         _DT_CODE[out_dtype], 1.0, C.byref(ep), self.stream)
+        if rc == L.ERR_UNSUPPORTED:
+            out.destroy()
+            return None
+        L.check(rc)
+        return out
+
+    def linearAfterRMSNorm(self, input: HipTensor, normWeight: HipTensor, eps: float, weight: HipTensor,
+                           bias: Optional[HipTensor] = None, activation: Optional[str] = None) -> HipTensor:
+        """`linear(rmsnorm(input, normWeight, eps), weight, bias)` (+ activation): the
+        norm is applied while the GEMV stages its activations when a fused kernel
+        covers the shape (M <= 4), else as its own launch."""
+        if normWeight.dtype != "f32" or normWeight.size != input.shape[-1]:
+            raise ValueError("linearAfterRMSNorm: norm weight must be f32 [K]")
+        out = self._linearWithPrologue(input, self._prologue(L.PRO_RMSNORM, normWeight, eps=eps), weight, bias,
+                                       activation)
+        if out is not None:
+            return out
+        d = input.shape[-1]
+        normed = self.ops.fusedRMSNormForward(input, normWeight, {"numRows": input.size // d, "featureDim": d,
+                                                                  "eps": eps})
+        out = self.linear(normed, weight, bias, activation, fused=True)
+        normed.destroy()
+        return out
+
+    def linearAfterGatedMul(self, gate: HipTensor, up: HipTensor, gateActivation: str, weight: HipTensor,
+                            bias: Optional[HipTensor] = None, activation: Optional[str] = None) -> HipTensor:
+        """`linear(mul(gateActivation(gate), up), weight, bias)`: the MLP's down
+        projection with its input formed while the GEMV stages it (M <= 4)."""
+        if gate.dtype != up.dtype or list(gate.shape) != list(up.shape) or not up.isContiguous:
+            raise ValueError("linearAfterGatedMul: gate and up must share shape and dtype")
+        out = self._linearWithPrologue(gate, self._prologue(L.PRO_GATED_MUL, up, gateActivation), weight, bias,
+                                       activation)
+        if out is not None:
+            return out
+        x = self.ops.gatedMul(gate, up, gateActivation)
+        out = self.linear(x, weight, bias, activation, fused=True)
+        x.destroy()
+        return out
+
+    def linearGroupedAfterRMSNorm(self, input: HipTensor, normWeight: HipTensor, eps: float,
+                                  weights: Sequence[HipTensor],
+                                  biases: Optional[Sequence[Optional[HipTensor]]] = None,
+                                  activation: Optional[str] = None) -> List[HipTensor]:
+        """linearGrouped on `rmsnorm(input, normWeight, eps)`: q/k/v (or gate/up) of a
+        decode step and the norm in front of them in one launch."""
+        return self.linearGrouped(input, weights, biases, activation,
+                                  _prologue=self._prologue(L.PRO_RMSNORM, normWeight, eps=eps))
 
     # tuning + counters -----------------------------------------------------
     def pretuneMatmulShapes(self, shapes: Sequence[Sequence[int]]) -> None:

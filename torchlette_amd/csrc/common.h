@@ -41,6 +41,14 @@ struct DevEpilogue {
   const void* input[TLHIP_MAX_EPILOGUE_OPS];
 };
 
+// Prologue of the VALU decode GEMV (tlhip_prologue_t as the kernel takes it).
+struct DevPrologue {
+  int kind;
+  int unary;
+  float eps;
+  const void* operand;
+};
+
 // Validated problem description handed to the launchers.
 struct Problem {
   int format;
@@ -54,6 +62,7 @@ struct Problem {
   int y_dtype;
   float alpha;
   DevEpilogue epi;
+  DevPrologue pro;  // kind NONE unless the entry point sets it
 };
 
 // Validation shared by every compute entry point.  Fills `p` on success.

@@ -134,6 +134,42 @@ __device__ __forceinline__ void unpack_int8_word(uint32_t w, half2_t out[2]) {
   out[1] = __builtin_bit_cast(half2_t, a1) + sub;
 }
 
+// One 16-byte unit of activations as floats and back (f16: one rounding).
+template <typename XT>
+__device__ __forceinline__ void unit_to_floats(u32x4 v, float (&f)[16 / sizeof(XT)]) {
+  if constexpr (sizeof(XT) == 2) {
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const half2_t h = as_half2(w[i]);
+      f[2 * i] = (float)h[0];
+      f[2 * i + 1] = (float)h[1];
+    }
+  } else {
+    f[0] = as_float(v.x);
+    f[1] = as_float(v.y);
+    f[2] = as_float(v.z);
+    f[3] = as_float(v.w);
+  }
+}
+template <typename XT>
+__device__ __forceinline__ u32x4 floats_to_unit(const float (&f)[16 / sizeof(XT)]) {
+  u32x4 v;
+  if constexpr (sizeof(XT) == 2) {
+    uint32_t w[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const half2_t h = {(_Float16)f[2 * i], (_Float16)f[2 * i + 1]};
+      w[i] = __builtin_bit_cast(uint32_t, h);
+    }
+    v = (u32x4){w[0], w[1], w[2], w[3]};
+  } else {
+    v = (u32x4){__builtin_bit_cast(uint32_t, f[0]), __builtin_bit_cast(uint32_t, f[1]),
+                __builtin_bit_cast(uint32_t, f[2]), __builtin_bit_cast(uint32_t, f[3])};
+  }
+  return v;
+}
+
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits
 // for every outstanding global load of the wave (vmcnt(0)), which would drain
 // the weight loads that were deliberately issued ahead; here only the wave's

@@ -106,10 +106,10 @@ bool config_applicable(const Problem& p, const tlhip_kernel_config_t& c, const c
   return gemv_config_applicable(p, c, why);
 }
 
+tlhip_kernel_config_t default_valu_config(const Problem& p);
+
 // Heuristic default, used when nothing is tuned.
 tlhip_kernel_config_t default_config(const Problem& p) {
-  const int cw = p.format == TLHIP_FMT_INT4_GROUPED ? 32 : 16;
-  const int64_t nchunks = p.k / cw;
   if (p.m > 16 && p.x_dtype == TLHIP_F16) {
     const int cus = device_cu_count() > 0 ? device_cu_count() : 256;
     // int4: the kernel that keeps the weights packed up to the operand registers;
@@ -137,6 +137,14 @@ tlhip_kernel_config_t default_config(const Problem& p) {
         if (gemv_mfma_config_applicable(p, c, nullptr)) return c;
       }
   }
+  return default_valu_config(p);
+}
+
+// Heuristic default of the VALU kernel (the only one for M <= 4, and the one the
+// prologue entry points use).
+tlhip_kernel_config_t default_valu_config(const Problem& p) {
+  const int cw = p.format == TLHIP_FMT_INT4_GROUPED ? 32 : 16;
+  const int64_t nchunks = p.k / cw;
   // lanes per row: every lane busy for short rows; all chunks of a row in flight at once
   int lpr = 64;
   if (nchunks % 64 != 0) lpr = (nchunks % 32 == 0) ? 32 : 16;
@@ -311,6 +319,7 @@ int make_problem(const tlhip_qweight_t* w, const void* x, int x_dtype, int64_t m
   p->y_dtype = y_dtype;
   p->alpha = alpha;
   memset(&p->epi, 0, sizeof p->epi);
+  memset(&p->pro, 0, sizeof p->pro);
   if (epilogue) {
     if (epilogue->n_ops < 0 || epilogue->n_ops > TLHIP_MAX_EPILOGUE_OPS)
       return set_error(TLHIP_ERR_INVALID, "%s: epilogue has %d ops (max %d)", who, epilogue->n_ops,
@@ -390,6 +399,82 @@ int tlhip_gemv_grouped(const tlhip_gemv_problem_t* problems, int count, int x_dt
   }
   for (int i = 0; i < count; ++i) {
     int rc = matmul_with(ps[i], select_config(ps[i]), s);
+    if (rc) return rc;
+  }
+  return TLHIP_OK;
+}
+
+// Checks a prologue against the problem it feeds and copies it into `p`.
+static int attach_prologue(const tlhip_prologue_t* pro, Problem* p, const char* who) {
+  if (!pro || pro->kind == TLHIP_PRO_NONE) return TLHIP_OK;
+  if (pro->kind != TLHIP_PRO_RMSNORM && pro->kind != TLHIP_PRO_GATED_MUL)
+    return set_error(TLHIP_ERR_INVALID, "%s: unknown prologue kind %d", who, pro->kind);
+  if (!pro->operand && p->m > 0 && p->k > 0) return set_error(TLHIP_ERR_INVALID, "%s: prologue without operand", who);
+  if (((uintptr_t)pro->operand & 15) != 0)
+    return set_error(TLHIP_ERR_INVALID, "%s: prologue operand must be 16-byte aligned", who);
+  if (pro->kind == TLHIP_PRO_GATED_MUL && (pro->unary < TLHIP_UNARY_NONE || pro->unary > TLHIP_UNARY_TANH))
+    return set_error(TLHIP_ERR_INVALID, "%s: unknown unary op %d", who, pro->unary);
+  if (pro->kind == TLHIP_PRO_RMSNORM && !(pro->eps >= 0.f))
+    return set_error(TLHIP_ERR_INVALID, "%s: eps must be >= 0", who);
+  if (p->m > 4)
+    return set_error(TLHIP_ERR_UNSUPPORTED, "%s: the fused prologue is built for M <= 4, got %lld", who, (long long)p->m);
+  p->pro.kind = pro->kind;
+  p->pro.unary = pro->unary;
+  p->pro.eps = pro->eps;
+  p->pro.operand = pro->operand;
+  return TLHIP_OK;
+}
+
+// The VALU configuration a prologue launch runs with: the tuned or selected one if
+// it is of that kernel, else the heuristic.
+static tlhip_kernel_config_t valu_config(const Problem& p) {
+  tlhip_kernel_config_t c = select_config(p);
+  if (c.variant != VARIANT_GEMV) c = default_valu_config(p);
+  return c;
+}
+
+int tlhip_gemv_prologue(const tlhip_qweight_t* w, const tlhip_prologue_t* prologue, const void* x, int x_dtype,
+                        int64_t m, void* y, int y_dtype, float alpha, const tlhip_epilogue_t* epilogue,
+                        tlhip_stream_t stream) {
+  TLHIP_REQUIRE_INIT();
+  if (!prologue || prologue->kind == TLHIP_PRO_NONE)
+    return tlhip_gemv(w, x, x_dtype, m, y, y_dtype, alpha, epilogue, stream);
+  Problem p;
+  int rc = make_problem(w, x, x_dtype, m, y, y_dtype, alpha, epilogue, &p, "gemv_prologue");
+  if (rc) return rc;
+  rc = attach_prologue(prologue, &p, "gemv_prologue");
+  if (rc) return rc;
+  return launch_gemv(p, valu_config(p), resolve_stream(stream));
+}
+
+int tlhip_gemv_grouped_prologue(const tlhip_gemv_problem_t* problems, int count, const tlhip_prologue_t* prologue,
+                                int x_dtype, int y_dtype, float alpha, tlhip_stream_t stream) {
+  TLHIP_REQUIRE_INIT();
+  if (!prologue || prologue->kind == TLHIP_PRO_NONE)
+    return tlhip_gemv_grouped(problems, count, x_dtype, y_dtype, alpha, stream);
+  if (count < 0 || (count > 0 && !problems))
+    return set_error(TLHIP_ERR_INVALID, "gemv_grouped_prologue: bad problem list");
+  if (count > 4)
+    return set_error(TLHIP_ERR_INVALID, "gemv_grouped_prologue: a group holds at most 4 problems, got %d", count);
+  Problem ps[4];
+  for (int i = 0; i < count; ++i) {
+    int rc = make_problem(&problems[i].w, problems[i].x, x_dtype, 1, problems[i].y, y_dtype, alpha,
+                          problems[i].epilogue, &ps[i], "gemv_grouped_prologue");
+    if (rc) return rc;
+    rc = attach_prologue(prologue, &ps[i], "gemv_grouped_prologue");
+    if (rc) return rc;
+  }
+  if (count == 0) return TLHIP_OK;
+  hipStream_t s = resolve_stream(stream);
+  int big = 0;
+  for (int i = 1; i < count; ++i)
+    if (ps[i].n > ps[big].n) big = i;
+  tlhip_kernel_config_t c = valu_config(ps[big]);
+  c.p4 = 2;
+  if (c.p1 > 2) c.p1 = 2;
+  if (gemv_group_compatible(ps, count, c, nullptr)) return launch_gemv_grouped(ps, count, c, s);
+  for (int i = 0; i < count; ++i) {
+    int rc = launch_gemv(ps[i], valu_config(ps[i]), s);
     if (rc) return rc;
   }
   return TLHIP_OK;

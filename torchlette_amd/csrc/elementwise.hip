@@ -1,8 +1,10 @@
-// The three small ops that sit either side of the packed matmul when the
-// frontend calls them unfused (api.linear issues matmul, then add —
+// The small ops that sit either side of the packed matmul when the frontend
+// calls them unfused (api.linear issues matmul, then add —
 // src/frontend/torchlette.ts:887-894 — and the model issues the activation):
-// bias add over the last dimension, a unary activation, and an f32<->f16 cast.
-// All are one pass over the data, 16 bytes per lane where alignment allows.
+// bias add over the last dimension, a unary activation, an f32<->f16 cast, and
+// the two producers of a decode Linear's input: RMSNorm
+// (src/backend/webgpu/rmsnorm-kernel.ts:31-66) and the MLP's act(gate) * up
+// (packages/qwen3-browser/src/model.ts:357-361).  All are one pass over the data.
 #include <algorithm>
 
 #include "device_utils.h"
@@ -36,6 +38,35 @@ __global__ __launch_bounds__(256) void cast_kernel(const S* __restrict__ in, D* 
   int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
   for (; i < count; i += stride) out[i] = (D)in[i];
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void gated_mul_kernel(int op, const T* __restrict__ gate, const T* __restrict__ up,
+                                                       T* __restrict__ out, int64_t count) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (; i < count; i += stride) out[i] = (T)(apply_unary(op, (float)gate[i]) * (float)up[i]);
+}
+
+// One workgroup per row.  The row is read twice (the second time from cache):
+// once for the sum of squares, once to scale.  f32 arithmetic throughout.
+template <typename XT, typename YT>
+__global__ __launch_bounds__(256) void rmsnorm_kernel(const XT* __restrict__ x, const float* __restrict__ weight,
+                                                     YT* __restrict__ y, int64_t d, float eps) {
+  __shared__ float red[4];
+  const XT* xr = x + (int64_t)blockIdx.x * d;
+  YT* yr = y + (int64_t)blockIdx.x * d;
+  float ss = 0.f;
+  for (int64_t i = threadIdx.x; i < d; i += 256) {
+    const float v = (float)xr[i];
+    ss = fmaf(v, v, ss);
+  }
+  ss = group_sum(ss, 64);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;
+  __syncthreads();
+  const float total = (red[0] + red[1]) + (red[2] + red[3]);
+  const float inv = 1.f / sqrtf(total / (float)d + eps);
+  for (int64_t i = threadIdx.x; i < d; i += 256) yr[i] = (YT)(((float)xr[i] * inv) * weight[i]);
 }
 
 int grid_for(int64_t count) {
@@ -85,6 +116,53 @@ int tlhip_unary(int op, const void* in, int dtype, void* out, int64_t count, tlh
   else
     hipLaunchKernelGGL(unary_kernel<float>, dim3(grid_for(count)), dim3(256), 0, s, op, (const float*)in,
                        (float*)out, count);
+  TLHIP_CHECK_HIP(hipGetLastError());
+  return TLHIP_OK;
+}
+
+int tlhip_gated_mul(int unary, const void* gate, const void* up, int dtype, void* out, int64_t count,
+                    tlhip_stream_t stream) {
+  TLHIP_REQUIRE_INIT();
+  if (count < 0) return set_error(TLHIP_ERR_INVALID, "gated_mul: negative count");
+  if (count == 0) return TLHIP_OK;
+  if (!gate || !up || !out) return set_error(TLHIP_ERR_INVALID, "gated_mul: null pointer");
+  if (unary < TLHIP_UNARY_NONE || unary > TLHIP_UNARY_TANH)
+    return set_error(TLHIP_ERR_INVALID, "gated_mul: unknown op %d", unary);
+  if (dtype != TLHIP_F32 && dtype != TLHIP_F16) return set_error(TLHIP_ERR_INVALID, "gated_mul: bad dtype");
+  hipStream_t s = resolve_stream(stream);
+  if (dtype == TLHIP_F16)
+    hipLaunchKernelGGL(gated_mul_kernel<_Float16>, dim3(grid_for(count)), dim3(256), 0, s, unary,
+                       (const _Float16*)gate, (const _Float16*)up, (_Float16*)out, count);
+  else
+    hipLaunchKernelGGL(gated_mul_kernel<float>, dim3(grid_for(count)), dim3(256), 0, s, unary, (const float*)gate,
+                       (const float*)up, (float*)out, count);
+  TLHIP_CHECK_HIP(hipGetLastError());
+  return TLHIP_OK;
+}
+
+int tlhip_rmsnorm(const void* x, int x_dtype, const float* weight, void* y, int y_dtype, int64_t m, int64_t d,
+                  float eps, tlhip_stream_t stream) {
+  TLHIP_REQUIRE_INIT();
+  if (m < 0 || d < 0) return set_error(TLHIP_ERR_INVALID, "rmsnorm: negative shape");
+  if (m == 0 || d == 0) return TLHIP_OK;
+  if (!x || !weight || !y) return set_error(TLHIP_ERR_INVALID, "rmsnorm: null pointer");
+  if ((x_dtype != TLHIP_F32 && x_dtype != TLHIP_F16) || (y_dtype != TLHIP_F32 && y_dtype != TLHIP_F16))
+    return set_error(TLHIP_ERR_INVALID, "rmsnorm: bad dtype");
+  if (!(eps >= 0.f)) return set_error(TLHIP_ERR_INVALID, "rmsnorm: eps must be >= 0");
+  if (m > 0x7fffffff) return set_error(TLHIP_ERR_INVALID, "rmsnorm: too many rows");
+  hipStream_t s = resolve_stream(stream);
+  const dim3 grid((unsigned)m), block(256);
+  if (x_dtype == TLHIP_F16 && y_dtype == TLHIP_F16)
+    hipLaunchKernelGGL((rmsnorm_kernel<_Float16, _Float16>), grid, block, 0, s, (const _Float16*)x, weight,
+                       (_Float16*)y, d, eps);
+  else if (x_dtype == TLHIP_F16)
+    hipLaunchKernelGGL((rmsnorm_kernel<_Float16, float>), grid, block, 0, s, (const _Float16*)x, weight, (float*)y, d,
+                       eps);
+  else if (y_dtype == TLHIP_F16)
+    hipLaunchKernelGGL((rmsnorm_kernel<float, _Float16>), grid, block, 0, s, (const float*)x, weight, (_Float16*)y, d,
+                       eps);
+  else
+    hipLaunchKernelGGL((rmsnorm_kernel<float, float>), grid, block, 0, s, (const float*)x, weight, (float*)y, d, eps);
   TLHIP_CHECK_HIP(hipGetLastError());
   return TLHIP_OK;
 }

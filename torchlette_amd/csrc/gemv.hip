@@ -72,6 +72,8 @@ static void fill_args(const Problem& p, const tlhip_kernel_config_t& c, int64_t 
   a.scale_mul = p.format == TLHIP_FMT_INT8_GROUPED ? (1.0f / 127.0f) : 1.0f;
   a.y_dtype = p.y_dtype;
   a.epi = p.epi;
+  a.pro = p.pro;
+  if (a.pro.kind == TLHIP_PRO_GATED_MUL) a.pro.operand = (const char*)p.pro.operand + m0 * p.k * xbytes;
   // LDS: staged x (mt rows) + split-K partials
   const int chunk_x_bytes = cw * xbytes;
   const size_t partial_bytes = a.kw > 1 ? (size_t)a.kw * a.rows_per_wg * mt * sizeof(float) : 0;

@@ -28,6 +28,7 @@ struct GemvArgs {
   float scale_mul;       // 1/127 for INT8_GROUPED, else 1
   int y_dtype;
   DevEpilogue epi;
+  DevPrologue pro;
 };
 
 // Several problems of one shape class in one launch: workgroups

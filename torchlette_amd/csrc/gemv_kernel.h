@@ -322,6 +322,155 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& a, const int bid, cons
     const int c = u / NQ, qd = u - c * NQ;
     return lds + (m * NQ + qd) * a.nchunks + c;
   };
+  if (a.pro.kind != TLHIP_PRO_NONE) {
+    // What is staged is f(x): see stage_with_prologue.
+    constexpr int E = 16 / (int)sizeof(XT);  // elements per 16-byte unit
+    constexpr bool PERMUTE = FMT == TLHIP_FMT_INT4_GROUPED && sizeof(XT) == 2;
+    const int T = (int)blockDim.x;
+    auto unit_off = [&](int idx, int& m, int& u) {
+      split(idx, m, u);
+      const int mm = m < a.m ? m : a.m - 1;
+      return (size_t)mm * x_units_per_row + u;
+    };
+    u32x4 xr[XS], orr[XS];
+    if (a.pro.kind == TLHIP_PRO_GATED_MUL) {
+      // f(x) = unary(gate) * up, elementwise: groups of XS units per thread; the
+      // first weight batch is issued behind the first group's loads.
+      const u32x4* ug = (const u32x4*)a.pro.operand;
+      auto issue = [&](int base) {
+#pragma unroll
+        for (int i = 0; i < XS; ++i) {
+          int m, u;
+          const size_t off = unit_off(min(base + tid + i * T, units_total - 1), m, u);
+          xr[i] = xg[off];
+          orr[i] = ug[off];
+        }
+      };
+      auto consume = [&](int base) {
+#pragma unroll
+        for (int i = 0; i < XS; ++i) {
+          const int idx = base + tid + i * T;
+          if (idx < units_total) {
+            float g[E], up[E];
+            unit_to_floats<XT>(xr[i], g);
+            unit_to_floats<XT>(orr[i], up);
+#pragma unroll
+            for (int e = 0; e < E; ++e) g[e] = apply_unary(a.pro.unary, g[e]) * up[e];
+            u32x4 v = floats_to_unit<XT>(g);
+            if (PERMUTE) v = permute_x_for_int4(v);
+            *x_dst(idx) = v;
+          }
+        }
+      };
+      issue(0);
+      load_batch(cur, rb, cfirst);
+      consume(0);
+      for (int base = XS * T; base < units_total; base += XS * T) {
+        issue(base);
+        consume(base);
+      }
+    } else {
+      // RMSNORM: pass 1 parks the raw rows in LDS (at their final places) and sums
+      // the squares; after the workgroup-wide sum every thread rescales the units
+      // it parked itself, so no barrier is needed between the passes beyond the
+      // one of the sum.
+      __shared__ float red[4][16];
+      float ss[MT];
+#pragma unroll
+      for (int m = 0; m < MT; ++m) ss[m] = 0.f;
+      auto issue = [&](int base) {
+#pragma unroll
+        for (int i = 0; i < XS; ++i) {
+          int m, u;
+          xr[i] = xg[unit_off(min(base + tid + i * T, units_total - 1), m, u)];
+        }
+      };
+      auto park = [&](int base) {
+#pragma unroll
+        for (int i = 0; i < XS; ++i) {
+          const int idx = base + tid + i * T;
+          if (idx < units_total) {
+            int m, u;
+            split(idx, m, u);
+            float f[E];
+            unit_to_floats<XT>(xr[i], f);
+            float sq = 0.f;
+#pragma unroll
+            for (int e = 0; e < E; ++e) sq = fmaf(f[e], f[e], sq);
+#pragma unroll
+            for (int mm = 0; mm < MT; ++mm) ss[mm] += (mm == m) ? sq : 0.f;
+            *x_dst(idx) = xr[i];
+          }
+        }
+      };
+      // norm weights of a group's units (E floats each)
+      const float* nw = (const float*)a.pro.operand;
+      u32x4 wv[XS][E / 4];
+      auto issue_w = [&](int base) {
+#pragma unroll
+        for (int i = 0; i < XS; ++i) {
+          int m, u;
+          split(min(base + tid + i * T, units_total - 1), m, u);
+#pragma unroll
+          for (int h = 0; h < E / 4; ++h) wv[i][h] = *(const u32x4*)(nw + (size_t)u * E + 4 * h);
+        }
+      };
+      float inv[MT];
+      auto rescale = [&](int base) {
+#pragma unroll
+        for (int i = 0; i < XS; ++i) {
+          const int idx = base + tid + i * T;
+          if (idx < units_total) {
+            int m, u;
+            split(idx, m, u);
+            float f[E];
+            unit_to_floats<XT>(*x_dst(idx), f);
+            float s = inv[0];
+#pragma unroll
+            for (int mm = 1; mm < MT; ++mm) s = (mm == m) ? inv[mm] : s;
+#pragma unroll
+            for (int h = 0; h < E / 4; ++h) {
+              f[4 * h + 0] = (f[4 * h + 0] * s) * as_float(wv[i][h].x);
+              f[4 * h + 1] = (f[4 * h + 1] * s) * as_float(wv[i][h].y);
+              f[4 * h + 2] = (f[4 * h + 2] * s) * as_float(wv[i][h].z);
+              f[4 * h + 3] = (f[4 * h + 3] * s) * as_float(wv[i][h].w);
+            }
+            u32x4 v = floats_to_unit<XT>(f);
+            if (PERMUTE) v = permute_x_for_int4(v);
+            *x_dst(idx) = v;
+          }
+        }
+      };
+      // the first group's rows and norm weights, then the first weight batch: the
+      // sum below waits for the rows only
+      issue(0);
+      issue_w(0);
+      load_batch(cur, rb, cfirst);
+      park(0);
+      for (int base = XS * T; base < units_total; base += XS * T) {
+        issue(base);
+        park(base);
+      }
+#pragma unroll
+      for (int m = 0; m < MT; ++m) {
+        ss[m] = group_sum(ss[m], 64);
+        if (lane == 0) red[m][wave] = ss[m];
+      }
+      lds_barrier();
+      const int nwaves = T >> 6;
+#pragma unroll
+      for (int m = 0; m < MT; ++m) {
+        float t = 0.f;
+        for (int w = 0; w < nwaves; ++w) t += red[m][w];
+        inv[m] = 1.f / sqrtf(t / (float)a.k + a.pro.eps);
+      }
+      rescale(0);
+      for (int base = XS * T; base < units_total; base += XS * T) {
+        issue_w(base);
+        rescale(base);
+      }
+    }
+  } else
   if (units_total <= XS * (int)blockDim.x) {
     u32x4 xr[XS];
 #pragma unroll
