@@ -1,0 +1,143 @@
+"use strict";
+/* Runs the JavaScript `hip` backend (torchlette_amd/addon/hip_backend.js) over the
+ * inputs a pytest run wrote into a directory, and writes what it computed back there.
+ * Usage: node addon_scenario.js <dir>.  <dir>/manifest.json lists the cases; every
+ * array is a raw little-endian file.  One process runs every case. */
+const fs = require("fs");
+const path = require("path");
+const H = require(path.join(__dirname, "..", "..", "torchlette_amd", "addon", "hip_backend.js"));
+
+const dir = process.argv[2];
+const manifest = JSON.parse(fs.readFileSync(path.join(dir, "manifest.json"), "utf8"));
+const TYPES = { f32: Float32Array, u32: Uint32Array, u16: Uint16Array, i32: Int32Array };
+
+function load(name, type) {
+  const buf = fs.readFileSync(path.join(dir, name));
+  const ab = buf.buffer.slice(buf.byteOffset, buf.byteOffset + buf.byteLength);
+  return new TYPES[type](ab);
+}
+function save(name, typed) {
+  fs.writeFileSync(path.join(dir, name), Buffer.from(typed.buffer, typed.byteOffset, typed.byteLength));
+}
+/* activations arrive as f32 files; an f16 tensor is made by the backend's own codec */
+function tensor(be, name, shape, dtype) {
+  return be.ops.tensorFromArray(load(name, "f32"), shape, dtype);
+}
+function weightOf(be, c) {
+  const fmt = H.resolveWeightFormat(c.format, c.element);
+  const scales = load(c.scales, c.format === "int8-row" ? "f32" : "u16");
+  return be.createQuantizedWeight(load(c.packed, "u32"), scales, c.n, c.k, fmt);
+}
+
+const results = { cases: {}, errors: {} };
+const be = H.getBackend(0);
+results.device = be.deviceInfo();
+
+for (const c of manifest.cases) {
+  const r = {};
+  if (c.kind === "linear") {
+    const w = weightOf(be, c);
+    const x = tensor(be, c.x, [c.m, c.k], c.xdtype);
+    const bias = c.bias ? tensor(be, c.bias, [c.n], "f32") : null;
+    const g0 = H.getQuantGemvDispatchCount(), m0 = H.getQuantGemmDispatchCount();
+    const y = be.linear(x, w, bias, c.act, c.fused);
+    r.gemv = H.getQuantGemvDispatchCount() - g0;
+    r.gemm = H.getQuantGemmDispatchCount() - m0;
+    r.shape = y.shape;
+    r.dtype = y.dtype;
+    save(c.out, be.ops.read(y));
+  } else if (c.kind === "quantize") {
+    const q = H.quantizeLinearWeight(load(c.weight, "f32"), c.n, c.k, c.g);
+    save(c.out_packed, q.packed);
+    save(c.out_scales, q.scales);
+    const w = be.createQuantizedWeight(q.packed, q.scales, c.n, c.k, H.resolveWeightFormat(c.g === 64 ? "int8-64" : "int8-128", "f32"));
+    const d0 = H.getDequantI8DispatchCount();
+    save(c.out_dequant, be.ops.read(be.dequantizeToF32(w)));
+    r.dequant = H.getDequantI8DispatchCount() - d0;
+    // and on the device, from the f32 weight uploaded as it is
+    const wdev = be.ops.tensorFromArray(load(c.weight, "f32"), [c.n, c.k], "f32");
+    const qd = be.quantizeLinearWeightOnDevice(wdev, c.g, "f32");
+    save(c.out_dequant_device, be.ops.read(be.dequantizeToF32(qd)));
+  } else if (c.kind === "rmsnorm_linear" || c.kind === "gated_linear") {
+    const w = weightOf(be, c);
+    const x = tensor(be, c.x, [c.m, c.k], c.xdtype);
+    let y, apart;
+    if (c.kind === "rmsnorm_linear") {
+      const nw = tensor(be, c.norm_weight, [c.k], "f32");
+      const normed = be.ops.fusedRMSNormForward(x, nw, { numRows: c.m, featureDim: c.k, eps: c.eps });
+      save(c.out_norm, be.ops.read(normed));
+      y = be.linearAfterRMSNorm(x, nw, c.eps, w);
+      apart = be.linear(normed, w, null, "none", true);
+    } else {
+      const up = tensor(be, c.up, [c.m, c.k], c.xdtype);
+      const prod = be.ops.mul(be.ops.silu(x), up);   // the model's two ops
+      save(c.out_prod, be.ops.read(prod));
+      y = be.linearAfterGatedMul(x, up, "silu", w);
+      apart = be.linear(prod, w, null, "none", true);
+    }
+    save(c.out, be.ops.read(y));
+    save(c.out_apart, be.ops.read(apart));
+  } else if (c.kind === "grouped") {
+    const x = tensor(be, c.x, [1, c.k], "f16");
+    const ws = c.weights.map((wc) => weightOf(be, Object.assign({ k: c.k, format: c.format, element: "f16" }, wc)));
+    const outs = be.linearGrouped(x, ws);
+    outs.forEach((o, i) => save(c.weights[i].out, be.ops.read(o)));
+  } else if (c.kind === "topk") {
+    const logits = tensor(be, c.logits, [c.length], "f32");
+    be.ops.readTopK(logits, c.k).then((t) => {
+      save(c.out_values, t.values);
+      save(c.out_indices, t.indices);
+    });
+    const packed = be.ops.deviceTopK(logits, c.k);
+    save(c.out_packed, be.ops.read(packed));
+  }
+  results.cases[c.name] = r;
+}
+
+/* the error channel: every failure is a thrown Error carrying the library's message */
+function expectThrow(name, fn) {
+  try {
+    fn();
+    results.errors[name] = null;
+  } catch (e) {
+    results.errors[name] = { message: e.message, code: e.code || null };
+  }
+}
+{
+  const c = manifest.cases.find((v) => v.kind === "linear");
+  const w = weightOf(be, c);
+  const bad = be.ops.zeros([1, c.k + 32], "f32");
+  expectThrow("dimension_mismatch", () => be.linear(bad, w));
+  expectThrow("dense_matmul", () => be.ops.matmul(bad, be.ops.zeros([c.k + 32, 8], "f32")));
+  expectThrow("quantize_bad_k", () => H.quantizeLinearWeight(new Float32Array(6), 2, 3, 64));
+  expectThrow("bad_config", () => {
+    const x = be.ops.zeros([1, c.k], c.xdtype);
+    be.linear(x, w, null, "none", true, new Int32Array([2, 256, 256, 64, 2, 2, 0, 0]));  // a prefill tile for M = 1
+  });
+  expectThrow("unknown_format", () => H.resolveWeightFormat("int3-7"));
+  // tuning cache: seed, export, clear, import
+  const x = be.ops.zeros([1, c.k], c.xdtype);
+  const cfg = be.candidates(w, c.xdtype, 1, c.element === "f16" && c.xdtype === "f16" ? "f16" : "f32")[0];
+  const ydt = c.element === "f16" && c.xdtype === "f16" ? "f16" : "f32";
+  be.seedPerShapeMatmulChoice(w, c.xdtype, 1, ydt, cfg);
+  const text = H.exportTuningCache();
+  H.clearTuningCache();
+  const cleared = H.exportTuningCache();
+  H.importTuningCache(text);
+  results.tuning = {
+    seeded: Array.from(cfg), exported_entries: Object.keys(JSON.parse(text).entries).length,
+    text_has_key: text.length > cleared.length,
+    selected_after_import: Array.from(be.selectedConfig(w, c.xdtype, 1, ydt)),
+  };
+  H.setAutotuneEnabled(true);
+  results.autotune_enabled = H.isAutotuneEnabled();
+  const a0 = H.getAutotuneRunCount();
+  H.clearTuningCache();
+  be.linear(x, w);
+  results.autotune_runs = H.getAutotuneRunCount() - a0;
+  H.setAutotuneEnabled(false);
+}
+be.synchronize();
+setImmediate(() => {
+  fs.writeFileSync(path.join(dir, "results.json"), JSON.stringify(results));
+});
