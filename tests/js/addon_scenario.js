@@ -29,6 +29,8 @@ function weightOf(be, c) {
   return be.createQuantizedWeight(load(c.packed, "u32"), scales, c.n, c.k, fmt);
 }
 
+const D = require(path.join(__dirname, "..", "..", "torchlette_amd", "addon", "hip_matmul_dispatch.js"));
+
 const results = { cases: {}, errors: {} };
 const be = H.getBackend(0);
 results.device = be.deviceInfo();
@@ -82,6 +84,32 @@ for (const c of manifest.cases) {
     const ws = c.weights.map((wc) => weightOf(be, Object.assign({ k: c.k, format: c.format, element: "f16" }, wc)));
     const outs = be.linearGrouped(x, ws);
     outs.forEach((o, i) => save(c.weights[i].out, be.ops.read(o)));
+  } else if (c.kind === "side_door") {
+    // the fused path's call for matmul -> bias -> unary (-> cast): executor.ts:2959-3049
+    const w = weightOf(be, c);
+    const x = tensor(be, c.x, [c.m, c.k], c.xdtype);
+    const bias = tensor(be, c.bias, [c.n], "f32");
+    const epilogue = { ops: [{ kind: "bias", inputIndex: 0 }, { kind: "unary", op: c.act }, { kind: "cast", toDtype: c.out_dtype }],
+                       additionalInputCount: 1, outputDtype: c.out_dtype };
+    const g0 = H.getQuantGemvDispatchCount() + H.getQuantGemmDispatchCount();
+    const y1 = D.dispatchMatmul(x, be.ops.transpose(w), false, false, undefined, { epilogue, epilogueInputs: [bias] });
+    r.launches = H.getQuantGemvDispatchCount() + H.getQuantGemmDispatchCount() - g0;
+    const y2 = D.dispatchMatmul(x, w, false, true, undefined, { epilogue, epilogueInputs: [bias] });
+    const donated = be.ops.zeros([c.m, c.n], "f32");   // larger than needed for f16: reused
+    const y3 = D.dispatchMatmul(x, be.ops.transpose(w), false, false, donated, { epilogue, epilogueInputs: [bias] });
+    r.donated_reused = y3.ptr === donated.ptr;
+    const y4 = D.dispatchMatmulDirect(x, w, { m: c.m, n: c.n, k: c.k, outShape: [c.m, c.n], dtypeA: c.xdtype,
+      outputDtype: c.out_dtype, epilogueConfig: epilogue, epilogueBuffers: [bias], packing: w.format.packing, scales: w.scales });
+    r.dtype = y1.dtype;
+    r.plan = D.planBareMatmul(x, be.ops.transpose(w));
+    [y1, y2, y3, y4].forEach((y, i) => save(c.out + i, be.ops.read(y)));
+    try {
+      D.dispatchMatmul(x, be.ops.transpose(w), false, false, undefined,
+        { epilogue: { ops: [{ kind: "binary", op: "mul", inputIndex: 0 }], additionalInputCount: 1, outputDtype: "f32" }, epilogueInputs: [bias] });
+      r.binary_error = null;
+    } catch (e) {
+      r.binary_error = e.message;
+    }
   } else if (c.kind === "topk") {
     const logits = tensor(be, c.logits, [c.length], "f32");
     be.ops.readTopK(logits, c.k).then((t) => {

@@ -105,6 +105,18 @@ def run(tmp_path_factory):
     cases.append({"kind": "grouped", "name": "grouped", "format": "int4-32", "k": k,
                   "x": put("g.x", x.astype(np.float32)), "weights": gw})
 
+    for name, m, xdt, out_dtype in (("door_m1", 1, "f32", "f32"), ("door_m64", 64, "f16", "f16")):
+        rng = seeded("addon", name)
+        n, k, g = 768, 1024, 32
+        packed, scales, deq = make_weight("int4-grouped", n, k, g, rng)
+        x = make_x(m, k, xdt, rng)
+        bias = rng.standard_normal(n).astype(np.float32)
+        cases.append({"kind": "side_door", "name": name, "format": "int4-32", "element": "f16", "n": n, "k": k, "m": m,
+                      "xdtype": xdt, "act": "silu", "out_dtype": out_dtype, "packed": put(name + ".packed", packed),
+                      "scales": put(name + ".scales", scales), "x": put(name + ".x", x.astype(np.float32)),
+                      "bias": put(name + ".bias", bias), "out": name + ".y"})
+        want[name] = (O.linear(x.astype(np.float32), deq, bias, "silu"), out_dtype, (m, n))
+
     rng = seeded("addon", "topk")
     logits = rng.standard_normal(50000).astype(np.float32)
     logits[[7, 49999]] = logits.max() + 1.0  # a tie at the top: the smaller index first
@@ -160,6 +172,21 @@ def test_producers_and_their_fused_form(run, kind, first):
     assert rel_l2(run["get"](kind + first).reshape(fx.shape), fx) <= 1e-3   # f16 tensors
     assert rel_l2(run["get"](kind + ".y").reshape(shape), want) <= 1e-3
     assert rel_l2(run["get"](kind + ".yapart").reshape(shape), want) <= 1e-3
+
+
+@pytest.mark.parametrize("name", ["door_m1", "door_m64"])
+def test_fused_side_door(run, name):
+    """matmul -> bias -> silu -> cast handed over as one EpilogueConfig: one launch, and the
+    four ways in (transposed view, transB, donated buffer, cached geometry) agree."""
+    want, dtype, shape = run["want"][name]
+    r = run["results"]["cases"][name]
+    assert r["launches"] == 1 and r["dtype"] == dtype and r["donated_reused"] is True
+    assert r["plan"] == "quantized-operand"           # planBareMatmul: webgpu/dispatch.ts:826
+    assert "binary" in r["binary_error"]
+    ys = [run["get"](f"{name}.y{i}").reshape(shape) for i in range(4)]
+    for y in ys:
+        assert rel_l2(y, want) <= (1e-5 if dtype == "f32" else 1e-3)
+        assert np.array_equal(y, ys[0])
 
 
 def test_grouped_launch(run):

@@ -362,6 +362,46 @@ static napi_value MatmulQuantized(napi_env env, napi_callback_info info) {
   }
   return undefined(env);
 }
+/* matmulQuantizedOps(format, groupSize, n, k, packed, scales, xPtr, xDtype, m, yPtr, yDtype,
+ *                    [[kind, unary, inputPtr | null, inputDtype], ...])
+ * An epilogue chain of up to TLHIP_MAX_EPILOGUE_OPS steps in the caller's order: the
+ * EpilogueConfig.ops of the fused path (src/backend/webgpu/matmul/types.ts:13-24). */
+static napi_value MatmulQuantizedOps(napi_env env, napi_callback_info info) {
+  ARGS(12);
+  WEIGHT(0, w);
+  PTR(6, x);
+  I32(7, xd);
+  I64(8, m);
+  PTR(9, y);
+  I32(10, yd);
+  bool is_array = false;
+  uint32_t count = 0;
+  if (napi_is_array(env, a[11], &is_array) != napi_ok || !is_array) return throw_type(env, "tlhip: ops must be an array");
+  napi_get_array_length(env, a[11], &count);
+  if (count > TLHIP_MAX_EPILOGUE_OPS) return throw_type(env, "tlhip: too many epilogue ops");
+  tlhip_epilogue_t ep;
+  memset(&ep, 0, sizeof ep);
+  for (uint32_t i = 0; i < count; ++i) {
+    napi_value row, f[4];
+    uint32_t len = 0;
+    napi_get_element(env, a[11], i, &row);
+    if (napi_is_array(env, row, &is_array) != napi_ok || !is_array) return throw_type(env, "tlhip: an op is [kind, unary, input, inputDtype]");
+    napi_get_array_length(env, row, &len);
+    if (len != 4) return throw_type(env, "tlhip: an op is [kind, unary, input, inputDtype]");
+    for (uint32_t j = 0; j < 4; ++j) napi_get_element(env, row, j, &f[j]);
+    int32_t kind, unary, idt;
+    void* input;
+    if (!get_i32(env, f[0], &kind) || !get_i32(env, f[1], &unary) || !get_ptr(env, f[2], &input) || !get_i32(env, f[3], &idt))
+      return throw_type(env, "tlhip: an op is [kind, unary, input, inputDtype]");
+    ep.ops[i].kind = kind;
+    ep.ops[i].unary = unary;
+    ep.ops[i].input = input;
+    ep.ops[i].input_dtype = idt;
+  }
+  ep.n_ops = (int32_t)count;
+  CHECK(tlhip_matmul_quantized(&w, x, xd, m, y, yd, 1.0f, count ? &ep : NULL, NULL));
+  return undefined(env);
+}
 /* gemvPrologue(format, groupSize, n, k, packed, scales, xPtr, xDtype, m, yPtr, yDtype,
  *              biasPtr | null, biasDtype, unary, kind, operandPtr, proUnary, eps)
  * -> true, or false when no fused kernel covers the request (run the steps apart). */
@@ -676,7 +716,7 @@ NAPI_MODULE_INIT() {
       FN("graphEndCapture", GraphEndCapture), FN("graphLaunch", GraphLaunch), FN("graphDestroy", GraphDestroy),
       FN("f32ToF16Bits", F32ToF16Bits), FN("f16BitsToF32", F16BitsToF32),
       FN("quantizeInt8Grouped", QuantizeInt8Grouped), FN("quantizeInt8GroupedDevice", QuantizeInt8GroupedDevice),
-      FN("dequant", Dequant), FN("matmulQuantized", MatmulQuantized), FN("gemvPrologue", GemvPrologue),
+      FN("dequant", Dequant), FN("matmulQuantized", MatmulQuantized), FN("matmulQuantizedOps", MatmulQuantizedOps), FN("gemvPrologue", GemvPrologue),
       FN("gemvGrouped", GemvGrouped), FN("biasAdd", BiasAdd), FN("unary", Unary), FN("cast", Cast),
       FN("rmsnorm", RmsNorm), FN("gatedMul", GatedMul), FN("topk", TopK), FN("selectedConfig", SelectedConfig),
       FN("candidates", Candidates), FN("autotune", Autotune), FN("tuneCacheSeed", TuneCacheSeed),
