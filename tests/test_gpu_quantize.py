@@ -96,3 +96,35 @@ def test_device_quantizer_errors(be):
     p = C.c_void_p(16)
     with pytest.raises(L.TlhipError, match="multiple of 4"):
         L.call("tlhip_quantize_int8_grouped_device", p, 2, 12, 6, p, p, None)
+
+
+@pytest.mark.parametrize("on_device", [False, True])
+def test_loader_branch_quantizes_once_and_then_hits_the_cache(be, tmp_path, on_device):
+    """browser-loader.ts:654-699: miss -> fetch f32, quantize, store; hit -> the tensor's
+    bytes are never fetched.  Either way the weight equals the oracle's bit for bit."""
+    n, k, g = 48, 512, 64
+    rng = np.random.default_rng(7)
+    w = (rng.standard_normal((n, k)) * 0.2).astype(np.float32)
+    cache = T.PackedWeightCache(str(tmp_path / "packed"))
+    fetched = []
+
+    def fetch():
+        fetched.append(1)
+        return w
+
+    want_packed, want_scales = O.quantize_int8_grouped(w.ravel(), n, k, g)
+    want = O.dequant_int8_grouped(want_packed, want_scales, n, k, g)
+    url, name = "https://host/model.safetensors", "model.layers.0.self_attn.q_proj.weight"
+    for expect_fetches in (1, 1):
+        q = T.loadQuantizedWeight(be, cache, url, name, n, k, "int8-64", fetch, "f32", onDevice=on_device)
+        assert len(fetched) == expect_fetches
+        got = be.dequantizeToF32(q).numpy()
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    rec = cache.getCachedPacked(T.packedKey(url, name, "int8-grouped", g))
+    assert np.array_equal(rec["packed"], want_packed.ravel()) and np.array_equal(rec["scales"], want_scales.ravel())
+    # another group size is another key: quantized again
+    T.loadQuantizedWeight(be, cache, url, name, n, k, "int8-128", fetch, "f32", onDevice=on_device)
+    assert len(fetched) == 2
+    # no cache at all still works
+    T.loadQuantizedWeight(be, None, url, name, n, k, "int8-64", fetch, "f32", onDevice=on_device)
+    assert len(fetched) == 3

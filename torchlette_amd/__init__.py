@@ -11,3 +11,4 @@ from .backend import (  # noqa: F401
     getQuantGemmDispatchCount, getQuantGemvDispatchCount, importTuningCache, isAutotuneEnabled,
     quantizeLinearWeight, resetMatmulState, resolveWeightFormat, setAutotuneEnabled,
 )
+from .packed_cache import PackedWeightCache, loadQuantizedWeight, packedKey  # noqa: F401

@@ -345,6 +345,17 @@ class HipBackend:
         L.call("tlhip_stream_synchronize", self.stream)
         return host.reshape(t.shape)
 
+    def _download_raw(self, t: HipTensor, count: int, dtype) -> np.ndarray:
+        """The first `count` elements of t's buffer as `dtype`, whatever t's logical view
+        says (the packed words or scale bits of a quantized weight, for the loader's cache)."""
+        host = np.empty(count, dtype)
+        if host.nbytes > t.nbytes:
+            raise ValueError("_download_raw: more bytes than the buffer holds")
+        if host.nbytes:
+            L.call("tlhip_memcpy_d2h", host.ctypes.data, t.ptr, host.nbytes, self.stream)
+        L.call("tlhip_stream_synchronize", self.stream)
+        return host
+
     def synchronize(self) -> None:
         L.call("tlhip_stream_synchronize", self.stream)
 
