@@ -294,8 +294,10 @@ int tlhip_topk(const float* logits, int64_t offset, int64_t length, int k, float
 /* A launch configuration.  variant 0 = "gemv" (VALU dot), 1 = "gemv_mfma"
  * (skinny MFMA), 2 = "tiled" (prefill MFMA GEMM, both operands through LDS),
  * 3 = "tiled_direct" (prefill MFMA GEMM for int4, weights dequantised in
- * registers; fields as "tiled" with tile K 128 and 2x4 or 4x2 waves).
- * Unused fields are 0. */
+ * registers; fields as "tiled" with tile K 128 and 2x4 or 4x2 waves),
+ * 4 = "gemv_mfma_xreg" (skinny MFMA for int4 g32 with the activations held in
+ * registers: p0 waves per workgroup, p1 iterations in flight, p2 workgroups per
+ * CU, p3 K slices across workgroups).  Unused fields are 0. */
 typedef struct {
   int32_t variant;
   int32_t p0; /* gemv: lanes per row (16/32/64)   gemv_mfma: waves per workgroup   tiled: tile M */

@@ -385,3 +385,60 @@ def test_k_slices_are_stable_over_many_back_to_back_launches(be):
     for wi in range(3):
         ref = be.linear(xt, ws[wi], config=valu).numpy()
         assert rel_l2(firsts[wi], ref) <= 2e-6
+
+
+@pytest.mark.parametrize("n,k", [(4096, 12288), (1000, 4096), (12288, 4096), (40, 1024), (2049, 2048)])
+@pytest.mark.parametrize("m", [1, 2, 7, 16])
+def test_matrix_core_kernel_with_activations_in_registers(be, n, k, m):
+    """Every configuration of the register-resident-activation kernel (waves, iterations
+    in flight, workgroups per CU, K slices): the oracle's answer, and the same bits on a
+    second launch (the K-slice sum runs in slice order whoever arrives last)."""
+    rng = np.random.default_rng(n * 3 + k + m)
+    packed, scales, deq = make_weight("int4-grouped", n, k, 32, rng)
+    x = make_x(m, k, "f16", rng)
+    bias = rng.standard_normal(n).astype(np.float32)
+    want = O.linear(x.astype(np.float32), deq, bias, "silu", threads=8)
+    w = be.createQuantizedWeight(packed, scales, n, k, T.resolveWeightFormat("int4-32", "f32"))
+    xt = be.ops.tensorFromArray(x, [m, k], "f16")
+    bt = be.ops.tensorFromArray(bias, [n], "f32")
+    cands = [c for c in be.candidates(w, "f16", m, "f32") if c.variant == L.VARIANT_GEMV_XREG]
+    assert len(cands) >= 4, len(cands)
+    seen_slices = set()
+    for c in cands:
+        seen_slices.add(max(1, c.p3))
+        y1 = be.linear(xt, w, bt, "silu", fused=True, config=c)
+        y2 = be.linear(xt, w, bt, "silu", fused=True, config=c)
+        a, b = y1.numpy(), y2.numpy()
+        y1.destroy()
+        y2.destroy()
+        assert np.array_equal(a, b), c.as_tuple()
+        assert rel_l2(a, want) <= 5e-6, (c.as_tuple(), rel_l2(a, want))
+    assert len(seen_slices) >= 2
+
+
+def test_activations_in_registers_f16_out_and_rejections(be):
+    rng = np.random.default_rng(91)
+    n, k, m = 512, 2048, 9
+    packed, scales, deq = make_weight("int4-grouped", n, k, 32, rng)
+    x = make_x(m, k, "f16", rng)
+    w = be.createQuantizedWeight(packed, scales, n, k, T.resolveWeightFormat("int4-32", "f16"))
+    xt = be.ops.tensorFromArray(x, [m, k], "f16")
+    y = be.linear(xt, w, config=L.KernelConfig.of(4, 8, 2, 1, 1))   # 16 iterations = 8 waves x 1 step x 2
+    assert y.dtype == "f16"
+    assert rel_l2(y.numpy().astype(np.float32), O.linear(x.astype(np.float32), deq)) <= REL_L2_TOL
+    for bad in ((4, 8, 2, 1, 4),    # 4 slices: 4 iterations per slice cannot feed 8 waves x 2
+                (4, 3, 1, 1, 1),    # waves
+                (4, 8, 2, 3, 1),    # workgroups per CU
+                (4, 4, 1, 1, 1)):   # 16 iterations / 4 waves = 4 steps... allowed: must run
+        c = L.KernelConfig.of(*bad)
+        if bad == (4, 4, 1, 1, 1):
+            be.linear(xt, w, config=c).destroy()
+            continue
+        with pytest.raises(L.TlhipError, match="config not applicable"):
+            be.linear(xt, w, config=c)
+    # other formats, f32 activations, K not a multiple of 256: not this kernel's
+    p8, s8, _ = make_weight("int8-row", 64, 1024, 0, rng)
+    w8 = be.createQuantizedWeight(p8, s8, 64, 1024, T.resolveWeightFormat("int8-row", "f32"))
+    x8 = be.ops.tensorFromArray(make_x(2, 1024, "f16", rng), [2, 1024], "f16")
+    with pytest.raises(L.TlhipError, match="config not applicable"):
+        be.linear(x8, w8, config=L.KernelConfig.of(4, 8, 1, 1, 1))

@@ -22,7 +22,7 @@ UNARY = {"none": 0, "relu": 1, "silu": 2, "gelu": 3, "gelu_tanh": 3, "gelu_erf":
          "sigmoid": 5, "tanh": 6}
 EPI_NONE, EPI_BIAS, EPI_UNARY = 0, 1, 2
 MAX_EPILOGUE_OPS = 4
-VARIANT_GEMV, VARIANT_GEMV_MFMA, VARIANT_TILED, VARIANT_TILED_DIRECT = 0, 1, 2, 3
+VARIANT_GEMV, VARIANT_GEMV_MFMA, VARIANT_TILED, VARIANT_TILED_DIRECT, VARIANT_GEMV_XREG = 0, 1, 2, 3, 4
 
 
 class TlhipError(RuntimeError):

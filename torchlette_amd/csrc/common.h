@@ -79,6 +79,8 @@ bool gemv_group_compatible(const Problem* ps, int count, const tlhip_kernel_conf
 int launch_gemv_grouped(const Problem* ps, int count, const tlhip_kernel_config_t& c, hipStream_t stream);
 bool gemv_mfma_config_applicable(const Problem& p, const tlhip_kernel_config_t& c, const char** why);
 int launch_gemv_mfma(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t stream);
+bool gemv_xreg_config_applicable(const Problem& p, const tlhip_kernel_config_t& c, const char** why);
+int launch_gemv_xreg(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t stream);
 bool gemm_config_applicable(const Problem& p, const tlhip_kernel_config_t& c, const char** why);
 int launch_gemm(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t stream);
 bool gemm_direct_config_applicable(const Problem& p, const tlhip_kernel_config_t& c, const char** why);
@@ -99,6 +101,6 @@ void count_gemm_dispatch();
 void count_dequant_dispatch();
 void count_autotune_run();
 
-enum { VARIANT_GEMV = 0, VARIANT_GEMV_MFMA = 1, VARIANT_TILED = 2, VARIANT_TILED_DIRECT = 3 };
+enum { VARIANT_GEMV = 0, VARIANT_GEMV_MFMA = 1, VARIANT_TILED = 2, VARIANT_TILED_DIRECT = 3, VARIANT_GEMV_XREG = 4 };
 
 }  // namespace tlhip

@@ -80,6 +80,17 @@ tlhip_kernel_config_t mfma_cfg(int waves, int unroll, int kw, int ks = 1) {
   return c;
 }
 
+tlhip_kernel_config_t xreg_cfg(int waves, int unroll, int per_cu, int ks) {
+  tlhip_kernel_config_t c;
+  memset(&c, 0, sizeof c);
+  c.variant = VARIANT_GEMV_XREG;
+  c.p0 = waves;
+  c.p1 = unroll;
+  c.p2 = per_cu;
+  c.p3 = ks;
+  return c;
+}
+
 tlhip_kernel_config_t tiled_cfg(int tm, int tn, int tk, int wm, int wn) {
   tlhip_kernel_config_t c;
   memset(&c, 0, sizeof c);
@@ -103,6 +114,7 @@ bool config_applicable(const Problem& p, const tlhip_kernel_config_t& c, const c
   if (c.variant == VARIANT_TILED_DIRECT) return gemm_direct_config_applicable(p, c, why);
   if (c.variant == VARIANT_TILED) return gemm_config_applicable(p, c, why);
   if (c.variant == VARIANT_GEMV_MFMA) return gemv_mfma_config_applicable(p, c, why);
+  if (c.variant == VARIANT_GEMV_XREG) return gemv_xreg_config_applicable(p, c, why);
   return gemv_config_applicable(p, c, why);
 }
 
@@ -180,6 +192,15 @@ std::vector<tlhip_kernel_config_t> candidates(const Problem& p) {
             if (gemv_mfma_config_applicable(p, c, nullptr)) out.push_back(c);
           }
   }
+  if (p.m <= 16) {
+    for (int waves : {4, 8, 16})
+      for (int unroll : {1, 2})
+        for (int per_cu : {1, 2})
+          for (int ks : {1, 2, 4, 8, 16}) {
+            tlhip_kernel_config_t c = xreg_cfg(waves, unroll, per_cu, ks);
+            if (gemv_xreg_config_applicable(p, c, nullptr)) out.push_back(c);
+          }
+  }
   if (p.x_dtype == TLHIP_F16 && p.m >= 16) {
     static const int tiles[][5] = {
         {128, 128, 64, 2, 2}, {256, 128, 64, 2, 2}, {128, 256, 64, 2, 2},
@@ -211,6 +232,7 @@ int run_config(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t str
   if (c.variant == VARIANT_TILED_DIRECT) return launch_gemm_direct(p, c, stream);
   if (c.variant == VARIANT_TILED) return launch_gemm(p, c, stream);
   if (c.variant == VARIANT_GEMV_MFMA) return launch_gemv_mfma(p, c, stream);
+  if (c.variant == VARIANT_GEMV_XREG) return launch_gemv_xreg(p, c, stream);
   return launch_gemv(p, c, stream);
 }
 

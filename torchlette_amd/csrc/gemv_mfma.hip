@@ -24,7 +24,7 @@
 // LDS; with kw = 1 a wave owns a row block alone and nothing is combined.  The
 // weight loads of all row blocks of a workgroup form one software pipeline, as
 // in the VALU kernel.
-#include "device_utils.h"
+#include "gemv_mfma_common.h"
 
 namespace tlhip {
 namespace {
@@ -72,30 +72,6 @@ template <>
 struct MfmaTraits<TLHIP_FMT_INT8_ROW> {
   static constexpr int STEPS = 2;
 };
-
-__device__ __forceinline__ half8_t join8(const half2_t (&h)[4]) {
-  half8_t r;
-  r[0] = h[0][0]; r[1] = h[0][1]; r[2] = h[1][0]; r[3] = h[1][1];
-  r[4] = h[2][0]; r[5] = h[2][1]; r[6] = h[3][0]; r[7] = h[3][1];
-  return r;
-}
-
-// 4x4 transpose of 32-bit words across the four lanes l, l+16, l+32, l+48:
-// afterwards register i of lane-group g holds what register g of lane-group i
-// held.  Two swap stages: distance 32 on register pairs (0,2) (1,3), then
-// distance 16 on pairs (0,1) (2,3).
-__device__ __forceinline__ void transpose4(uint32_t& r0, uint32_t& r1, uint32_t& r2, uint32_t& r3) {
-  // v_permlane32_swap: lanes 32..63 of the first operand <-> lanes 0..31 of the second
-  auto s02 = __builtin_amdgcn_permlane32_swap(r0, r2, false, false);
-  r0 = s02[0]; r2 = s02[1];
-  auto s13 = __builtin_amdgcn_permlane32_swap(r1, r3, false, false);
-  r1 = s13[0]; r3 = s13[1];
-  // v_permlane16_swap: odd 16-lane rows of the first operand <-> even rows of the second
-  auto s01 = __builtin_amdgcn_permlane16_swap(r0, r1, false, false);
-  r0 = s01[0]; r1 = s01[1];
-  auto s23 = __builtin_amdgcn_permlane16_swap(r2, r3, false, false);
-  r2 = s23[0]; r3 = s23[1];
-}
 
 // Activations live in LDS row by row, as in global memory, 16-byte units, each
 // row padded by one unit: the 16 lanes of an MFMA operand read (16 different
@@ -287,13 +263,7 @@ __global__ __launch_bounds__(MAXT) void gemv_mfma_kernel(const MfmaArgs a) {
       owner = old == a.ks - 1;
       if (owner) {
         const float* tiles = a.workspace + (size_t)rb * a.ks * 256;
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          float sum = 0.f;
-          for (int sl = 0; sl < a.ks; ++sl)
-            sum += __hip_atomic_load(tiles + sl * 256 + (4 * g + r) * 16 + nl, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          t[r] = sum;
-        }
+        t = sum_slices(tiles, a.ks, (4 * g) * 16 + nl);
         if (lane == 0) __hip_atomic_store(a.counters + rb, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
     }
