@@ -204,10 +204,15 @@ def main() -> int:
     ap.add_argument("--no-details", action="store_true", help="skip the secondary measurements")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-autotune", action="store_true", help="use the heuristic kernel choices")
+    ap.add_argument("--dominant", default="",
+                    help="M,N,K of the call to report in `roofline` instead of the slowest one measured in this run "
+                         "(under a profiler the per-launch overhead shifts which call is slowest)")
+    ap.add_argument("--no-graphs", action="store_true",
+                    help="time the decode-token sections as stream launches only (no HIP graph capture / replay)")
     ap.add_argument("--autotune", action="store_true",
                     help="re-tune every case (weights rotating through HBM) even if a tuning cache file exists")
     ap.add_argument("--traffic-probe", action="store_true",
-                    help="for a counter run under rocprofv3 --pmc: 20 launches of the step's slowest call, then "
+                    help="for a counter run under rocprofv3 --pmc: 10 launches of each of the step's calls, then "
                          "three device-to-device copies of 256 MiB (the known size the counters are scaled by), and exit")
     ap.add_argument("--traffic-file", default=os.path.join(ROOT, "torchlette_amd", "tuning", "mi355x_traffic.json"),
                     help="measured HBM bytes per launch (from the counter runs), keyed by call; fills roofline.traffic")
@@ -254,21 +259,20 @@ def main() -> int:
     step_bytes = sum(c["bytes"] for c in cases)
 
     if args.traffic_probe:
-        for c in cases:
-            c["us"] = B.median_time(c["call"], 50, batches=3)
-        dom = max(cases, key=lambda c: c["us"])
         be.synchronize()
-        for _ in range(20):
-            dom["call"]()
-        be.synchronize()
+        for c in cases:  # fixed order, so that the FETCH and the WRITE run line up
+            for _ in range(10):
+                c["call"]()
+            be.synchronize()
+        slowest = cases
         nbytes = 256 << 20
         src, dst = be._alloc([nbytes // 4], "f32"), be._alloc([nbytes // 4], "f32")
         for _ in range(3):
             L.call("tlhip_memcpy_d2d", dst.ptr, src.ptr, nbytes, None)
         be.synchronize()
-        print(json.dumps({"traffic_probe": {"m": dom["m"], "n": dom["n"], "k": dom["k"], "kernel": dom["kernel"],
-                                            "config": dom["config"], "algorithmic_bytes": dom["bytes"],
-                                            "launches": 20, "copy_bytes": nbytes, "copies": 3}}))
+        print(json.dumps({"traffic_probe": {"cases": [
+            {"m": c["m"], "n": c["n"], "k": c["k"], "kernel": c["kernel"], "config": c["config"],
+             "algorithmic_bytes": c["bytes"]} for c in slowest], "launches": 10, "copy_bytes": nbytes, "copies": 3}}))
         return 0
 
     def step():
@@ -289,6 +293,9 @@ def main() -> int:
         c["us"] = B.median_time(c["call"], 200)
         c["gbps"] = c["bytes"] / c["us"] / 1e3
     dominant = max(cases, key=lambda c: c["us"])
+    if args.dominant:  # a profiler run: time the case the unprofiled run found dominant
+        dm, dn, dk = (int(v) for v in args.dominant.split(","))
+        dominant = next(c for c in cases if (c["m"], c["n"], c["k"]) == (dm, dn, dk))
     dom_us = B.median_time(dominant["call"], 500, batches=7)
     # HBM bytes per launch measured with FETCH_SIZE / WRITE_SIZE counter runs of --traffic-probe
     traffic = None
@@ -317,30 +324,6 @@ def main() -> int:
     }
 
     details = {}
-    # The same step submitted as ONE HIP graph launch (the reference batches a decode
-    # step's dispatches into one command-buffer submission, webgpu/shared-encoder.ts):
-    # eight captured steps, so that the weights still rotate through their pools.
-    L.call("tlhip_set_autotune_enabled", 0)
-    graphs = []
-    for _ in range(8):
-        g = C.c_void_p()
-        L.call("tlhip_graph_begin_capture", None)
-        step()
-        L.call("tlhip_graph_end_capture", None, C.byref(g))
-        graphs.append(g)
-    gstate = {"i": 0}
-
-    def step_graph():
-        L.call("tlhip_graph_launch", graphs[gstate["i"] % len(graphs)], None)
-        gstate["i"] += 1
-    for _ in range(args.warmup):
-        step_graph()
-    be.synchronize()
-    graph_us = float(np.median([B.time_region(step_graph, args.steps) for _ in range(3)]))
-    for g in graphs:
-        L.call("tlhip_graph_destroy", g)
-    details["step_as_hip_graph"] = {"us_per_step": round(graph_us, 2), "gbps": round(step_bytes / graph_us / 1e3, 1),
-                                    "frac_of_hbm_peak": round(step_bytes / graph_us / 1e3 / HBM_PEAK_GBPS, 4)}
     details["decode_calls"] = [
         {"m": c["m"], "n": c["n"], "k": c["k"], "us": round(c["us"], 2), "gbps": round(c["gbps"], 1),
          "frac_of_peak": round(c["gbps"] / HBM_PEAK_GBPS, 4), "kernel": c["kernel"], "config": c["config"]}
@@ -426,15 +409,21 @@ def main() -> int:
         token_bytes = 28 * sum(algorithmic_bytes("int4", n, k, 32, 1, 2, 2) for (n, k) in layer)
         us_stream = B.median_time(token, 5)
         L.call("tlhip_set_autotune_enabled", 0)
-        graph = C.c_void_p()
-        L.call("tlhip_graph_begin_capture", None)
-        token()
-        L.call("tlhip_graph_end_capture", None, C.byref(graph))
 
-        def replay():
-            L.call("tlhip_graph_launch", graph, None)
-        us_graph = B.median_time(replay, 5)
-        L.call("tlhip_graph_destroy", graph)
+        def graph_time(enqueue):
+            """Median time of replaying `enqueue`'s launches from one HIP graph (with
+            --no-graphs: of the stream launches themselves)."""
+            if args.no_graphs:
+                return B.median_time(enqueue, 5)
+            graph = C.c_void_p()
+            enqueue()
+            L.call("tlhip_graph_begin_capture", None)
+            enqueue()
+            L.call("tlhip_graph_end_capture", None, C.byref(graph))
+            us = B.median_time(lambda: L.call("tlhip_graph_launch", graph, None), 5)
+            L.call("tlhip_graph_destroy", graph)
+            return us
+        us_graph = graph_time(token)
 
         # the same 196 GEMVs with the Linears that share an activation row issued as
         # one launch each: (q, k, v), o, (gate, up), down = 4 launches per layer
@@ -461,11 +450,7 @@ def main() -> int:
                 if rc:
                     L.check(rc)
         us_grouped = B.median_time(token_grouped, 5)
-        L.call("tlhip_graph_begin_capture", None)
-        token_grouped()
-        L.call("tlhip_graph_end_capture", None, C.byref(graph))
-        us_grouped_graph = B.median_time(replay, 5)
-        L.call("tlhip_graph_destroy", graph)
+        us_grouped_graph = graph_time(token_grouped)
         # the same token with the producers of the Linears' inputs: RMSNorm in front of
         # (q, k, v) and of (gate, up), silu(gate) * up in front of down.  Apart: 7
         # launches per layer; fused into the GEMVs' activation staging: still 4.
@@ -508,16 +493,10 @@ def main() -> int:
                 chk(gpro(pg, ng, C.byref(pro_norm), L.F16, L.F16, 1.0, None))
                 chk(gpro(down_x[j], 1, C.byref(pro_gate), L.F16, L.F16, 1.0, None))
 
-        producer_us = {}
-        for name, fn in (("apart", token_producers_apart), ("fused", token_producers_fused)):
-            fn()
-            L.call("tlhip_graph_begin_capture", None)
-            fn()
-            L.call("tlhip_graph_end_capture", None, C.byref(graph))
-            producer_us[name] = B.median_time(replay, 5)
-            L.call("tlhip_graph_destroy", graph)
+        producer_us = {"apart": graph_time(token_producers_apart), "fused": graph_time(token_producers_fused)}
         details["qwen3_0p6b_decode_token_with_producers"] = {
-            "what": "28 layers: rmsnorm -> (q,k,v), o, rmsnorm -> (gate,up), silu(gate)*up -> down; HIP graph",
+            "what": "28 layers: rmsnorm -> (q,k,v), o, rmsnorm -> (gate,up), silu(gate)*up -> down; "
+                    + ("stream launches" if args.no_graphs else "HIP graph"),
             "launches_apart": 28 * 7, "us_per_token_apart": round(producer_us["apart"], 1),
             "launches_fused": 28 * 4, "us_per_token_fused": round(producer_us["fused"], 1)}
 

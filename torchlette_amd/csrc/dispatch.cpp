@@ -228,6 +228,14 @@ tlhip_kernel_config_t select_config(const Problem& p) {
   return default_config(p);
 }
 
+// The VALU configuration for launches only that kernel has (grouped, with a prologue):
+// the tuned or selected one if it is of that kernel, else the heuristic.
+tlhip_kernel_config_t valu_config(const Problem& p) {
+  tlhip_kernel_config_t c = select_config(p);
+  if (c.variant != VARIANT_GEMV) c = default_valu_config(p);
+  return c;
+}
+
 int run_config(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t stream) {
   if (c.variant == VARIANT_TILED_DIRECT) return launch_gemm_direct(p, c, stream);
   if (c.variant == VARIANT_TILED) return launch_gemm(p, c, stream);
@@ -413,12 +421,12 @@ int tlhip_gemv_grouped(const tlhip_gemv_problem_t* problems, int count, int x_dt
   int big = 0;
   for (int i = 1; i < count; ++i)
     if (ps[i].n > ps[big].n) big = i;
-  tlhip_kernel_config_t c = select_config(ps[big]);
-  if (c.variant == VARIANT_GEMV) {
-    c.p4 = 2;
-    if (c.p1 > 2) c.p1 = 2;
-    if (gemv_group_compatible(ps, count, c, nullptr)) return launch_gemv_grouped(ps, count, c, s);
-  }
+  // (one grouped launch of the VALU kernel beats separate launches of whichever kernel is
+  // fastest for a single problem: every launch costs 2-3 us)
+  tlhip_kernel_config_t c = valu_config(ps[big]);
+  c.p4 = 2;
+  if (c.p1 > 2) c.p1 = 2;
+  if (count > 1 && gemv_group_compatible(ps, count, c, nullptr)) return launch_gemv_grouped(ps, count, c, s);
   for (int i = 0; i < count; ++i) {
     int rc = matmul_with(ps[i], select_config(ps[i]), s);
     if (rc) return rc;
@@ -445,14 +453,6 @@ static int attach_prologue(const tlhip_prologue_t* pro, Problem* p, const char* 
   p->pro.eps = pro->eps;
   p->pro.operand = pro->operand;
   return TLHIP_OK;
-}
-
-// The VALU configuration a prologue launch runs with: the tuned or selected one if
-// it is of that kernel, else the heuristic.
-static tlhip_kernel_config_t valu_config(const Problem& p) {
-  tlhip_kernel_config_t c = select_config(p);
-  if (c.variant != VARIANT_GEMV) c = default_valu_config(p);
-  return c;
 }
 
 int tlhip_gemv_prologue(const tlhip_qweight_t* w, const tlhip_prologue_t* prologue, const void* x, int x_dtype,
