@@ -294,3 +294,47 @@ def test_grouped_gemv_with_rmsnorm_prologue(be, fmt, k, g, ns):
         assert rel_l2(o.numpy().astype(np.float32), single.numpy().astype(np.float32)) <= 2e-3
         single.destroy()
         o.destroy()
+
+
+def test_prologue_empty_problems(be):
+    """N = 0 and M = 0 launch nothing and say so (an empty output, no error)."""
+    rng = seeded("pro-empty")
+    k = 1024
+    packed, scales, _ = make_weight("int4-grouped", 16, k, 32, rng)
+    w = be.createQuantizedWeight(packed, scales, 16, k, T.resolveWeightFormat("int4-32", "f16"))
+    nwt = be.ops.tensorFromArray(norm_weight(k, rng), [k], "f32")
+    x0 = be.ops.zeros([0, k], "f16")
+    y0 = be.linearAfterRMSNorm(x0, nwt, 1e-6, w)
+    assert y0.numpy().shape == (0, 16)
+    u0 = be.ops.zeros([0, k], "f16")
+    assert be.linearAfterGatedMul(x0, u0, "silu", w).numpy().shape == (0, 16)
+    assert be.ops.gatedMul(x0, u0, "silu").numpy().shape == (0, k)
+
+
+def test_full_size_properties_of_the_fused_forms(be):
+    """At the Qwen3-8B decode shapes the oracle would take minutes; what must hold at any
+    size: the fused launch equals the two launches apart (same roundings of f(x), f32
+    accumulation order aside), RMSNorm ignores a power-of-two rescaling of x (eps = 0), and
+    a zero `up` row gives exactly zero."""
+    rng = seeded("pro-full")
+    n, k = 4096, 12288
+    packed = rng.integers(0, 2 ** 32, n * k // 8, dtype=np.uint64).astype(np.uint32)
+    scales = f16_round(rng.uniform(0.01, 0.05, n * k // 32)).view(np.uint16)
+    w = be.createQuantizedWeight(packed, scales, n, k, T.resolveWeightFormat("int4-32", "f16"))
+    x = make_x(2, k, "f16", rng, std=1.5)
+    xt = be.ops.tensorFromArray(x, [2, k], "f16")
+    nwt = be.ops.tensorFromArray(norm_weight(k, rng), [k], "f32")
+    fused = be.linearAfterRMSNorm(xt, nwt, 0.0, w).numpy().astype(np.float32)
+    normed = be.ops.fusedRMSNormForward(xt, nwt, {"numRows": 2, "featureDim": k, "eps": 0.0})
+    apart = be.linear(normed, w, fused=True).numpy().astype(np.float32)
+    assert rel_l2(fused, apart) <= F16_BAR
+    x4 = be.ops.tensorFromArray((x.astype(np.float32) * 4).astype(np.float16), [2, k], "f16")
+    again = be.linearAfterRMSNorm(x4, nwt, 0.0, w).numpy().astype(np.float32)
+    assert rel_l2(again, fused) <= F16_BAR
+    up = make_x(2, k, "f16", rng)
+    up[1] = 0
+    ut = be.ops.tensorFromArray(up, [2, k], "f16")
+    g = be.linearAfterGatedMul(xt, ut, "silu", w).numpy().astype(np.float32)
+    assert np.all(g[1] == 0.0) and np.any(g[0] != 0.0)
+    prod = be.ops.gatedMul(xt, ut, "silu")
+    assert rel_l2(g, be.linear(prod, w, fused=True).numpy().astype(np.float32)) <= F16_BAR
