@@ -481,12 +481,13 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& a, const int bid, cons
     load_batch(cur, rb, cfirst);
 #pragma unroll
     for (int i = 0; i < XS; ++i) {
-      const int idx = tid + i * (int)blockDim.x;
-      if (idx < units_total) {
-        u32x4 v = xr[i];
-        if (FMT == TLHIP_FMT_INT4_GROUPED && sizeof(XT) == 2) v = permute_x_for_int4(v);
-        *x_dst(idx) = v;
-      }
+      // Unconditional store at the clamped place (a thread past the end writes again
+      // what the last one writes): a store under a branch lets the compiler sink its
+      // load into the branch, behind the weight loads, and wait there for all of them.
+      const int idx = min(tid + i * (int)blockDim.x, units_total - 1);
+      u32x4 v = xr[i];
+      if (FMT == TLHIP_FMT_INT4_GROUPED && sizeof(XT) == 2) v = permute_x_for_int4(v);
+      *x_dst(idx) = v;
     }
   } else {
     load_batch(cur, rb, cfirst);
@@ -496,13 +497,11 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& a, const int bid, cons
 #pragma unroll
       for (int i = 0; i < 8; ++i) xr[i] = *x_src(min(base + tid + i * (int)blockDim.x, units_total - 1));
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const int idx = base + tid + i * (int)blockDim.x;
-        if (idx < units_total) {
-          u32x4 v = xr[i];
-          if (FMT == TLHIP_FMT_INT4_GROUPED && sizeof(XT) == 2) v = permute_x_for_int4(v);
-          *x_dst(idx) = v;
-        }
+      for (int i = 0; i < 8; ++i) {  // unconditional, clamped: see above
+        const int idx = min(base + tid + i * (int)blockDim.x, units_total - 1);
+        u32x4 v = xr[i];
+        if (FMT == TLHIP_FMT_INT4_GROUPED && sizeof(XT) == 2) v = permute_x_for_int4(v);
+        *x_dst(idx) = v;
       }
     }
   }
