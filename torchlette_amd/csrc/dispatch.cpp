@@ -139,9 +139,11 @@ tlhip_kernel_config_t default_config(const Problem& p) {
       if ((wgs >= cus || t[0] == 64) && gemm_config_applicable(p, c, nullptr)) return c;
     }
   }
-  // five or more activation rows: the matrix-core kernel streams the weights once
-  // (below that the VALU kernel with its rows held in registers measures faster)
-  if (p.m >= 5 && p.m <= 16) {
+  // three or more activation rows: the matrix-core kernel, whose time hardly depends on
+  // M (measured at the Qwen3-8B shapes: M = 4 takes 5.3 / 10.9 / 11.2 us against 7.5 /
+  // 13.4 / 15.1 us for the VALU kernel, whose dot products grow with M; at M = 2 the VALU
+  // kernel is still ahead, 5.3 / 8.9 / 9.9 against 6.0 / 10.3 / 11.5 us)
+  if (p.m >= 3 && p.m <= 16) {
     // the fewest K slices across workgroups whose activations fit LDS (measured best)
     for (int ks = 1; ks <= 16; ks *= 2)
       for (int unroll : {2, 1}) {
