@@ -442,3 +442,46 @@ def test_activations_in_registers_f16_out_and_rejections(be):
     x8 = be.ops.tensorFromArray(make_x(2, 1024, "f16", rng), [2, 1024], "f16")
     with pytest.raises(L.TlhipError, match="config not applicable"):
         be.linear(x8, w8, config=L.KernelConfig.of(4, 8, 1, 1, 1))
+
+
+@pytest.mark.parametrize("n,k,g", [(4096, 4096, 32), (1001, 2048, 32), (520, 12288, 32), (96, 256, 64), (300, 1024, 128)])
+@pytest.mark.parametrize("m", [1, 2, 3, 4])
+def test_dot_products_on_the_4x4x4_matrix_core_instruction(be, n, k, g, m):
+    """The form of the decode GEMV whose dot products go through v_mfma_f32_4x4x4_16b_f16
+    (config field p5 = 1): every such configuration, every M it takes, ragged N, bias and
+    activation in the epilogue; the products are exact, so the f32 bar applies."""
+    rng = np.random.default_rng(n + k + g + m)
+    packed, scales, deq = make_weight("int4-grouped", n, k, g, rng)
+    x = make_x(m, k, "f16", rng)
+    bias = rng.standard_normal(n).astype(np.float32)
+    want = O.linear(x.astype(np.float32), deq, bias, "silu", threads=8)
+    w = be.createQuantizedWeight(packed, scales, n, k, T.resolveWeightFormat(fmt_name("int4-grouped", g), "f32"))
+    xt = be.ops.tensorFromArray(x, [m, k], "f16")
+    bt = be.ops.tensorFromArray(bias, [n], "f32")
+    cands = [c for c in be.candidates(w, "f16", m, "f32") if c.variant == L.VARIANT_GEMV and c.p5 == 1]
+    assert len(cands) >= 6
+    for c in cands:
+        y = be.linear(xt, w, bt, "silu", fused=True, config=c)
+        got = y.numpy()
+        y.destroy()
+        assert rel_l2(got, want) <= 2e-6, (c.as_tuple(), rel_l2(got, want))
+
+
+def test_the_4x4x4_form_rejects_what_it_does_not_cover(be):
+    rng = np.random.default_rng(17)
+    packed, scales, _ = make_weight("int4-grouped", 64, 1024, 32, rng)
+    w = be.createQuantizedWeight(packed, scales, 64, 1024, T.resolveWeightFormat("int4-32", "f32"))
+    x5 = be.ops.tensorFromArray(make_x(5, 1024, "f16", rng), [5, 1024], "f16")
+    x1 = be.ops.tensorFromArray(make_x(1, 1024, "f16", rng), [1, 1024], "f16")
+    x32 = be.ops.tensorFromArray(make_x(1, 1024, "f32", rng), [1, 1024], "f32")
+    for xt, cfg in ((x5, (0, 16, 1, 4, 1, 2, 1)),     # five rows
+                    (x1, (0, 32, 1, 4, 1, 2, 1)),     # 32 lanes per row
+                    (x1, (0, 16, 2, 4, 1, 2, 1)),     # two rows per lane group
+                    (x32, (0, 16, 1, 4, 1, 2, 1)),    # f32 activations
+                    (x1, (0, 16, 1, 4, 1, 2, 2))):    # unknown form
+        with pytest.raises(L.TlhipError, match="config not applicable"):
+            be.linear(xt, w, config=L.KernelConfig.of(*cfg))
+    p8, s8, _ = make_weight("int8-row", 64, 1024, 0, rng)
+    w8 = be.createQuantizedWeight(p8, s8, 64, 1024, T.resolveWeightFormat("int8-row", "f32"))
+    with pytest.raises(L.TlhipError, match="config not applicable"):
+        be.linear(x1, w8, config=L.KernelConfig.of(0, 16, 1, 4, 1, 2, 1))

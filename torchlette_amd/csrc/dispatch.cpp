@@ -184,6 +184,17 @@ std::vector<tlhip_kernel_config_t> candidates(const Problem& p) {
               if (gemv_config_applicable(p, c, nullptr)) out.push_back(c);
             }
   }
+  if (p.m <= 4) {
+    // the 4x4x4 matrix-core form of the same kernel
+    for (int waves : {2, 4, 8})
+      for (int kw : {1, 2, 4})
+        for (int unroll : {2, 4, 8}) {
+          if (kw > waves) continue;
+          tlhip_kernel_config_t c = gemv_cfg(16, 1, waves, kw, unroll);
+          c.p5 = 1;
+          if (gemv_config_applicable(p, c, nullptr)) out.push_back(c);
+        }
+  }
   if (p.m <= 16) {
     for (int waves : {4, 8, 16})
       for (int unroll : {1, 2, 4})
@@ -427,6 +438,7 @@ int tlhip_gemv_grouped(const tlhip_gemv_problem_t* problems, int count, int x_dt
   // fastest for a single problem: every launch costs 2-3 us)
   tlhip_kernel_config_t c = valu_config(ps[big]);
   c.p4 = 2;
+  c.p5 = 0;  // the grouped kernel is the dot2 form
   if (c.p1 > 2) c.p1 = 2;
   if (count > 1 && gemv_group_compatible(ps, count, c, nullptr)) return launch_gemv_grouped(ps, count, c, s);
   for (int i = 0; i < count; ++i) {
@@ -495,6 +507,7 @@ int tlhip_gemv_grouped_prologue(const tlhip_gemv_problem_t* problems, int count,
     if (ps[i].n > ps[big].n) big = i;
   tlhip_kernel_config_t c = valu_config(ps[big]);
   c.p4 = 2;
+  c.p5 = 0;
   if (c.p1 > 2) c.p1 = 2;
   if (gemv_group_compatible(ps, count, c, nullptr)) return launch_gemv_grouped(ps, count, c, s);
   for (int i = 0; i < count; ++i) {

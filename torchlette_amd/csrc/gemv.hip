@@ -23,6 +23,7 @@ bool gemv_config_applicable(const Problem& p, const tlhip_kernel_config_t& c, co
       "group size must be a multiple of the chunk (32 for int4, 16 for int8)",
       "M above 16",
       "chunks in flight must be 2, 4 or 8 with rows*chunks <= 8",
+      "the 4x4x4 matrix-core form (p5 = 1) is built for int4 weights, f16 activations, M <= 4, 16 lanes per row, one row per lane group",
   };
   auto fail = [&](int i) {
     if (why) *why = reasons[i];
@@ -39,6 +40,9 @@ bool gemv_config_applicable(const Problem& p, const tlhip_kernel_config_t& c, co
   if (p.m > 16) return fail(7);
   const int u = c.p4 == 0 ? 2 : c.p4;
   if ((u != 2 && u != 4 && u != 8) || u * c.p1 > 8) return fail(8);
+  if (c.p5 != 0 && (c.p5 != 1 || p.format != TLHIP_FMT_INT4_GROUPED || p.x_dtype != TLHIP_F16 || p.m > 4 || c.p0 != 16 ||
+                    c.p1 != 1))
+    return fail(9);
   return true;
 }
 
@@ -48,7 +52,7 @@ static void fill_args(const Problem& p, const tlhip_kernel_config_t& c, int64_t 
   const int cw = chunk_weights(p.format);
   const int xbytes = p.x_dtype == TLHIP_F16 ? 2 : 4;
   const int ybytes = p.y_dtype == TLHIP_F16 ? 2 : 4;
-  mt = mrows == 1 ? 1 : (mrows == 2 ? 2 : 4);
+  mt = c.p5 == 1 ? 4 : (mrows == 1 ? 1 : (mrows == 2 ? 2 : 4));
   a.packed = (const u32x4*)p.packed;
   a.scales = p.scales;
   a.x = (const char*)p.x + m0 * p.k * xbytes;
@@ -77,7 +81,7 @@ static void fill_args(const Problem& p, const tlhip_kernel_config_t& c, int64_t 
   // LDS: staged x (mt rows) + split-K partials
   const int chunk_x_bytes = cw * xbytes;
   const size_t partial_bytes = a.kw > 1 ? (size_t)a.kw * a.rows_per_wg * mt * sizeof(float) : 0;
-  lds_bytes = (size_t)mt * chunk_x_bytes * a.nchunks + partial_bytes;
+  lds_bytes = (size_t)mt * chunk_x_bytes * a.nchunks + partial_bytes + (c.p5 == 1 ? 4 * 16 * 16 : 0);  // + the row skew
   threads = waves * 64;
   const int cus = device_cu_count();
   // resident workgroups per CU: bounded by 2048 lanes and by LDS
@@ -113,7 +117,8 @@ int launch_gemv(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t st
     int rc;
     switch (p.format) {
       case TLHIP_FMT_INT4_GROUPED:
-        rc = launch_gemv_int4(p.x_dtype, mt, r, unroll, a, threads, grid, lds_bytes, stream);
+        if (c.p5 == 1) rc = launch_gemv_mf4_int4(unroll, a, threads, grid, lds_bytes, stream);
+        else rc = launch_gemv_int4(p.x_dtype, mt, r, unroll, a, threads, grid, lds_bytes, stream);
         break;
       case TLHIP_FMT_INT8_GROUPED:
         rc = launch_gemv_int8_grouped(p.x_dtype, mt, r, unroll, a, threads, grid, lds_bytes, stream);

@@ -46,6 +46,7 @@ struct GroupedGemvArgs {
                          size_t lds_bytes, hipStream_t stream);                                          \
   int launch_gemv_grouped_##NAME(int r, const GroupedGemvArgs& g, int threads, size_t lds_bytes,          \
                                  hipStream_t stream);
+int launch_gemv_mf4_int4(int u, const GemvArgs& a, int threads, int grid, size_t lds_bytes, hipStream_t stream);
 TLHIP_DECLARE_GEMV_FORMAT(int4)
 TLHIP_DECLARE_GEMV_FORMAT(int8_grouped)
 TLHIP_DECLARE_GEMV_FORMAT(int8_row)

@@ -155,8 +155,20 @@ struct ChunkDot<TLHIP_FMT_INT4_GROUPED, float> {
 // `bid` / `nblk`: this workgroup's index among, and the number of, the workgroups
 // that work on this problem (the whole grid for a single launch; a slice of it
 // when several problems share one launch).
-template <int FMT, typename XT, int MT, int R, int U>
+// MF4 (int4, f16 activations, MT = 4, R = 1): the dot products of up to four activation
+// rows go through v_mfma_f32_4x4x4_16b_f16 instead of one v_dot2 chain per row.  The
+// instruction multiplies 16 independent 4 x 4 blocks: in block b (lanes 4b .. 4b+3) lane
+// 4b+i supplies row i of A (4 k-values of activation row i) and column i of B (the same 4
+// k-values of ITS weight row), and receives column i of D = A * B in its four
+// accumulators: D[m][i] = sum_k x[m][k] * w[row i][k] for m = 0..3.  So the four lanes of
+// a block hold four different weight rows and the same 16-byte chunk; the unpacked chunk
+// is consumed by 8 such instructions whatever M is, where the VALU form needs 16 dot2 per
+// activation row.  Lane mapping: row in the quad = lane % 4, chunk slot = lane / 4 (16
+// chunk slots per wave: "lanes per row" is 16).
+template <int FMT, typename XT, int MT, int R, int U, bool MF4 = false>
 __device__ __forceinline__ void gemv_body(const GemvArgs& a, const int bid, const int nblk) {
+  static_assert(!MF4 || (FMT == TLHIP_FMT_INT4_GROUPED && sizeof(XT) == 2 && MT == 4 && R == 1),
+                "the 4x4x4 form is built for int4 weights, f16 activations, four rows");
   using Dot = ChunkDot<FMT, XT>;
   constexpr int NQ = Dot::NQ;
   constexpr bool GROUPED = (FMT != TLHIP_FMT_INT8_ROW);
@@ -167,13 +179,17 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& a, const int bid, cons
   const int wave = tid >> 6;
   const int kw_idx = wave & (a.kw - 1);
   const int rg = wave >> a.kw_shift;
-  const int sub = lane >> a.lpr_shift;
-  const int lj = lane & (a.lpr - 1);
+  const int sub = MF4 ? (lane & 3) : (lane >> a.lpr_shift);
+  const int lj = MF4 ? (lane >> 2) : (lane & (a.lpr - 1));
   const int cstride = a.lpr * a.kw;
   const int cfirst = kw_idx * a.lpr + lj;
   const int x_units_per_row = a.k * (int)sizeof(XT) / 16;  // 16-byte units per activation row
   const u32x4* xg = (const u32x4*)a.x;
-  float* partial = (float*)(lds + (size_t)MT * NQ * a.nchunks);  // kw x rows_per_wg x MT, if kw > 1
+  // MF4: the four lanes of a block read four different activation rows at the same
+  // chunk; a skew of 16 units per row keeps them (and the 16 blocks) on 64 different
+  // 16-byte units instead of 4 lanes on each bank.
+  constexpr int XSKEW = MF4 ? 16 : 0;
+  float* partial = (float*)(lds + (size_t)MT * NQ * a.nchunks + MT * XSKEW);  // kw x rows_per_wg x MT, if kw > 1
   const int row_in_wg = rg * a.rows_per_wave + sub * R;
   const int last_chunk = a.nchunks - 1;
 
@@ -214,6 +230,36 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& a, const int bid, cons
   }
 
   auto compute_batch = [&](const Batch& b, int cb) {
+    if constexpr (MF4) {
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int c = cb + u * cstride;
+        const int cc = min(c, last_chunk);
+        // this lane's operand row: activation row `sub` of the chunk (rows past M read the last one)
+        const int xrow = min(sub, a.m - 1);
+        u32x4 xq[NQ];
+#pragma unroll
+        for (int qd = 0; qd < NQ; ++qd) xq[qd] = lds[(xrow * NQ + qd) * a.nchunks + xrow * XSKEW + cc];
+        Dot d;
+        d.unpack(b.w[u][0]);
+        float4_t dd = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+          // half2 pairs 2t, 2t+1 of the chunk, in the order the unpack produces (the
+          // staged activations have the same order)
+          const uint32_t xw[4] = {xq[t >> 1].x, xq[t >> 1].y, xq[t >> 1].z, xq[t >> 1].w};
+          const half2_t x0 = as_half2(xw[(2 * t) & 3]), x1 = as_half2(xw[(2 * t + 1) & 3]);
+          const half4_t av = {x0[0], x0[1], x1[0], x1[1]};
+          const half2_t w0 = d.q[2 * t], w1 = d.q[2 * t + 1];
+          const half4_t bv = {w0[0], w0[1], w1[0], w1[1]};
+          dd = __builtin_amdgcn_mfma_f32_4x4x4f16(av, bv, dd, 0, 0, 0);
+        }
+        const float sc = c <= last_chunk ? half_bits_to_float(b.s[u][0]) : 0.f;
+#pragma unroll
+        for (int m = 0; m < 4; ++m) acc[0][m] = fmaf(sc, dd[m], acc[0][m]);
+      }
+      return;
+    }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int c = cb + u * cstride;
@@ -243,7 +289,19 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& a, const int bid, cons
 #pragma unroll
     for (int r = 0; r < R; ++r)
 #pragma unroll
-      for (int m = 0; m < MT; ++m) acc[r][m] = group_sum(acc[r][m], a.lpr);
+      for (int m = 0; m < MT; ++m) {
+        if constexpr (MF4) {
+          // the 16 lanes of a weight row are lane % 4 apart
+          float v = acc[r][m];
+          v += __shfl_xor(v, 4);
+          v += __shfl_xor(v, 8);
+          v += __shfl_xor(v, 16);
+          v += __shfl_xor(v, 32);
+          acc[r][m] = v;
+        } else {
+          acc[r][m] = group_sum(acc[r][m], a.lpr);
+        }
+      }
 
     if (a.kw > 1) {
       // split-K combine through LDS: partial[kw][row in wg][m]
@@ -298,7 +356,9 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& a, const int bid, cons
   // the activations only, and the barrier for LDS only.
   constexpr int XS = 4;  // activation units a thread holds while its weight loads are in flight
   const int units = a.nchunks * NQ;
-  const int units_total = units * MT;
+  // MF4 stages the rows that exist (its lanes read row min(lane % 4, M - 1)); the dot2
+  // form stages MT rows, the ones past M as copies of the last
+  const int units_total = units * (MF4 ? a.m : MT);
   // idx -> (activation row m, 16-byte unit u) without a division: MT <= 4
   auto split = [&](int idx, int& m, int& u) {
     m = 0;
@@ -320,7 +380,7 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& a, const int bid, cons
     int m, u;
     split(idx, m, u);
     const int c = u / NQ, qd = u - c * NQ;
-    return lds + (m * NQ + qd) * a.nchunks + c;
+    return lds + (m * NQ + qd) * a.nchunks + m * XSKEW + c;
   };
   if (a.pro.kind != TLHIP_PRO_NONE) {
     // What is staged is f(x): see stage_with_prologue.
@@ -490,12 +550,15 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& a, const int bid, cons
       *x_dst(idx) = v;
     }
   } else {
-    load_batch(cur, rb, cfirst);
-    // groups of 8 units per thread: 8 loads in flight, then 8 LDS stores
-    for (int base = 0; base < units_total; base += 8 * (int)blockDim.x) {
-      u32x4 xr[8];
+    // groups of 8 units per thread: 8 loads in flight, then 8 LDS stores; the first
+    // group's loads go ahead of the first weight batch (they come from L2 and return
+    // first), the later groups queue behind it
+    u32x4 xr[8];
+    auto issue_x = [&](int base) {
 #pragma unroll
       for (int i = 0; i < 8; ++i) xr[i] = *x_src(min(base + tid + i * (int)blockDim.x, units_total - 1));
+    };
+    auto store_x = [&](int base) {
 #pragma unroll
       for (int i = 0; i < 8; ++i) {  // unconditional, clamped: see above
         const int idx = min(base + tid + i * (int)blockDim.x, units_total - 1);
@@ -503,6 +566,13 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& a, const int bid, cons
         if (FMT == TLHIP_FMT_INT4_GROUPED && sizeof(XT) == 2) v = permute_x_for_int4(v);
         *x_dst(idx) = v;
       }
+    };
+    issue_x(0);
+    load_batch(cur, rb, cfirst);
+    store_x(0);
+    for (int base = 8 * (int)blockDim.x; base < units_total; base += 8 * (int)blockDim.x) {
+      issue_x(base);
+      store_x(base);
     }
   }
   lds_barrier();
@@ -553,9 +623,9 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& a, const int bid, cons
   }
 }
 
-template <int FMT, typename XT, int MT, int R, int U>
+template <int FMT, typename XT, int MT, int R, int U, bool MF4 = false>
 __global__ __launch_bounds__(512) void gemv_kernel(const GemvArgs a) {
-  gemv_body<FMT, XT, MT, R, U>(a, blockIdx.x, gridDim.x);
+  gemv_body<FMT, XT, MT, R, U, MF4>(a, blockIdx.x, gridDim.x);
 }
 
 // Several problems of one shape class (same format, K, activation type, rows and
@@ -573,9 +643,9 @@ __global__ __launch_bounds__(512) void gemv_grouped_kernel(const GroupedGemvArgs
   gemv_body<FMT, XT, MT, R, U>(g.p[i], (int)blockIdx.x - g.first[i], g.first[i + 1] - g.first[i]);
 }
 
-template <int FMT, typename XT, int MT, int R, int U>
+template <int FMT, typename XT, int MT, int R, int U, bool MF4 = false>
 int launch_t(const GemvArgs& a, int threads, int grid, size_t lds_bytes, hipStream_t stream) {
-  const void* fn = (const void*)gemv_kernel<FMT, XT, MT, R, U>;
+  const void* fn = (const void*)gemv_kernel<FMT, XT, MT, R, U, MF4>;
   if (lds_bytes > 64 * 1024)
     TLHIP_CHECK_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
   void* args[] = {(void*)&a};
