@@ -434,7 +434,7 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& a, const int bid, cons
       // the squares; after the workgroup-wide sum every thread rescales the units
       // it parked itself, so no barrier is needed between the passes beyond the
       // one of the sum.
-      __shared__ float red[4][16];
+      __shared__ float red[4][17];  // [m][wave], and [m][16] = 1 / rms of row m
       float ss[MT];
 #pragma unroll
       for (int m = 0; m < MT; ++m) ss[m] = 0.f;
@@ -485,9 +485,7 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& a, const int bid, cons
             split(idx, m, u);
             float f[E];
             unit_to_floats<XT>(*x_dst(idx), f);
-            float s = inv[0];
-#pragma unroll
-            for (int mm = 1; mm < MT; ++mm) s = (mm == m) ? inv[mm] : s;
+            const float s = red[m][16];  // inv[m]: a register array indexed by m would live in scratch
 #pragma unroll
             for (int h = 0; h < E / 4; ++h) {
               f[4 * h + 0] = (f[4 * h + 0] * s) * as_float(wv[i][h].x);
@@ -524,6 +522,11 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& a, const int bid, cons
         for (int w = 0; w < nwaves; ++w) t += red[m][w];
         inv[m] = 1.f / sqrtf(t / (float)a.k + a.pro.eps);
       }
+      // Every thread holds the same values and writes them all, so each reads back
+      // what it wrote itself (a write by one lane for the others would need a barrier:
+      // the compiler may move the other lanes' read ahead of it).
+#pragma unroll
+      for (int m = 0; m < MT; ++m) red[m][16] = inv[m];
       rescale(0);
       for (int base = XS * T; base < units_total; base += XS * T) {
         issue_w(base);
