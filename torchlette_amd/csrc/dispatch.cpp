@@ -249,6 +249,16 @@ tlhip_kernel_config_t valu_config(const Problem& p) {
   return c;
 }
 
+// The grouped kernel is the dot2 form with two chunks in flight and one or two rows
+// per lane group: the tuned geometry where it is of that form, else the default one.
+tlhip_kernel_config_t grouped_config(const Problem& p) {
+  tlhip_kernel_config_t c = valu_config(p);
+  if (c.p5 != 0) c = default_valu_config(p);
+  c.p4 = 2;
+  if (c.p1 > 2) c.p1 = 2;
+  return c;
+}
+
 int run_config(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t stream) {
   if (c.variant == VARIANT_TILED_DIRECT) return launch_gemm_direct(p, c, stream);
   if (c.variant == VARIANT_TILED) return launch_gemm(p, c, stream);
@@ -436,10 +446,7 @@ int tlhip_gemv_grouped(const tlhip_gemv_problem_t* problems, int count, int x_dt
     if (ps[i].n > ps[big].n) big = i;
   // (one grouped launch of the VALU kernel beats separate launches of whichever kernel is
   // fastest for a single problem: every launch costs 2-3 us)
-  tlhip_kernel_config_t c = valu_config(ps[big]);
-  c.p4 = 2;
-  c.p5 = 0;  // the grouped kernel is the dot2 form
-  if (c.p1 > 2) c.p1 = 2;
+  const tlhip_kernel_config_t c = grouped_config(ps[big]);
   if (count > 1 && gemv_group_compatible(ps, count, c, nullptr)) return launch_gemv_grouped(ps, count, c, s);
   for (int i = 0; i < count; ++i) {
     int rc = matmul_with(ps[i], select_config(ps[i]), s);
@@ -505,10 +512,7 @@ int tlhip_gemv_grouped_prologue(const tlhip_gemv_problem_t* problems, int count,
   int big = 0;
   for (int i = 1; i < count; ++i)
     if (ps[i].n > ps[big].n) big = i;
-  tlhip_kernel_config_t c = valu_config(ps[big]);
-  c.p4 = 2;
-  c.p5 = 0;
-  if (c.p1 > 2) c.p1 = 2;
+  const tlhip_kernel_config_t c = grouped_config(ps[big]);
   if (gemv_group_compatible(ps, count, c, nullptr)) return launch_gemv_grouped(ps, count, c, s);
   for (int i = 0; i < count; ++i) {
     int rc = launch_gemv(ps[i], valu_config(ps[i]), s);

@@ -305,7 +305,7 @@ __global__ __launch_bounds__(MAXT) void gemv_mfma_kernel(const MfmaArgs a) {
   };
 
   // Activations first (they return first), then the first weight batch, then
-  // the LDS store.  Row by row, consecutive threads on consecutive 16-byte units.
+  // the LDS store; consecutive threads on consecutive 16-byte units of a row.
   const u32x4* xg = (const u32x4*)a.x + ku0;
   const int res_units = slice_units;
   int step = 0;
@@ -327,22 +327,53 @@ __global__ __launch_bounds__(MAXT) void gemv_mfma_kernel(const MfmaArgs a) {
       lds[min(m, mrows - 1) * row_units + ku] = v;
     }
   } else {
-    load_batch(cur, wgb, 0);
-    // 8 rows at a time: 8 loads in flight per thread, then 8 LDS stores
-    for (int kb = 0; kb < res_units; kb += blockDim.x) {
-      const int kuv = kb + tid;
-      const int ku = min(kuv, res_units - 1);
-      for (int m0 = 0; m0 < mrows; m0 += 8) {
-        u32x4 xr[8];
+    // The mrows x res_units resident units as one flat index, consecutive threads on
+    // consecutive units of a row; a thread issues a group of 16 loads, then the first
+    // weight batch, then stores the group to LDS.  The copy is bound by the latency of
+    // a round trip to L2, so what counts is the number of rounds (16 rows of K = 4096,
+    // or of a 3072-wide slice, on 512 threads: one).  A place past the end loads
+    // nothing and stores to the padding unit of the last row, which nobody reads: the
+    // store stays unconditional (see above), the load is what costs.
+    constexpr int G = 16;
+    const int T = (int)blockDim.x;
+    const int total_units = mrows * res_units;
+    const int pad = (mrows - 1) * row_units + res_units;
+    // idx -> (row, unit): one division per thread, then stepped by T
+    const int qT = T / res_units, rT = T - qT * res_units;
+    int m = tid / res_units, ku = tid - m * res_units;
+    u32x4 xr[G];
+    int dst[G];
+    auto issue_x = [&]() {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) xr[i] = xg[(size_t)min(m0 + i, mrows - 1) * k_units + ku];
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {  // unconditional, clamped: see above
-          u32x4 v = xr[i];
-          if (FMT == TLHIP_FMT_INT4_GROUPED) v = permute_x_for_int4(v);
-          lds[min(m0 + i, mrows - 1) * row_units + ku] = v;
+      for (int i = 0; i < G; ++i) {
+        xr[i] = (u32x4){0u, 0u, 0u, 0u};
+        dst[i] = pad;
+        if (m < mrows) {
+          xr[i] = xg[(size_t)m * k_units + ku];
+          dst[i] = m * row_units + ku;
+        }
+        m += qT;
+        ku += rT;
+        if (ku >= res_units) {
+          ku -= res_units;
+          ++m;
         }
       }
+    };
+    auto store_x = [&]() {
+#pragma unroll
+      for (int i = 0; i < G; ++i) {
+        u32x4 v = xr[i];
+        if (FMT == TLHIP_FMT_INT4_GROUPED) v = permute_x_for_int4(v);
+        lds[dst[i]] = v;
+      }
+    };
+    issue_x();
+    load_batch(cur, wgb, 0);
+    store_x();
+    for (int base = G * T; base < total_units; base += G * T) {
+      issue_x();
+      store_x();
     }
   }
   lds_barrier();
