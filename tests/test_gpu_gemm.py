@@ -58,7 +58,8 @@ def test_every_tile_config_ragged_shapes(be, fmt, g, bm, bn):
     assert rel_l2(got, want) <= REL_L2_TOL, rel_l2(got, want)
 
 
-DIRECT_TILES = [(256, 256, 2, 4), (256, 128, 2, 4), (128, 256, 2, 4), (256, 128, 4, 2), (128, 128, 2, 2), (256, 256, 2, 2)]
+DIRECT_TILES = [(256, 256, 2, 4), (256, 128, 2, 4), (128, 256, 2, 4), (256, 128, 4, 2), (128, 128, 2, 2), (256, 256, 2, 2),
+                (128, 256, 1, 4)]
 
 
 @pytest.mark.parametrize("bm,bn,wm,wn", DIRECT_TILES)

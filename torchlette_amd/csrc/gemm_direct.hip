@@ -36,7 +36,12 @@ namespace tlhip {
 namespace {
 
 constexpr int DK = 128;            // k per step
-constexpr int DROW_UNITS = 17;     // LDS row of X: 128 f16 = 16 units + 1 unit of padding
+// LDS row of X: 128 f16 = 16 units of 16 bytes.  Two layouts keep the A operand reads
+// (32 rows, one unit column) off each other's banks: a 17th unit of padding per row, or
+// (SWZ) no padding and the unit column XOR-ed with the low four bits of the row.  The
+// second one makes a 128-row tile with its 256-row W buffer exactly 80 KB: two
+// workgroups per CU.
+constexpr int row_units(bool swz) { return swz ? 16 : 17; }
 
 struct DirectArgs {
   const uint8_t* packed;  // row stride K/2 bytes
@@ -54,8 +59,9 @@ struct DirectArgs {
 // WM x WN waves, each owning TM x TN MFMA tiles of 32 x 32.  G32: one scale per
 // 16-byte chunk (group size 32), the two scales of a lane's step come as one
 // 4-byte load.
-template <int WM, int WN, int TM, int TN, bool G32>
-__global__ __launch_bounds__(WM * WN * 64) void gemm_direct_kernel(const DirectArgs a) {
+template <int WM, int WN, int TM, int TN, bool G32, bool SWZ>
+__global__ __launch_bounds__(WM * WN * 64, (TM * TN >= 16 ? 1 : 2)) void gemm_direct_kernel(const DirectArgs a) {
+  constexpr int DROW_UNITS = row_units(SWZ);
   constexpr int THREADS = WM * WN * 64;
   constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
   constexpr int X_LOADS = BM * 16 / THREADS;  // 16-byte units of the X tile per thread per step
@@ -139,7 +145,8 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_direct_kernel(const DirectA
 #pragma unroll
     for (int i = 0; i < XH; ++i) {
       const int u = tid + (part * XH + i) * THREADS;
-      xs[(u >> 4) * DROW_UNITS + (u & 15)] = permute_x_for_int4(xr[i]);
+      const int r = u >> 4, c = u & 15;
+      xs[r * DROW_UNITS + (SWZ ? (c ^ (r & 15)) : c)] = permute_x_for_int4(xr[i]);
     }
   };
 
@@ -186,8 +193,11 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_direct_kernel(const DirectA
     }
   };
   half8_t af[TM];
+  // SWZ: the lane's unit column for group kk is (8*lk + kk) ^ (row & 15) = acol ^ kk with
+  // row & 15 = lrow & 15 (the other terms of the row are multiples of 32)
+  const int acol = (lk * 8) ^ (lrow & 15);
   auto read_a = [&](int buf, int kk, int i) {
-    const u32x4* xs = lds + buf * X_UNITS + (wm * TM * 32 + lrow) * DROW_UNITS + lk * 8 + kk;
+    const u32x4* xs = lds + buf * X_UNITS + (wm * TM * 32 + lrow) * DROW_UNITS + (SWZ ? (acol ^ kk) : lk * 8 + kk);
     af[i] = __builtin_bit_cast(half8_t, xs[i * 32 * DROW_UNITS]);
   };
   // MFMAs of one group; `next` >= 0: re-read each A operand for group `next`
@@ -279,12 +289,12 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_direct_kernel(const DirectA
     wave_epilogue<TN>(patch, acc[i], lane, m0 + (wm * TM + i) * 32, n0 + wn * TN * 32, a.out);
 }
 
-template <int WM, int WN, int TM, int TN>
+template <int WM, int WN, int TM, int TN, bool SWZ = false>
 int launch_direct_tile(const DirectArgs& a, bool g32, hipStream_t stream) {
   constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
-  const void* fn = g32 ? (const void*)gemm_direct_kernel<WM, WN, TM, TN, true>
-                       : (const void*)gemm_direct_kernel<WM, WN, TM, TN, false>;
-  size_t lds_bytes = (size_t)(2 * BM * DROW_UNITS + BN * 4) * 16;
+  const void* fn = g32 ? (const void*)gemm_direct_kernel<WM, WN, TM, TN, true, SWZ>
+                       : (const void*)gemm_direct_kernel<WM, WN, TM, TN, false, SWZ>;
+  size_t lds_bytes = (size_t)(2 * BM * row_units(SWZ) + BN * 4) * 16;
   const size_t patch_bytes = (size_t)WM * WN * 32 * (TN * 32 + 4) * sizeof(float);
   if (lds_bytes < patch_bytes) lds_bytes = patch_bytes;
   if (lds_bytes > 64 * 1024)
@@ -308,6 +318,7 @@ constexpr DirectTile kDirectTiles[] = {
     {256, 128, 4, 2},  // wave tile 64 x 64
     {128, 128, 2, 2},  // wave tile 64 x 64, 4 waves: two workgroups share a CU
     {256, 256, 2, 2},  // wave tile 128 x 128, 4 waves, one per SIMD
+    {128, 256, 1, 4},  // wave tile 128 x 64, 4 waves, swizzled X: 80 KB of LDS, two workgroups share a CU
 };
 
 }  // namespace
@@ -319,7 +330,7 @@ bool gemm_direct_config_applicable(const Problem& p, const tlhip_kernel_config_t
       "activations must be f16",
       "K must be a multiple of 128",
       "group size must be a multiple of 32",
-      "tile (M, N, waves M, waves N) must be one of 256x256 2x4, 256x128 2x4, 128x256 2x4, 256x128 4x2, 128x128 2x2, 256x256 2x2 with tile K 128",
+      "tile (M, N, waves M, waves N) must be one of 256x256 2x4, 256x128 2x4, 128x256 2x4, 256x128 4x2, 128x128 2x2, 256x256 2x2, 128x256 1x4 with tile K 128",
   };
   auto fail = [&](int i) {
     if (why) *why = reasons[i];
@@ -364,6 +375,7 @@ int launch_gemm_direct(const Problem& p, const tlhip_kernel_config_t& c, hipStre
   if (c.p0 == 256 && c.p1 == 256 && c.p4 == 2) rc = launch_direct_tile<2, 2, 4, 4>(a, g32, stream);
   else if (c.p0 == 256 && c.p1 == 256) rc = launch_direct_tile<2, 4, 4, 2>(a, g32, stream);
   else if (c.p0 == 256 && c.p1 == 128 && c.p3 == 2) rc = launch_direct_tile<2, 4, 4, 1>(a, g32, stream);
+  else if (c.p0 == 128 && c.p1 == 256 && c.p3 == 1) rc = launch_direct_tile<1, 4, 4, 2, true>(a, g32, stream);
   else if (c.p0 == 128 && c.p1 == 256) rc = launch_direct_tile<2, 4, 2, 2>(a, g32, stream);
   else if (c.p0 == 128 && c.p1 == 128) rc = launch_direct_tile<2, 2, 2, 2>(a, g32, stream);
   else rc = launch_direct_tile<4, 2, 2, 2>(a, g32, stream);
