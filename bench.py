@@ -214,6 +214,8 @@ def main() -> int:
     ap.add_argument("--traffic-probe", action="store_true",
                     help="for a counter run under rocprofv3 --pmc: 10 launches of each of the step's calls, then "
                          "three device-to-device copies of 256 MiB (the known size the counters are scaled by), and exit")
+    ap.add_argument("--prefill-probe", action="store_true",
+                    help="counter runs: only launch the prefill GEMM (M = 512, 2048, 8192; bias + silu), 5 launches each")
     ap.add_argument("--traffic-file", default=os.path.join(ROOT, "torchlette_amd", "tuning", "mi355x_traffic.json"),
                     help="measured HBM bytes per launch (from the counter runs), keyed by call; fills roofline.traffic")
     ap.add_argument("--tuning-cache", default=os.path.join(ROOT, "torchlette_amd", "tuning", "mi355x.json"),
@@ -273,6 +275,24 @@ def main() -> int:
         print(json.dumps({"traffic_probe": {"cases": [
             {"m": c["m"], "n": c["n"], "k": c["k"], "kernel": c["kernel"], "config": c["config"],
              "algorithmic_bytes": c["bytes"]} for c in slowest], "launches": 10, "copy_bytes": nbytes, "copies": 3}}))
+        return 0
+
+    if args.prefill_probe:
+        n, k = 12288, 4096
+        w = pools[(n, k)][0]
+        bias = be.ops.tensorFromArray((B.rng.standard_normal(n) * 0.1).astype(np.float16), [n], "f16")
+        ep = be.makeEpilogue(bias, "silu")
+        runs = []
+        for m in (512, 2048, 8192):
+            x, _ = B.activations(m, k, std=0.5)
+            out = be._alloc([m, n], "f16")
+            call = B.make_call([w], x, m, out, epilogue=ep)
+            for _ in range(5):
+                call()
+            be.synchronize()
+            runs.append({"m": m, "n": n, "k": k, "flops": 2.0 * m * n * k,
+                         "config": list(be.selectedConfig(w, "f16", m, "f16").as_tuple())})
+        print(json.dumps({"prefill_probe": {"cases": runs, "launches": 5}}))
         return 0
 
     def step():

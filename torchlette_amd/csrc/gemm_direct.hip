@@ -23,11 +23,15 @@
 //     covers k = 64*lk + 32*c + 8*w + (0..7) for lane half lk, and the A operand
 //     reads the activations of exactly those k from LDS;
 //   * X goes global -> registers -> LDS in parts spread over the step, written
-//     with the (0,4,1,5,2,6,3,7) order the int4 unpack produces, rows padded to
-//     272 bytes, double buffered; the W buffer is single (a second LDS-only
-//     barrier in the middle of the step frees it), which keeps a 256 x 256 tile
-//     within the 160 KB of LDS;
-//   * 8 waves (2 per SIMD) per workgroup.
+//     with the (0,4,1,5,2,6,3,7) order the int4 unpack produces.  LDS holds HALF a
+//     step of X twice: the MFMA groups 0..3 of a step read the k-columns
+//     {0..3, 8..11} (16-byte units of the 128-k row), the groups 4..7 the columns
+//     {4..7, 12..15}; while one half is read the other is written (the second half
+//     of this step during its first half, the first half of the next step during
+//     its second half), and the two LDS-only barriers of a step - in the middle
+//     and at the end - are what the single W buffer needs anyway.  A 128-row tile
+//     with a 256-row W buffer takes 48 KB, so two workgroups share a CU;
+//   * 4 or 8 waves per workgroup, two waves per SIMD resident.
 // MFMA-bound by design: per MFMA a wave reads 1 KB / TN from LDS and spends
 // 14 / TM VALU instructions on dequantisation.
 #include "gemm_common.h"
@@ -36,12 +40,10 @@ namespace tlhip {
 namespace {
 
 constexpr int DK = 128;            // k per step
-// LDS row of X: 128 f16 = 16 units of 16 bytes.  Two layouts keep the A operand reads
-// (32 rows, one unit column) off each other's banks: a 17th unit of padding per row, or
-// (SWZ) no padding and the unit column XOR-ed with the low four bits of the row.  The
-// second one makes a 128-row tile with its 256-row W buffer exactly 80 KB: two
-// workgroups per CU.
-constexpr int row_units(bool swz) { return swz ? 16 : 17; }
+// LDS row of half a step of X: 8 units of 16 bytes, the unit column XOR-ed with bits
+// 1..3 of the row, so that the 16 lanes of an A operand read (16 rows, one column)
+// fall on 16 different bank groups.
+constexpr int HROW_UNITS = 8;
 
 struct DirectArgs {
   const uint8_t* packed;  // row stride K/2 bytes
@@ -59,16 +61,15 @@ struct DirectArgs {
 // WM x WN waves, each owning TM x TN MFMA tiles of 32 x 32.  G32: one scale per
 // 16-byte chunk (group size 32), the two scales of a lane's step come as one
 // 4-byte load.
-template <int WM, int WN, int TM, int TN, bool G32, bool SWZ>
+template <int WM, int WN, int TM, int TN, bool G32>
 __global__ __launch_bounds__(WM * WN * 64, (TM * TN >= 16 ? 1 : 2)) void gemm_direct_kernel(const DirectArgs a) {
-  constexpr int DROW_UNITS = row_units(SWZ);
   constexpr int THREADS = WM * WN * 64;
   constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
   constexpr int X_LOADS = BM * 16 / THREADS;  // 16-byte units of the X tile per thread per step
   constexpr int W_LOADS = BN * 4 / THREADS;   // 16-byte chunks of the W tile per thread per step
   static_assert(BM * 16 % THREADS == 0 && BN * 4 % THREADS == 0, "tiles must divide over the threads");
-  constexpr int X_UNITS = BM * DROW_UNITS;
-  extern __shared__ u32x4 lds[];  // X buffer 0, X buffer 1, W buffer
+  constexpr int X_UNITS = BM * HROW_UNITS;  // half a step of the X tile
+  extern __shared__ u32x4 lds[];  // X first half, X second half, W buffer
   u32x4* const lds_w = lds + 2 * X_UNITS;
 
   const int tid = threadIdx.x;
@@ -126,27 +127,29 @@ __global__ __launch_bounds__(WM * WN * 64, (TM * TN >= 16 ? 1 : 2)) void gemm_di
     }
   };
 
-  // ---- X: global -> registers -> LDS in NXP parts per step ---------------------
-  constexpr int NXP = X_LOADS >= 4 ? 4 : 2;
-  constexpr int XH = X_LOADS / NXP;
-  static_assert(X_LOADS % NXP == 0, "X tile units per thread must divide into the staging parts");
+  // ---- X: global -> registers -> LDS, two parts per half step -----------------------
+  // unit u of a half: row u / 8, column c = u % 8 = 4 * lk + j, which is unit
+  // 8 * lk + 4 * half + j of the step's 128-k row
+  static_assert(X_LOADS % 4 == 0, "X tile units per thread must divide into four staging parts");
+  constexpr int XH = X_LOADS / 4;
   u32x4 xr[XH];
-  auto load_x = [&](int step, int part) {
+  auto load_x = [&](int step, int half, int part) {
     const int k0 = min(step, a.ksteps - 1) * DK;
 #pragma unroll
     for (int i = 0; i < XH; ++i) {
       const int u = tid + (part * XH + i) * THREADS;
-      const int row = min(m0 + (u >> 4), a.m - 1);
-      xr[i] = *(const u32x4*)(a.x + (size_t)row * a.k + k0 + (u & 15) * 8);
+      const int row = min(m0 + (u >> 3), a.m - 1);
+      const int c = u & 7;
+      xr[i] = *(const u32x4*)(a.x + (size_t)row * a.k + k0 + ((c >> 2) * 8 + half * 4 + (c & 3)) * 8);
     }
   };
-  auto store_x = [&](int buf, int part) {
-    u32x4* xs = lds + buf * X_UNITS;
+  auto store_x = [&](int half, int part) {
+    u32x4* xs = lds + half * X_UNITS;
 #pragma unroll
     for (int i = 0; i < XH; ++i) {
       const int u = tid + (part * XH + i) * THREADS;
-      const int r = u >> 4, c = u & 15;
-      xs[r * DROW_UNITS + (SWZ ? (c ^ (r & 15)) : c)] = permute_x_for_int4(xr[i]);
+      const int r = u >> 3, c = u & 7;
+      xs[r * HROW_UNITS + (c ^ ((r >> 1) & 7))] = permute_x_for_int4(xr[i]);
     }
   };
 
@@ -193,36 +196,36 @@ __global__ __launch_bounds__(WM * WN * 64, (TM * TN >= 16 ? 1 : 2)) void gemm_di
     }
   };
   half8_t af[TM];
-  // SWZ: the lane's unit column for group kk is (8*lk + kk) ^ (row & 15) = acol ^ kk with
-  // row & 15 = lrow & 15 (the other terms of the row are multiples of 32)
-  const int acol = (lk * 8) ^ (lrow & 15);
-  auto read_a = [&](int buf, int kk, int i) {
-    const u32x4* xs = lds + buf * X_UNITS + (wm * TM * 32 + lrow) * DROW_UNITS + (SWZ ? (acol ^ kk) : lk * 8 + kk);
-    af[i] = __builtin_bit_cast(half8_t, xs[i * 32 * DROW_UNITS]);
+  // group kk reads column 4 * lk + kk % 4 of half kk / 4; the row's swizzle term is
+  // (lrow >> 1) & 7 (the other terms of the row are multiples of 32)
+  const int acol = (lk * 4) ^ ((lrow >> 1) & 7);
+  auto read_a = [&](int kk, int i) {
+    const u32x4* xs = lds + (kk >> 2) * X_UNITS + (wm * TM * 32 + lrow) * HROW_UNITS + (acol ^ (kk & 3));
+    af[i] = __builtin_bit_cast(half8_t, xs[i * 32 * HROW_UNITS]);
   };
   // MFMAs of one group; `next` >= 0: re-read each A operand for group `next`
-  auto group = [&](int buf, const half8_t (&bf)[TN], int next) {
+  auto group = [&](const half8_t (&bf)[TN], int next) {
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
 #pragma unroll
       for (int j = 0; j < TN; ++j)
         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
-      if (next >= 0) read_a(buf, next, i);
+      if (next >= 0) read_a(next, i);
     }
   };
 
   // ---- pipeline -----------------------------------------------------------------
-  // X and W of step s+1 are loaded to registers while step s computes and go to
-  // the other LDS buffers before the barrier that ends the step; the scales are
-  // one more step ahead.  Every load is unconditional (clamped past the end).
+  // W of step s+1 and the halves of X are loaded to registers while step s computes
+  // and go to LDS before the barrier behind which they are read; the scales are one
+  // more step ahead.  Every load is unconditional (clamped past the end).
   Scales s0, s1;
   half8_t bfA[TN], bfB[TN];
   load_s(0, s0);
   load_s(1, s1);
   load_w(0);
 #pragma unroll
-  for (int p = 0; p < NXP; ++p) {
-    load_x(0, p);
+  for (int p = 0; p < 2; ++p) {
+    load_x(0, 0, p);
     store_x(0, p);
   }
   store_w();
@@ -230,46 +233,44 @@ __global__ __launch_bounds__(WM * WN * 64, (TM * TN >= 16 ? 1 : 2)) void gemm_di
   // The scheduling fences keep the compiler from sinking the global loads to
   // their use (the LDS store), which would expose their latency.
   auto step = [&](int s, Scales& sc) {
-    const int buf = s & 1;
     load_w(s + 1);
-    load_x(s + 1, 0);
+    load_x(s, 1, 0);
     read_w(0);
     read_w(1);
 #pragma unroll
-    for (int i = 0; i < TM; ++i) read_a(buf, 0, i);
+    for (int i = 0; i < TM; ++i) read_a(0, i);
     dequant(sc, 0, bfA);
     __builtin_amdgcn_sched_barrier(0);
-    dequant(sc, 1, bfB); group(buf, bfA, 1);
-    dequant(sc, 2, bfA); group(buf, bfB, 2);
-    if (NXP == 4) {
-      __builtin_amdgcn_sched_barrier(0);
-      store_x(buf ^ 1, 0);
-      load_x(s + 1, 1);
-      __builtin_amdgcn_sched_barrier(0);
-    }
-    dequant(sc, 3, bfB); group(buf, bfA, 3);
-    dequant(sc, 4, bfA); group(buf, bfB, 4);
+    dequant(sc, 1, bfB); group(bfA, 1);
+    dequant(sc, 2, bfA); group(bfB, 2);
     __builtin_amdgcn_sched_barrier(0);
-    store_x(buf ^ 1, NXP == 4 ? 1 : 0);
-    load_x(s + 1, NXP == 4 ? 2 : 1);
-    // the single W buffer: every wave took its chunks of this step at the top of
-    // the step; the barrier makes that certain before the next step's go in
+    store_x(1, 0);
+    load_x(s, 1, 1);
+    __builtin_amdgcn_sched_barrier(0);
+    dequant(sc, 3, bfB); group(bfA, 3);
+    // group 3 re-reads nothing: the second half of X is whole only behind the barrier
+    dequant(sc, 4, bfA); group(bfB, -1);
+    __builtin_amdgcn_sched_barrier(0);
+    store_x(1, 1);
+    load_x(s + 1, 0, 0);
+    // the barrier also frees the single W buffer: every wave took its chunks of this
+    // step at the top of the step
     lds_barrier();
     store_w();
+#pragma unroll
+    for (int i = 0; i < TM; ++i) read_a(4, i);
     __builtin_amdgcn_sched_barrier(0);
-    dequant(sc, 5, bfB); group(buf, bfA, 5);
-    dequant(sc, 6, bfA); group(buf, bfB, 6);
-    if (NXP == 4) {
-      __builtin_amdgcn_sched_barrier(0);
-      store_x(buf ^ 1, 2);
-      load_x(s + 1, 3);
-      __builtin_amdgcn_sched_barrier(0);
-    }
-    dequant(sc, 7, bfB); group(buf, bfA, 7);
-    group(buf, bfB, -1);
+    dequant(sc, 5, bfB); group(bfA, 5);
+    dequant(sc, 6, bfA); group(bfB, 6);
+    __builtin_amdgcn_sched_barrier(0);
+    store_x(0, 0);
+    load_x(s + 1, 0, 1);
+    __builtin_amdgcn_sched_barrier(0);
+    dequant(sc, 7, bfB); group(bfA, 7);
+    group(bfB, -1);
     __builtin_amdgcn_sched_barrier(0);
     load_s(s + 2, sc);
-    store_x(buf ^ 1, NXP - 1);
+    store_x(0, 1);
     lds_barrier();
   };
   // Whole pairs in the loop and the odd step after it: a step under a branch
@@ -289,12 +290,12 @@ __global__ __launch_bounds__(WM * WN * 64, (TM * TN >= 16 ? 1 : 2)) void gemm_di
     wave_epilogue<TN>(patch, acc[i], lane, m0 + (wm * TM + i) * 32, n0 + wn * TN * 32, a.out);
 }
 
-template <int WM, int WN, int TM, int TN, bool SWZ = false>
+template <int WM, int WN, int TM, int TN>
 int launch_direct_tile(const DirectArgs& a, bool g32, hipStream_t stream) {
   constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
-  const void* fn = g32 ? (const void*)gemm_direct_kernel<WM, WN, TM, TN, true, SWZ>
-                       : (const void*)gemm_direct_kernel<WM, WN, TM, TN, false, SWZ>;
-  size_t lds_bytes = (size_t)(2 * BM * row_units(SWZ) + BN * 4) * 16;
+  const void* fn = g32 ? (const void*)gemm_direct_kernel<WM, WN, TM, TN, true>
+                       : (const void*)gemm_direct_kernel<WM, WN, TM, TN, false>;
+  size_t lds_bytes = (size_t)(2 * BM * HROW_UNITS + BN * 4) * 16;
   const size_t patch_bytes = (size_t)WM * WN * 32 * (TN * 32 + 4) * sizeof(float);
   if (lds_bytes < patch_bytes) lds_bytes = patch_bytes;
   if (lds_bytes > 64 * 1024)
@@ -318,7 +319,7 @@ constexpr DirectTile kDirectTiles[] = {
     {256, 128, 4, 2},  // wave tile 64 x 64
     {128, 128, 2, 2},  // wave tile 64 x 64, 4 waves: two workgroups share a CU
     {256, 256, 2, 2},  // wave tile 128 x 128, 4 waves, one per SIMD
-    {128, 256, 1, 4},  // wave tile 128 x 64, 4 waves, swizzled X: 80 KB of LDS, two workgroups share a CU
+    {128, 256, 1, 4},  // wave tile 128 x 64, 4 waves, 48 KB of LDS: two workgroups share a CU
 };
 
 }  // namespace
@@ -375,7 +376,7 @@ int launch_gemm_direct(const Problem& p, const tlhip_kernel_config_t& c, hipStre
   if (c.p0 == 256 && c.p1 == 256 && c.p4 == 2) rc = launch_direct_tile<2, 2, 4, 4>(a, g32, stream);
   else if (c.p0 == 256 && c.p1 == 256) rc = launch_direct_tile<2, 4, 4, 2>(a, g32, stream);
   else if (c.p0 == 256 && c.p1 == 128 && c.p3 == 2) rc = launch_direct_tile<2, 4, 4, 1>(a, g32, stream);
-  else if (c.p0 == 128 && c.p1 == 256 && c.p3 == 1) rc = launch_direct_tile<1, 4, 4, 2, true>(a, g32, stream);
+  else if (c.p0 == 128 && c.p1 == 256 && c.p3 == 1) rc = launch_direct_tile<1, 4, 4, 2>(a, g32, stream);
   else if (c.p0 == 128 && c.p1 == 256) rc = launch_direct_tile<2, 4, 2, 2>(a, g32, stream);
   else if (c.p0 == 128 && c.p1 == 128) rc = launch_direct_tile<2, 2, 2, 2>(a, g32, stream);
   else rc = launch_direct_tile<4, 2, 2, 2>(a, g32, stream);
