@@ -137,6 +137,33 @@ def test_matrix_core_kernel_with_k_slices_across_workgroups(be, fmt, n, k, g, m)
     assert ran >= 3
 
 
+@pytest.mark.parametrize("fmt,n,k,g", [
+    ("int4-grouped", 200, 256, 32),     # a row shorter than a workgroup: several rows per staging step
+    ("int4-grouped", 130, 768, 64),     # 96 units per row: not a divisor of any workgroup size
+    ("int4-grouped", 96, 5120, 128),    # more than one staging round at M = 16
+    ("int8-row", 150, 1344, 0),
+    ("int8-grouped", 64, 640, 64),
+])
+@pytest.mark.parametrize("m", [5, 9, 16])
+def test_matrix_core_kernel_activation_staging_geometries(be, fmt, n, k, g, m):
+    """The flat (row, unit) staging of the 16x16x32 kernel: every workgroup size, K split
+    and slice count the kernel takes for these shapes, rows longer and shorter than a
+    workgroup, M below a full tile (the rows past M alias the last row)."""
+    rng = np.random.default_rng(7 * n + k + m)
+    packed, scales, deq = make_weight(fmt, n, k, g, rng)
+    x = make_x(m, k, "f16", rng)
+    want = O.linear(x.astype(np.float32), deq, threads=8)
+    w = be.createQuantizedWeight(packed, scales, n, k, T.resolveWeightFormat(fmt_name(fmt, g), "f32"))
+    xt = be.ops.tensorFromArray(x, [m, k], "f16")
+    cands = [c for c in be.candidates(w, "f16", m, "f32") if c.variant == L.VARIANT_GEMV_MFMA]
+    assert len(cands) >= 4
+    for c in cands:
+        y = be.linear(xt, w, config=c)
+        got = y.numpy()
+        y.destroy()
+        assert rel_l2(got, want) <= 5e-6, (c.as_tuple(), rel_l2(got, want))
+
+
 def test_k_slices_reject_what_the_workspace_cannot_hold(be):
     rng = np.random.default_rng(5)
     n, k, m = 256, 1024, 8
