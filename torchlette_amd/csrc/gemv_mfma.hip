@@ -164,6 +164,9 @@ __global__ __launch_bounds__(MAXT) void gemv_mfma_kernel(const MfmaArgs a) {
   };
 
   float4_t acc = {0.f, 0.f, 0.f, 0.f};
+  // one scale per row (no per-group f32 step between the MFMAs): two accumulators take
+  // the MFMA steps in turn, so that consecutive MFMAs of a wave do not depend on each other
+  float4_t acc_odd = {0.f, 0.f, 0.f, 0.f};
 
   auto compute_batch = [&](const Batch& b, int step) {
     const int bidx = kw_idx + step * a.kw;
@@ -199,7 +202,8 @@ __global__ __launch_bounds__(MAXT) void gemv_mfma_kernel(const MfmaArgs a) {
 #pragma unroll
           for (int s = 0; s < STEPS; ++s) {
             const u32x4 xa = lds[x_unit<FMT>(tl + s, g, ml, row_units)];
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, xa), bw[s], acc, 0, 0, 0);
+            if (s & 1) acc_odd = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, xa), bw[s], acc_odd, 0, 0, 0);
+            else acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, xa), bw[s], acc, 0, 0, 0);
           }
         }
       } else if (FMT == TLHIP_FMT_INT8_GROUPED) {
@@ -292,6 +296,10 @@ __global__ __launch_bounds__(MAXT) void gemv_mfma_kernel(const MfmaArgs a) {
   // block: 3 us of a 12 us kernel, 6 us with four K slices.)
   int round = 0;
   auto finish = [&](int wb) {
+    if (!GROUPED) {
+      acc += acc_odd;
+      acc_odd = (float4_t){0.f, 0.f, 0.f, 0.f};
+    }
     if (a.kw == 1) {
       const int rb = wb * a.blocks_per_wg + bw_idx;
       if (rb < a.nblocks) emit(rb, acc);
