@@ -113,9 +113,13 @@ class Bench:
         L.call("tlhip_event_elapsed_us", self.ev0, self.ev1, C.byref(us))
         return us.value / reps
 
-    def median_time(self, enqueue, reps: int, batches: int = 5) -> float:
-        enqueue()
-        self.be.synchronize()
+    def median_time(self, enqueue, reps: int, batches: int = 5, warm_ms: float = 50.0) -> float:
+        # untimed batches first, `warm_ms` of GPU time: the section before may have left the
+        # GPU idle while the host prepared data, and the launches after that run at a lower
+        # clock for some milliseconds (the same kernel measured 8-12 % slower without)
+        spent = 0.0
+        while spent < warm_ms * 1e3:
+            spent += self.time_region(enqueue, reps) * reps
         return float(np.median([self.time_region(enqueue, reps) for _ in range(batches)]))
 
     def make_call(self, pool, x, m: int, out, epilogue=None, out_dtype: str = "f16"):
@@ -199,8 +203,8 @@ def cpu_step(cases, host_weights, host_x, threads: int) -> float:
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--no-details", action="store_true", help="skip the secondary measurements")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-autotune", action="store_true", help="use the heuristic kernel choices")
