@@ -113,12 +113,14 @@ class Bench:
         L.call("tlhip_event_elapsed_us", self.ev0, self.ev1, C.byref(us))
         return us.value / reps
 
-    def median_time(self, enqueue, reps: int, batches: int = 5, warm_ms: float = 50.0) -> float:
+    warm_ms = 50.0
+
+    def median_time(self, enqueue, reps: int, batches: int = 5) -> float:
         # untimed batches first, `warm_ms` of GPU time: the section before may have left the
         # GPU idle while the host prepared data, and the launches after that run at a lower
         # clock for some milliseconds (the same kernel measured 8-12 % slower without)
         spent = 0.0
-        while spent < warm_ms * 1e3:
+        while spent < self.warm_ms * 1e3:
             spent += self.time_region(enqueue, reps) * reps
         return float(np.median([self.time_region(enqueue, reps) for _ in range(batches)]))
 
@@ -205,6 +207,9 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=100)
+    ap.add_argument("--warm-ms", type=float, default=50.0,
+                    help="GPU milliseconds of untimed launches before each timed section (small for profiler runs, "
+                         "whose traces grow with every launch)")
     ap.add_argument("--no-details", action="store_true", help="skip the secondary measurements")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-autotune", action="store_true", help="use the heuristic kernel choices")
@@ -231,6 +236,7 @@ def main() -> int:
         return 2
 
     B = Bench()
+    B.warm_ms = args.warm_ms
     T, L, be = B.T, B.L, B.be
     info = be.deviceInfo()
     # Kernel choices: a committed tuning cache (importTuningCache) when there is one,

@@ -69,6 +69,13 @@ __global__ __launch_bounds__(WM * WN * 64, (TM * TN >= 16 ? 1 : 2)) void gemm_di
   constexpr int W_LOADS = BN * 4 / THREADS;   // 16-byte chunks of the W tile per thread per step
   static_assert(BM * 16 % THREADS == 0 && BN * 4 % THREADS == 0, "tiles must divide over the threads");
   constexpr int X_UNITS = BM * HROW_UNITS;  // half a step of the X tile
+  // The 256x128 tile of eight 128x32 waves issues its MFMA groups at raised priority,
+  // so that the wave it shares a SIMD with (same workgroup, same barriers, the same
+  // phase of the step) does not delay them with its dequantisation: measured 2.5-3.5 %
+  // faster at M = 512..8192.  Every other tile measured 2-7 % SLOWER with the same two
+  // instructions (the four-wave tiles whichever way round the priorities are), so they
+  // stay without.
+  constexpr bool MFMA_PRIO = WM == 2 && WN == 4 && TM == 4 && TN == 1;
   extern __shared__ u32x4 lds[];  // X first half, X second half, W buffer
   u32x4* const lds_w = lds + 2 * X_UNITS;
 
@@ -205,6 +212,7 @@ __global__ __launch_bounds__(WM * WN * 64, (TM * TN >= 16 ? 1 : 2)) void gemm_di
   };
   // MFMAs of one group; `next` >= 0: re-read each A operand for group `next`
   auto group = [&](const half8_t (&bf)[TN], int next) {
+    if constexpr (MFMA_PRIO) __builtin_amdgcn_s_setprio(1);
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
 #pragma unroll
@@ -212,6 +220,7 @@ __global__ __launch_bounds__(WM * WN * 64, (TM * TN >= 16 ? 1 : 2)) void gemm_di
         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
       if (next >= 0) read_a(next, i);
     }
+    if constexpr (MFMA_PRIO) __builtin_amdgcn_s_setprio(0);
   };
 
   // ---- pipeline -----------------------------------------------------------------
