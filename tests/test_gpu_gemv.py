@@ -229,6 +229,46 @@ def test_reference_probe_shapes_int8_grouped(be):
             assert per_row_err(got, O.linear(a.reshape(1, k), deq)) <= cases["per_row_tol"]
 
 
+@pytest.mark.parametrize("waves,unroll", [(4, 4), (4, 2), (8, 4), (8, 2), (16, 2)])
+@pytest.mark.parametrize("n,k,m", [(515, 1280, 2), (100, 256, 16), (4103, 2304, 8), (16, 128, 1), (9000, 512, 5)])
+def test_matrix_core_gemv_with_whole_line_weight_loads(be, n, k, m, waves, unroll):
+    """int8 with one scale per row, the form whose loads take 128-byte lines (8 lanes to a
+    row) and pass through a wave-private LDS patch: ragged N (rows past the end alias the
+    last row), one to many 128-k pairs per batch, several row blocks per wave; bias +
+    activation; against the oracle and against the same kernel with operand-layout loads."""
+    rng = np.random.default_rng(n + k + m + waves + unroll)
+    packed, scales, deq = make_weight("int8-row", n, k, 0, rng)
+    x = make_x(m, k, "f16", rng)
+    bias = rng.standard_normal(n).astype(np.float32)
+    cfg = L.KernelConfig.of(1, waves, unroll, 1, 1, 0, 1)
+    if (k // 64) % unroll != 0:
+        with pytest.raises(L.TlhipError, match="config not applicable"):
+            run_linear(be, "int8-row", packed, scales, n, k, 0, x, "f32", config=cfg)
+        return
+    got = run_linear(be, "int8-row", packed, scales, n, k, 0, x, "f32", bias=bias, act="silu", fused=True, config=cfg)
+    want = O.linear(x.astype(np.float32), deq, bias, "silu")
+    assert got.shape == (m, n)
+    assert rel_l2(got, want) <= 2e-6, rel_l2(got, want)
+    plain = run_linear(be, "int8-row", packed, scales, n, k, 0, x, "f32", bias=bias, act="silu", fused=True,
+                       config=L.KernelConfig.of(1, waves, unroll, 1, 1))
+    assert np.array_equal(got, plain)
+
+
+def test_whole_line_weight_loads_reject_what_they_do_not_cover(be):
+    rng = np.random.default_rng(9)
+    x = make_x(2, 192, "f16", rng)
+    packed, scales, _ = make_weight("int8-row", 64, 192, 0, rng)
+    with pytest.raises(L.TlhipError, match="whole-line weight loads"):   # K = 192 is not a multiple of 128
+        run_linear(be, "int8-row", packed, scales, 64, 192, 0, x, "f32", config=L.KernelConfig.of(1, 4, 1, 1, 1, 0, 1))
+    x = make_x(2, 256, "f16", rng)
+    packed, scales, _ = make_weight("int8-row", 64, 256, 0, rng)
+    with pytest.raises(L.TlhipError, match="whole-line weight loads"):   # a K split across waves
+        run_linear(be, "int8-row", packed, scales, 64, 256, 0, x, "f32", config=L.KernelConfig.of(1, 4, 2, 2, 1, 0, 1))
+    packed4, scales4, _ = make_weight("int4-grouped", 64, 256, 32, rng)
+    with pytest.raises(L.TlhipError, match="whole-line weight loads"):   # another format
+        run_linear(be, "int4-grouped", packed4, scales4, 64, 256, 32, x, "f32", config=L.KernelConfig.of(1, 4, 2, 1, 1, 0, 1))
+
+
 def test_lm_head_sized_n(be):
     """N = 151936 (the probe's lm_head case) and the Gemma-shaped 256000 x 2304 int8-row."""
     rng = np.random.default_rng(3)

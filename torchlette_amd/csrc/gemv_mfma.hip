@@ -86,8 +86,18 @@ __device__ __forceinline__ int x_unit(int t, int g, int m, int row_units) {
   return m * row_units + ku;
 }
 
-template <int FMT, int U, bool WIDE, int MAXT>
+//
+// LINE (int8 with one scale per row, no K split, U even): a wave's weight loads take
+// whole 128-byte lines, 8 lanes to a row and 8 rows to an instruction, with the
+// nontemporal hint, instead of the operand layout's 64-byte pieces of 16 rows; a batch
+// then goes through a wave-private LDS patch (written as loaded, read back in the
+// operand layout, no barrier: one wave's LDS accesses stay in order) before it is
+// consumed exactly as before.  A read-only kernel streams the LM head's 590 MB in
+// 84-86 us with the first load shape and in 94-95 us (plain) or 102-106 us (hint) with
+// the second.
+template <int FMT, int U, bool WIDE, int MAXT, bool LINE = false>
 __global__ __launch_bounds__(MAXT) void gemv_mfma_kernel(const MfmaArgs a) {
+  static_assert(!LINE || (FMT == TLHIP_FMT_INT8_ROW && U % 2 == 0), "whole-line loads: int8-row, even U");
   using Tr = MfmaTraits<FMT>;
   constexpr int STEPS = Tr::STEPS;
   constexpr bool GROUPED = (FMT != TLHIP_FMT_INT8_ROW);
@@ -137,13 +147,28 @@ __global__ __launch_bounds__(MAXT) void gemv_mfma_kernel(const MfmaArgs a) {
     const u32x4* wrow = a.packed + row * a.nchunks;
     const uint16_t* srow = (const uint16_t*)a.scales + row * a.groups_per_row;
     const int itb = it_begin + min(kw_idx + step * a.kw, nbatches - 1) * U;
+    if constexpr (LINE) {
+      // pair p of the batch = 128 k = one line per row: rows 0..7 of the block in
+      // register 2p, rows 8..15 in register 2p+1, lane = 8 * row + 16-byte chunk
+      const int r8 = lane >> 3, c8 = lane & 7;
+      const int64_t row_lo = min((int64_t)rb * 16 + r8, a.n - 1);
+      const int64_t row_hi = min((int64_t)rb * 16 + 8 + r8, a.n - 1);
+      const u32x4* wlo = a.packed + row_lo * a.nchunks + c8;
+      const u32x4* whi = a.packed + row_hi * a.nchunks + c8;
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      // Nontemporal loads for the grouped formats (measured 0.3-0.5 us per call faster at
-      // the 8-28 MB decode shapes); plain loads for one scale per row, the format of the
-      // 590 MB LM head, where they measured 5 % faster (115.7 -> 110.1 us at M = 8).
-      if (GROUPED) b.w[u] = __builtin_nontemporal_load(wrow + (itb + u) * 4 + g);
-      else b.w[u] = wrow[(itb + u) * 4 + g];
+      for (int p2 = 0; p2 < U / 2; ++p2) {
+        b.w[2 * p2] = __builtin_nontemporal_load(wlo + (itb + 2 * p2) * 4);
+        b.w[2 * p2 + 1] = __builtin_nontemporal_load(whi + (itb + 2 * p2) * 4);
+      }
+    } else {
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        // Nontemporal loads for the grouped formats (measured 0.3-0.5 us per call faster at
+        // the 8-28 MB decode shapes); plain loads for one scale per row, the format of the
+        // 590 MB LM head, where they measured 5 % faster (115.7 -> 110.1 us at M = 8).
+        if (GROUPED) b.w[u] = __builtin_nontemporal_load(wrow + (itb + u) * 4 + g);
+        else b.w[u] = wrow[(itb + u) * 4 + g];
+      }
     }
     if (WIDE) {
       if (U == 1) {
@@ -178,10 +203,29 @@ __global__ __launch_bounds__(MAXT) void gemv_mfma_kernel(const MfmaArgs a) {
     const int bidx = kw_idx + step * a.kw;
     const bool valid = bidx < nbatches;  // wave-uniform
     const int tlb = min(bidx, nbatches - 1) * U * STEPS;
+    u32x4 wv[U];
+    if constexpr (LINE) {
+      // through the wave's patch: 16 rows x 8 chunks per pair, the chunk position
+      // XOR-ed with the row so that the operand reads (16 rows, one chunk) spread
+      // over the banks
+      u32x4* st = lds + (size_t)row_units * mrows + wave * (U / 2 * 128);
+      const int r8 = lane >> 3, c8 = lane & 7;
+#pragma unroll
+      for (int p2 = 0; p2 < U / 2; ++p2) {
+        st[p2 * 128 + r8 * 8 + (c8 ^ r8)] = b.w[2 * p2];
+        st[p2 * 128 + (r8 + 8) * 8 + (c8 ^ r8)] = b.w[2 * p2 + 1];
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        wv[u] = st[(u >> 1) * 128 + nl * 8 + ((g + 4 * (u & 1)) ^ (nl & 7))];
+    } else {
+#pragma unroll
+      for (int u = 0; u < U; ++u) wv[u] = b.w[u];
+    }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int tl = tlb + u * STEPS;
-      uint32_t w0 = b.w[u].x, w1 = b.w[u].y, w2 = b.w[u].z, w3 = b.w[u].w;
+      uint32_t w0 = wv[u].x, w1 = wv[u].y, w2 = wv[u].z, w3 = wv[u].w;
       half8_t bw[STEPS];
       if (FMT == TLHIP_FMT_INT4_GROUPED) {
         transpose4(w0, w1, w2, w3);  // register s now holds word g of chunk 4*it+s
@@ -466,7 +510,7 @@ struct MfmaGeometry {
   int grid;
   size_t lds_bytes;
 };
-static bool mfma_geometry(int64_t n, int64_t k, int64_t m, int waves, int kw, int ks, MfmaGeometry* out) {
+static bool mfma_geometry(int64_t n, int64_t k, int64_t m, int waves, int kw, int ks, size_t patch_bytes, MfmaGeometry* out) {
   const int threads = waves * 64;
   const int64_t nblocks = (n + 15) / 16;
   const int blocks_per_wg = waves / kw;
@@ -484,7 +528,7 @@ static bool mfma_geometry(int64_t n, int64_t k, int64_t m, int waves, int kw, in
     if (sets < 1) sets = 1;
     const int64_t rounds = (nwgblocks + sets - 1) / sets;
     const size_t parked = kw > 1 ? (size_t)rounds * waves * 1024 : 0;
-    const size_t lds = x_bytes + parked;
+    const size_t lds = x_bytes + parked + patch_bytes;
     if (lds * per_cu <= kXLdsBudget) {
       out->grid = (int)(sets * ks);
       out->lds_bytes = lds;
@@ -492,6 +536,11 @@ static bool mfma_geometry(int64_t n, int64_t k, int64_t m, int waves, int kw, in
     }
   }
   return false;
+}
+
+// LDS of the wave-private patches of the whole-line form: 2 KB per pair of iterations.
+static size_t line_patch_bytes(const tlhip_kernel_config_t& c) {
+  return c.p5 == 1 ? (size_t)c.p0 * c.p1 * 1024 : 0;
 }
 
 bool gemv_mfma_config_applicable(const Problem& p, const tlhip_kernel_config_t& c, const char** why) {
@@ -508,6 +557,8 @@ bool gemv_mfma_config_applicable(const Problem& p, const tlhip_kernel_config_t& 
       "K slices must be a power of two (1..16) that divides K/128 (int4) or K/64 (int8)",
       "K slices need more partial-tile workspace or counters than the library holds",
       "iterations in flight must divide the 128-weight (int4) or 64-weight (int8) steps of a K slice",
+      "whole-line weight loads (p5 = 1) need int8 with one scale per row, K a multiple of 128, 2 or 4 iterations in "
+      "flight and no K split (p2 = 1, p3 <= 1)",
   };
   auto fail = [&](int i) {
     if (why) *why = reasons[i];
@@ -528,8 +579,11 @@ bool gemv_mfma_config_applicable(const Problem& p, const tlhip_kernel_config_t& 
   const int ks = c.p3 < 1 ? 1 : c.p3;
   const int64_t iters = p.k / kper;
   if (ks > 16 || (ks & (ks - 1)) != 0 || iters % ks != 0) return fail(9);
+  if (c.p5 != 0 && !(c.p5 == 1 && p.format == TLHIP_FMT_INT8_ROW && p.k % 128 == 0 && (c.p1 == 2 || c.p1 == 4) &&
+                     kw == 1 && ks == 1))
+    return fail(12);
   MfmaGeometry geo;
-  if (!mfma_geometry(p.n, p.k, p.m, c.p0, kw, ks, &geo)) return fail(8);
+  if (!mfma_geometry(p.n, p.k, p.m, c.p0, kw, ks, line_patch_bytes(c), &geo)) return fail(8);
   if ((iters / ks) % c.p1 != 0) return fail(11);
   if (ks > 1) {
     const int64_t nblocks = (p.n + 15) / 16;
@@ -551,6 +605,19 @@ static int launch_mfma_u(int unroll, const MfmaArgs& a, int grid, int threads, s
       default: fn = (const void*)gemv_mfma_kernel<FMT, 4, WIDE, 512>; break;
     }
   }
+  if (lds_bytes > 64 * 1024)
+    TLHIP_CHECK_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+  void* args[] = {(void*)&a};
+  TLHIP_CHECK_HIP(hipLaunchKernel(fn, dim3(grid), dim3(threads), args, lds_bytes, stream));
+  return TLHIP_OK;
+}
+
+// int8 with one scale per row, whole-line weight loads (2 or 4 iterations in flight).
+static int launch_mfma_line(int unroll, const MfmaArgs& a, int grid, int threads, size_t lds_bytes, hipStream_t stream) {
+  const void* fn;
+  if (threads > 512) fn = (const void*)gemv_mfma_kernel<TLHIP_FMT_INT8_ROW, 2, false, 1024, true>;
+  else if (unroll == 2) fn = (const void*)gemv_mfma_kernel<TLHIP_FMT_INT8_ROW, 2, false, 512, true>;
+  else fn = (const void*)gemv_mfma_kernel<TLHIP_FMT_INT8_ROW, 4, false, 512, true>;
   if (lds_bytes > 64 * 1024)
     TLHIP_CHECK_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
   void* args[] = {(void*)&a};
@@ -599,7 +666,7 @@ int launch_gemv_mfma(const Problem& p, const tlhip_kernel_config_t& c, hipStream
   a.y_dtype = p.y_dtype;
   a.epi = p.epi;
   MfmaGeometry geo;
-  if (!mfma_geometry(p.n, p.k, p.m, waves, a.kw, a.ks, &geo))
+  if (!mfma_geometry(p.n, p.k, p.m, waves, a.kw, a.ks, line_patch_bytes(c), &geo))
     return set_error(TLHIP_ERR_INVALID, "gemv_mfma: launch geometry does not close");
   const size_t lds_bytes = geo.lds_bytes;
   const int threads = waves * 64;
@@ -614,7 +681,10 @@ int launch_gemv_mfma(const Problem& p, const tlhip_kernel_config_t& c, hipStream
         rc = launch_mfma_u<TLHIP_FMT_INT4_GROUPED, false>(unroll, a, grid, threads, lds_bytes, stream);
       break;
     case TLHIP_FMT_INT8_GROUPED: rc = launch_mfma_u<TLHIP_FMT_INT8_GROUPED, false>(unroll, a, grid, threads, lds_bytes, stream); break;
-    default: rc = launch_mfma_u<TLHIP_FMT_INT8_ROW, false>(unroll, a, grid, threads, lds_bytes, stream); break;
+    default:
+      if (c.p5 == 1) rc = launch_mfma_line(unroll, a, grid, threads, lds_bytes, stream);
+      else rc = launch_mfma_u<TLHIP_FMT_INT8_ROW, false>(unroll, a, grid, threads, lds_bytes, stream);
+      break;
   }
   if (rc) return rc;
   TLHIP_CHECK_HIP(hipGetLastError());
