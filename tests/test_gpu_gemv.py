@@ -254,6 +254,33 @@ def test_matrix_core_gemv_with_whole_line_weight_loads(be, n, k, m, waves, unrol
     assert np.array_equal(got, plain)
 
 
+@pytest.mark.parametrize("waves,unroll,kw,ks", [(8, 2, 8, 1), (8, 4, 4, 1), (8, 2, 1, 1), (4, 4, 2, 2), (8, 2, 8, 4), (16, 2, 16, 1),
+                                                (8, 2, 2, 8)])
+@pytest.mark.parametrize("n,k,m", [(515, 2048, 3), (100, 4096, 16), (4103, 2048, 8), (16, 4096, 1)])
+def test_whole_line_weight_loads_int4_with_k_splits(be, n, k, m, waves, unroll, kw, ks):
+    """The same load shape for int4 with group size 32 (a pair of iterations = 256 k), with
+    the K splits across waves and across workgroups the decode shapes use: the patches then
+    lie behind the parked tiles in LDS.  Bit-equal to the operand-layout loads."""
+    rng = np.random.default_rng(n + k + m + waves + unroll + kw + ks)
+    packed, scales, deq = make_weight("int4-grouped", n, k, 32, rng)
+    x = make_x(m, k, "f16", rng)
+    cfg = L.KernelConfig.of(1, waves, unroll, kw, ks, 0, 1)
+    base = L.KernelConfig.of(1, waves, unroll, kw, ks)
+    try:
+        plain = run_linear(be, "int4-grouped", packed, scales, n, k, 32, x, "f32", config=base)
+    except L.TlhipError:
+        with pytest.raises(L.TlhipError, match="config not applicable"):
+            run_linear(be, "int4-grouped", packed, scales, n, k, 32, x, "f32", config=cfg)
+        return
+    try:
+        got = run_linear(be, "int4-grouped", packed, scales, n, k, 32, x, "f32", config=cfg)
+    except L.TlhipError as e:   # the patches can push a launch that just fitted over the LDS budget
+        assert "do not fit LDS" in str(e)
+        return
+    assert rel_l2(got, O.linear(x.astype(np.float32), deq)) <= 2e-6
+    assert np.array_equal(got, plain)
+
+
 def test_whole_line_weight_loads_reject_what_they_do_not_cover(be):
     rng = np.random.default_rng(9)
     x = make_x(2, 192, "f16", rng)
@@ -262,11 +289,14 @@ def test_whole_line_weight_loads_reject_what_they_do_not_cover(be):
         run_linear(be, "int8-row", packed, scales, 64, 192, 0, x, "f32", config=L.KernelConfig.of(1, 4, 1, 1, 1, 0, 1))
     x = make_x(2, 256, "f16", rng)
     packed, scales, _ = make_weight("int8-row", 64, 256, 0, rng)
-    with pytest.raises(L.TlhipError, match="whole-line weight loads"):   # a K split across waves
-        run_linear(be, "int8-row", packed, scales, 64, 256, 0, x, "f32", config=L.KernelConfig.of(1, 4, 2, 2, 1, 0, 1))
-    packed4, scales4, _ = make_weight("int4-grouped", 64, 256, 32, rng)
-    with pytest.raises(L.TlhipError, match="whole-line weight loads"):   # another format
-        run_linear(be, "int4-grouped", packed4, scales4, 64, 256, 32, x, "f32", config=L.KernelConfig.of(1, 4, 2, 1, 1, 0, 1))
+    with pytest.raises(L.TlhipError, match="whole-line weight loads"):   # one iteration in flight
+        run_linear(be, "int8-row", packed, scales, 64, 256, 0, x, "f32", config=L.KernelConfig.of(1, 4, 1, 1, 1, 0, 1))
+    packed4, scales4, _ = make_weight("int4-grouped", 64, 256, 64, rng)
+    with pytest.raises(L.TlhipError, match="whole-line weight loads"):   # int4 with another group size
+        run_linear(be, "int4-grouped", packed4, scales4, 64, 256, 64, x, "f32", config=L.KernelConfig.of(1, 4, 2, 1, 1, 0, 1))
+    packed8, scales8, _ = make_weight("int8-grouped", 64, 256, 64, rng)
+    with pytest.raises(L.TlhipError, match="whole-line weight loads"):   # a format it is not built for
+        run_linear(be, "int8-grouped", packed8, scales8, 64, 256, 64, x, "f32", config=L.KernelConfig.of(1, 4, 2, 1, 1, 0, 1))
 
 
 def test_lm_head_sized_n(be):

@@ -144,6 +144,13 @@ tlhip_kernel_config_t default_config(const Problem& p) {
   // 13.4 / 15.1 us for the VALU kernel, whose dot products grow with M; at M = 2 the VALU
   // kernel is still ahead, 5.3 / 8.9 / 9.9 against 6.0 / 10.3 / 11.5 us)
   if (p.m >= 3 && p.m <= 16) {
+    // a long int8-row matrix (an LM head): the form with whole-line weight loads
+    if (p.format == TLHIP_FMT_INT8_ROW && p.n >= 32768)
+      for (int unroll : {4, 2}) {
+        tlhip_kernel_config_t c = mfma_cfg(8, unroll, 1, 1);
+        c.p5 = 1;
+        if (gemv_mfma_config_applicable(p, c, nullptr)) return c;
+      }
     // the fewest K slices across workgroups whose activations fit LDS (measured best)
     for (int ks = 1; ks <= 16; ks *= 2)
       for (int unroll : {2, 1}) {
@@ -202,6 +209,8 @@ std::vector<tlhip_kernel_config_t> candidates(const Problem& p) {
           for (int ks : {1, 2, 4, 8}) {
             if (kw > waves) continue;
             tlhip_kernel_config_t c = mfma_cfg(waves, unroll, kw, ks);
+            if (gemv_mfma_config_applicable(p, c, nullptr)) out.push_back(c);
+            c.p5 = 1;  // whole-line weight loads (int8 with one scale per row)
             if (gemv_mfma_config_applicable(p, c, nullptr)) out.push_back(c);
           }
   }

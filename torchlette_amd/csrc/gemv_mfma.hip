@@ -56,6 +56,7 @@ struct MfmaArgs {
   float scale_mul;
   int y_dtype;
   DevEpilogue epi;
+  int patch_unit;     // whole-line form: first 16-byte LDS unit of the waves' patches
 };
 
 template <int FMT>
@@ -87,7 +88,8 @@ __device__ __forceinline__ int x_unit(int t, int g, int m, int row_units) {
 }
 
 //
-// LINE (int8 with one scale per row, no K split, U even): a wave's weight loads take
+// LINE (U even; built for int8 with one scale per row and for int4 with group size 32):
+// a wave's weight loads take
 // whole 128-byte lines, 8 lanes to a row and 8 rows to an instruction, with the
 // nontemporal hint, instead of the operand layout's 64-byte pieces of 16 rows; a batch
 // then goes through a wave-private LDS patch (written as loaded, read back in the
@@ -97,7 +99,7 @@ __device__ __forceinline__ int x_unit(int t, int g, int m, int row_units) {
 // the second.
 template <int FMT, int U, bool WIDE, int MAXT, bool LINE = false>
 __global__ __launch_bounds__(MAXT) void gemv_mfma_kernel(const MfmaArgs a) {
-  static_assert(!LINE || (FMT == TLHIP_FMT_INT8_ROW && U % 2 == 0), "whole-line loads: int8-row, even U");
+  static_assert(!LINE || U % 2 == 0, "whole-line loads: an even number of iterations in flight");
   using Tr = MfmaTraits<FMT>;
   constexpr int STEPS = Tr::STEPS;
   constexpr bool GROUPED = (FMT != TLHIP_FMT_INT8_ROW);
@@ -208,7 +210,7 @@ __global__ __launch_bounds__(MAXT) void gemv_mfma_kernel(const MfmaArgs a) {
       // through the wave's patch: 16 rows x 8 chunks per pair, the chunk position
       // XOR-ed with the row so that the operand reads (16 rows, one chunk) spread
       // over the banks
-      u32x4* st = lds + (size_t)row_units * mrows + wave * (U / 2 * 128);
+      u32x4* st = lds + a.patch_unit + wave * (U / 2 * 128);
       const int r8 = lane >> 3, c8 = lane & 7;
 #pragma unroll
       for (int p2 = 0; p2 < U / 2; ++p2) {
@@ -509,6 +511,7 @@ static constexpr size_t kXLdsBudget = 160 * 1024;
 struct MfmaGeometry {
   int grid;
   size_t lds_bytes;
+  size_t patch_offset;  // bytes of activations and parked tiles in front of the patches
 };
 static bool mfma_geometry(int64_t n, int64_t k, int64_t m, int waves, int kw, int ks, size_t patch_bytes, MfmaGeometry* out) {
   const int threads = waves * 64;
@@ -532,6 +535,7 @@ static bool mfma_geometry(int64_t n, int64_t k, int64_t m, int waves, int kw, in
     if (lds * per_cu <= kXLdsBudget) {
       out->grid = (int)(sets * ks);
       out->lds_bytes = lds;
+      out->patch_offset = x_bytes + parked;
       return true;
     }
   }
@@ -557,8 +561,8 @@ bool gemv_mfma_config_applicable(const Problem& p, const tlhip_kernel_config_t& 
       "K slices must be a power of two (1..16) that divides K/128 (int4) or K/64 (int8)",
       "K slices need more partial-tile workspace or counters than the library holds",
       "iterations in flight must divide the 128-weight (int4) or 64-weight (int8) steps of a K slice",
-      "whole-line weight loads (p5 = 1) need int8 with one scale per row, K a multiple of 128, 2 or 4 iterations in "
-      "flight and no K split (p2 = 1, p3 <= 1)",
+      "whole-line weight loads (p5 = 1) need int8 with one scale per row (K % 128 == 0) or int4 with group size 32 "
+      "(K % 256 == 0), 2 or 4 iterations in flight and an even number of iterations per K slice",
   };
   auto fail = [&](int i) {
     if (why) *why = reasons[i];
@@ -579,9 +583,12 @@ bool gemv_mfma_config_applicable(const Problem& p, const tlhip_kernel_config_t& 
   const int ks = c.p3 < 1 ? 1 : c.p3;
   const int64_t iters = p.k / kper;
   if (ks > 16 || (ks & (ks - 1)) != 0 || iters % ks != 0) return fail(9);
-  if (c.p5 != 0 && !(c.p5 == 1 && p.format == TLHIP_FMT_INT8_ROW && p.k % 128 == 0 && (c.p1 == 2 || c.p1 == 4) &&
-                     kw == 1 && ks == 1))
-    return fail(12);
+  if (c.p5 != 0) {
+    // a pair of iterations = one 128-byte line per row: 128 k of int8, 256 k of int4
+    const bool fmt_ok = (p.format == TLHIP_FMT_INT8_ROW && p.k % 128 == 0) ||
+                        (p.format == TLHIP_FMT_INT4_GROUPED && p.group_size == 32 && p.k % 256 == 0);
+    if (!(c.p5 == 1 && fmt_ok && (c.p1 == 2 || c.p1 == 4) && (iters / ks) % 2 == 0)) return fail(12);
+  }
   MfmaGeometry geo;
   if (!mfma_geometry(p.n, p.k, p.m, c.p0, kw, ks, line_patch_bytes(c), &geo)) return fail(8);
   if ((iters / ks) % c.p1 != 0) return fail(11);
@@ -612,12 +619,13 @@ static int launch_mfma_u(int unroll, const MfmaArgs& a, int grid, int threads, s
   return TLHIP_OK;
 }
 
-// int8 with one scale per row, whole-line weight loads (2 or 4 iterations in flight).
+// The form with whole-line weight loads (2 or 4 iterations in flight).
+template <int FMT, bool WIDE>
 static int launch_mfma_line(int unroll, const MfmaArgs& a, int grid, int threads, size_t lds_bytes, hipStream_t stream) {
   const void* fn;
-  if (threads > 512) fn = (const void*)gemv_mfma_kernel<TLHIP_FMT_INT8_ROW, 2, false, 1024, true>;
-  else if (unroll == 2) fn = (const void*)gemv_mfma_kernel<TLHIP_FMT_INT8_ROW, 2, false, 512, true>;
-  else fn = (const void*)gemv_mfma_kernel<TLHIP_FMT_INT8_ROW, 4, false, 512, true>;
+  if (threads > 512) fn = (const void*)gemv_mfma_kernel<FMT, 2, WIDE, 1024, true>;
+  else if (unroll == 2) fn = (const void*)gemv_mfma_kernel<FMT, 2, WIDE, 512, true>;
+  else fn = (const void*)gemv_mfma_kernel<FMT, 4, WIDE, 512, true>;
   if (lds_bytes > 64 * 1024)
     TLHIP_CHECK_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
   void* args[] = {(void*)&a};
@@ -669,20 +677,23 @@ int launch_gemv_mfma(const Problem& p, const tlhip_kernel_config_t& c, hipStream
   if (!mfma_geometry(p.n, p.k, p.m, waves, a.kw, a.ks, line_patch_bytes(c), &geo))
     return set_error(TLHIP_ERR_INVALID, "gemv_mfma: launch geometry does not close");
   const size_t lds_bytes = geo.lds_bytes;
+  a.patch_unit = (int)(geo.patch_offset / 16);
   const int threads = waves * 64;
   const int grid = geo.grid;
   int rc;
   switch (p.format) {
     case TLHIP_FMT_INT4_GROUPED:
       // one scale per 16-byte chunk and 16-byte aligned scale vectors: wide scale loads
-      if (p.group_size == 32 && (unroll == 1 || p.k % 256 == 0))
+      if (c.p5 == 1)  // group size 32 and K % 256 == 0: the wide scale loads as well
+        rc = launch_mfma_line<TLHIP_FMT_INT4_GROUPED, true>(unroll, a, grid, threads, lds_bytes, stream);
+      else if (p.group_size == 32 && (unroll == 1 || p.k % 256 == 0))
         rc = launch_mfma_u<TLHIP_FMT_INT4_GROUPED, true>(unroll, a, grid, threads, lds_bytes, stream);
       else
         rc = launch_mfma_u<TLHIP_FMT_INT4_GROUPED, false>(unroll, a, grid, threads, lds_bytes, stream);
       break;
     case TLHIP_FMT_INT8_GROUPED: rc = launch_mfma_u<TLHIP_FMT_INT8_GROUPED, false>(unroll, a, grid, threads, lds_bytes, stream); break;
     default:
-      if (c.p5 == 1) rc = launch_mfma_line(unroll, a, grid, threads, lds_bytes, stream);
+      if (c.p5 == 1) rc = launch_mfma_line<TLHIP_FMT_INT8_ROW, false>(unroll, a, grid, threads, lds_bytes, stream);
       else rc = launch_mfma_u<TLHIP_FMT_INT8_ROW, false>(unroll, a, grid, threads, lds_bytes, stream);
       break;
   }
