@@ -308,8 +308,8 @@ typedef struct {
   int32_t p3; /* gemv: K-split waves (LDS combine) gemv_mfma: K slices across workgroups (0/1 = none)  tiled: waves M */
   int32_t p4; /* gemv: chunks in flight (2/4/8)    tiled: waves N */
   int32_t p5; /* gemv: 1 = dot products on the 4x4x4 matrix-core instruction (int4, f16 x, m <= 4, p0 = 16, p1 = 1)
-               * gemv_mfma: 1 = whole-line weight loads through a wave-private LDS patch (int8-row, K % 128 == 0,
-               * p1 = 2 or 4, no K split) */
+               * gemv_mfma: 1 = whole-line weight loads through a wave-private LDS patch (int8 with
+               * K % 128 == 0 or int4-g32 with K % 256 == 0; p1 = 2 or 4) */
   int32_t p6;
 } tlhip_kernel_config_t;
 

@@ -294,9 +294,29 @@ def test_whole_line_weight_loads_reject_what_they_do_not_cover(be):
     packed4, scales4, _ = make_weight("int4-grouped", 64, 256, 64, rng)
     with pytest.raises(L.TlhipError, match="whole-line weight loads"):   # int4 with another group size
         run_linear(be, "int4-grouped", packed4, scales4, 64, 256, 64, x, "f32", config=L.KernelConfig.of(1, 4, 2, 1, 1, 0, 1))
-    packed8, scales8, _ = make_weight("int8-grouped", 64, 256, 64, rng)
-    with pytest.raises(L.TlhipError, match="whole-line weight loads"):   # a format it is not built for
-        run_linear(be, "int8-grouped", packed8, scales8, 64, 256, 64, x, "f32", config=L.KernelConfig.of(1, 4, 2, 1, 1, 0, 1))
+    x = make_x(2, 192, "f16", rng)
+    packed8, scales8, _ = make_weight("int8-grouped", 64, 192, 64, rng)
+    with pytest.raises(L.TlhipError, match="whole-line weight loads"):   # K = 192 again, grouped
+        run_linear(be, "int8-grouped", packed8, scales8, 64, 192, 64, x, "f32", config=L.KernelConfig.of(1, 4, 1, 1, 1, 0, 1))
+
+
+@pytest.mark.parametrize("g", [64, 128])
+@pytest.mark.parametrize("waves,unroll,kw,ks", [(4, 4, 1, 1), (8, 2, 8, 1), (8, 2, 2, 2), (16, 2, 1, 1)])
+@pytest.mark.parametrize("n,k,m", [(515, 1024, 2), (4103, 2048, 8), (100, 512, 16)])
+def test_whole_line_weight_loads_int8_grouped(be, n, k, m, waves, unroll, kw, ks, g):
+    """The reference's own format (int8, f16 absmax per group of 64 or 128) through the same
+    load shape; bit-equal to the operand-layout loads."""
+    rng = np.random.default_rng(n + k + m + waves + unroll + kw + ks + g)
+    packed, scales, deq = make_weight("int8-grouped", n, k, g, rng)
+    x = make_x(m, k, "f16", rng)
+    try:
+        plain = run_linear(be, "int8-grouped", packed, scales, n, k, g, x, "f32", config=L.KernelConfig.of(1, waves, unroll, kw, ks))
+        got = run_linear(be, "int8-grouped", packed, scales, n, k, g, x, "f32", config=L.KernelConfig.of(1, waves, unroll, kw, ks, 0, 1))
+    except L.TlhipError as e:
+        assert "config not applicable" in str(e)
+        return
+    assert rel_l2(got, O.linear(x.astype(np.float32), deq)) <= 2e-6
+    assert np.array_equal(got, plain)
 
 
 def test_lm_head_sized_n(be):

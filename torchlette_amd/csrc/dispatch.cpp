@@ -144,8 +144,8 @@ tlhip_kernel_config_t default_config(const Problem& p) {
   // 13.4 / 15.1 us for the VALU kernel, whose dot products grow with M; at M = 2 the VALU
   // kernel is still ahead, 5.3 / 8.9 / 9.9 against 6.0 / 10.3 / 11.5 us)
   if (p.m >= 3 && p.m <= 16) {
-    // a long int8-row matrix (an LM head): the form with whole-line weight loads
-    if (p.format == TLHIP_FMT_INT8_ROW && p.n >= 32768)
+    // a long int8 matrix (an LM head): the form with whole-line weight loads
+    if ((p.format == TLHIP_FMT_INT8_ROW || p.format == TLHIP_FMT_INT8_GROUPED) && p.n >= 32768)
       for (int unroll : {4, 2}) {
         tlhip_kernel_config_t c = mfma_cfg(8, unroll, 1, 1);
         c.p5 = 1;
@@ -210,7 +210,7 @@ std::vector<tlhip_kernel_config_t> candidates(const Problem& p) {
             if (kw > waves) continue;
             tlhip_kernel_config_t c = mfma_cfg(waves, unroll, kw, ks);
             if (gemv_mfma_config_applicable(p, c, nullptr)) out.push_back(c);
-            c.p5 = 1;  // whole-line weight loads (int8 with one scale per row)
+            c.p5 = 1;  // whole-line weight loads
             if (gemv_mfma_config_applicable(p, c, nullptr)) out.push_back(c);
           }
   }

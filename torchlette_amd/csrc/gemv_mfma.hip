@@ -88,7 +88,7 @@ __device__ __forceinline__ int x_unit(int t, int g, int m, int row_units) {
 }
 
 //
-// LINE (U even; built for int8 with one scale per row and for int4 with group size 32):
+// LINE (U even; built for both int8 formats and for int4 with group size 32):
 // a wave's weight loads take
 // whole 128-byte lines, 8 lanes to a row and 8 rows to an instruction, with the
 // nontemporal hint, instead of the operand layout's 64-byte pieces of 16 rows; a batch
@@ -561,7 +561,7 @@ bool gemv_mfma_config_applicable(const Problem& p, const tlhip_kernel_config_t& 
       "K slices must be a power of two (1..16) that divides K/128 (int4) or K/64 (int8)",
       "K slices need more partial-tile workspace or counters than the library holds",
       "iterations in flight must divide the 128-weight (int4) or 64-weight (int8) steps of a K slice",
-      "whole-line weight loads (p5 = 1) need int8 with one scale per row (K % 128 == 0) or int4 with group size 32 "
+      "whole-line weight loads (p5 = 1) need int8 (K % 128 == 0) or int4 with group size 32 "
       "(K % 256 == 0), 2 or 4 iterations in flight and an even number of iterations per K slice",
   };
   auto fail = [&](int i) {
@@ -585,7 +585,7 @@ bool gemv_mfma_config_applicable(const Problem& p, const tlhip_kernel_config_t& 
   if (ks > 16 || (ks & (ks - 1)) != 0 || iters % ks != 0) return fail(9);
   if (c.p5 != 0) {
     // a pair of iterations = one 128-byte line per row: 128 k of int8, 256 k of int4
-    const bool fmt_ok = (p.format == TLHIP_FMT_INT8_ROW && p.k % 128 == 0) ||
+    const bool fmt_ok = ((p.format == TLHIP_FMT_INT8_ROW || p.format == TLHIP_FMT_INT8_GROUPED) && p.k % 128 == 0) ||
                         (p.format == TLHIP_FMT_INT4_GROUPED && p.group_size == 32 && p.k % 256 == 0);
     if (!(c.p5 == 1 && fmt_ok && (c.p1 == 2 || c.p1 == 4) && (iters / ks) % 2 == 0)) return fail(12);
   }
@@ -691,7 +691,10 @@ int launch_gemv_mfma(const Problem& p, const tlhip_kernel_config_t& c, hipStream
       else
         rc = launch_mfma_u<TLHIP_FMT_INT4_GROUPED, false>(unroll, a, grid, threads, lds_bytes, stream);
       break;
-    case TLHIP_FMT_INT8_GROUPED: rc = launch_mfma_u<TLHIP_FMT_INT8_GROUPED, false>(unroll, a, grid, threads, lds_bytes, stream); break;
+    case TLHIP_FMT_INT8_GROUPED:
+      if (c.p5 == 1) rc = launch_mfma_line<TLHIP_FMT_INT8_GROUPED, false>(unroll, a, grid, threads, lds_bytes, stream);
+      else rc = launch_mfma_u<TLHIP_FMT_INT8_GROUPED, false>(unroll, a, grid, threads, lds_bytes, stream);
+      break;
     default:
       if (c.p5 == 1) rc = launch_mfma_line<TLHIP_FMT_INT8_ROW, false>(unroll, a, grid, threads, lds_bytes, stream);
       else rc = launch_mfma_u<TLHIP_FMT_INT8_ROW, false>(unroll, a, grid, threads, lds_bytes, stream);
