@@ -391,6 +391,27 @@ def main() -> int:
                        "config": list(cfg.as_tuple())})
             out.destroy()
         details["lm_head_int8_row_256000x2304"] = lm
+        # the same kind of matrix in the reference's own format: 151936 x 2048 (a Qwen3 LM head),
+        # int8 with an f16 absmax per group of 64 (quantizeLinearWeight's default)
+        g64_pool, _ = B.weight_pool("int8-grouped", 151936, 2048, 64, "f32", pool_bytes=1.0e9)
+        lm64 = []
+        for m in (1, 8):
+            x, _ = B.activations(m, 2048)
+            out = be._alloc([m, 151936], "f32")
+            if not args.no_autotune:
+                B.tune(g64_pool, x, m, out, out_dtype="f32")
+            call = B.make_call(g64_pool, x, m, out, out_dtype="f32")
+            us = B.median_time(call, 30)
+            by = algorithmic_bytes("int8-grouped", 151936, 2048, 64, m, 2, 4)
+            cfg = be.selectedConfig(g64_pool[0], "f16", m, "f32")
+            lm64.append({"m": m, "us": round(us, 2), "gbps": round(by / us / 1e3, 1),
+                         "frac_of_peak": round(by / us / 1e3 / HBM_PEAK_GBPS, 4), "kernel": kernel_name_of(cfg),
+                         "config": list(cfg.as_tuple())})
+            out.destroy()
+        details["lm_head_int8_g64_151936x2048"] = lm64
+        for w in g64_pool[1:]:
+            w._base.destroy()
+            w.scales.destroy()
         # the LM head's consumer: device top-k of the 256 000 logits (k = 64), 512 B read back
         logits = be._alloc([256000], "f32")
         tv, ti = be._alloc([64], "f32"), be._alloc([64], "i32")
