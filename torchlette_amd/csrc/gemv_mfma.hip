@@ -172,7 +172,18 @@ __global__ __launch_bounds__(MAXT) void gemv_mfma_kernel(const MfmaArgs a) {
         else b.w[u] = wrow[(itb + u) * 4 + g];
       }
     }
-    if (WIDE) {
+    if (WIDE && FMT == TLHIP_FMT_INT8_GROUPED) {
+      // group size 64 = one scale per iteration: the U scales of a batch, contiguous and
+      // aligned (U divides the iterations of a row), as one 4- or 8-byte load
+      static_assert(!(WIDE && FMT == TLHIP_FMT_INT8_GROUPED) || U == 2 || U == 4, "wide int8 scales: U = 2 or 4");
+      if (U == 2) {
+        b.sv[0] = *(const uint32_t*)(srow + itb);
+      } else {
+        const uint2 v = *(const uint2*)(srow + itb);
+        b.sv[0] = v.x;
+        b.sv[1] = v.y;
+      }
+    } else if (WIDE) {
       if (U == 1) {
         const uint2 v = *(const uint2*)(srow + itb * 4);
         b.sv[0] = v.x;
@@ -265,7 +276,8 @@ __global__ __launch_bounds__(MAXT) void gemv_mfma_kernel(const MfmaArgs a) {
         float4_t d = {0.f, 0.f, 0.f, 0.f};
         d = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, xa0), bw[0], d, 0, 0, 0);
         d = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, xa1), bw[1], d, 0, 0, 0);
-        const float sc = valid ? half_bits_to_float(b.s[u][0]) : 0.f;
+        const uint16_t sbits = WIDE ? (uint16_t)((u & 1) ? (b.sv[u >> 1] >> 16) : (b.sv[u >> 1] & 0xffffu)) : b.s[u][0];
+        const float sc = valid ? half_bits_to_float(sbits) : 0.f;
 #pragma unroll
         for (int r = 0; r < 4; ++r) acc[r] = fmaf(sc, d[r], acc[r]);
       } else {
@@ -692,7 +704,10 @@ int launch_gemv_mfma(const Problem& p, const tlhip_kernel_config_t& c, hipStream
         rc = launch_mfma_u<TLHIP_FMT_INT4_GROUPED, false>(unroll, a, grid, threads, lds_bytes, stream);
       break;
     case TLHIP_FMT_INT8_GROUPED:
-      if (c.p5 == 1) rc = launch_mfma_line<TLHIP_FMT_INT8_GROUPED, false>(unroll, a, grid, threads, lds_bytes, stream);
+      if (c.p5 == 1 && p.group_size == 64)  // one scale per iteration: the wide scale loads as well
+        rc = launch_mfma_line<TLHIP_FMT_INT8_GROUPED, true>(unroll, a, grid, threads, lds_bytes, stream);
+      else if (c.p5 == 1)
+        rc = launch_mfma_line<TLHIP_FMT_INT8_GROUPED, false>(unroll, a, grid, threads, lds_bytes, stream);
       else rc = launch_mfma_u<TLHIP_FMT_INT8_GROUPED, false>(unroll, a, grid, threads, lds_bytes, stream);
       break;
     default:
