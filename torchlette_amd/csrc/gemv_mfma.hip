@@ -88,10 +88,9 @@ __device__ __forceinline__ int x_unit(int t, int g, int m, int row_units) {
 }
 
 //
-// LINE (U even; built for both int8 formats and for int4 with group size 32):
-// a wave's weight loads take
-// whole 128-byte lines, 8 lanes to a row and 8 rows to an instruction, with the
-// nontemporal hint, instead of the operand layout's 64-byte pieces of 16 rows; a batch
+// LINE (U even; built for both int8 formats and for int4 with group size 32): a wave's
+// weight loads take whole 128-byte lines, 8 lanes to a row and 8 rows to an instruction,
+// with the nontemporal hint, instead of the operand layout's 64-byte pieces of 16 rows; a batch
 // then goes through a wave-private LDS patch (written as loaded, read back in the
 // operand layout, no barrier: one wave's LDS accesses stay in order) before it is
 // consumed exactly as before.  A read-only kernel streams the LM head's 590 MB in
