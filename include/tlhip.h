@@ -186,6 +186,21 @@ int tlhip_dequant(const tlhip_qweight_t* w, float* out, tlhip_stream_t stream);
 int tlhip_gemv(const tlhip_qweight_t* w, const void* x, int x_dtype, int64_t m, void* y,
                int y_dtype, float alpha, const tlhip_epilogue_t* epilogue, tlhip_stream_t stream);
 
+/* tlhip_gemv for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  It has no
+ * counterpart in the reference.  Same arguments, kernels and results as tlhip_gemv,
+ * but where tlhip_gemv combines K slices of different workgroups through a workspace
+ * the library allocates on a stream's first use, this entry point uses a fixed
+ * device array inside the library (4 MiB of partial tiles + 4096 counters per GPU,
+ * resolved at tlhip_init) and calls no hipMalloc / hipFree.  A problem whose
+ * configuration needs more (output rows / 16 * K slices * 1 KiB above 4 MiB, or more
+ * than 65536 output rows with K slices) fails with TLHIP_ERR_INVALID.  All calls on a
+ * GPU share the array: calls that overlap on one GPU (two streams, or a replaying
+ * graph next to eager calls) race. */
+int tlhip_gemv_noalloc(const tlhip_qweight_t* w, const void* x, int x_dtype, int64_t m, void* y,
+                       int y_dtype, float alpha, const tlhip_epilogue_t* epilogue,
+                       tlhip_stream_t stream);
+
 /* Up to 4 decode GEMVs of one shape class in ONE launch (q/k/v or gate/up of a
  * decode step: the frontend issues them back to back on the same activations,
  * src/frontend/torchlette.ts:878-894 once per Linear, and each is too small to

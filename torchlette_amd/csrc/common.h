@@ -49,6 +49,17 @@ struct DevPrologue {
   const void* operand;
 };
 
+// Caller-provided device scratch for the kernels that combine partial results of
+// several workgroups (instead of the library's per-stream workspace): `tile_floats`
+// floats of partial tiles and `ncounters` arrival counters that are zero when the
+// launch starts.
+struct SplitScratch {
+  float* tiles;
+  int* counters;
+  size_t tile_floats;
+  int ncounters;
+};
+
 // Validated problem description handed to the launchers.
 struct Problem {
   int format;
@@ -63,6 +74,7 @@ struct Problem {
   float alpha;
   DevEpilogue epi;
   DevPrologue pro;  // kind NONE unless the entry point sets it
+  const SplitScratch* scratch;  // null: the library's per-stream workspace
 };
 
 // Validation shared by every compute entry point.  Fills `p` on success.
@@ -94,6 +106,23 @@ int launch_gemm_direct(const Problem& p, const tlhip_kernel_config_t& c, hipStre
 constexpr size_t kSplitWorkspaceFloats = 4u << 20;  // 16 MiB
 constexpr int kSplitCounters = 1 << 16;
 int split_workspace(hipStream_t stream, float** workspace, int** counters);
+// The scratch a launch of `p` combines its K slices through: the caller's, or the
+// stream's own (created on first use).
+int problem_scratch(const Problem& p, hipStream_t stream, float** workspace, int** counters);
+inline size_t scratch_tile_floats(const Problem& p) { return p.scratch ? p.scratch->tile_floats : kSplitWorkspaceFloats; }
+inline int scratch_counters(const Problem& p) { return p.scratch ? p.scratch->ncounters : kSplitCounters; }
+
+// Kernel choice of the decode entry points (dispatch.cpp): the tuned winner for the
+// problem if one is cached and applicable, else the heuristic default; never a
+// prefill GEMM configuration.
+tlhip_kernel_config_t select_gemv_config(const Problem& p);
+int run_kernel_config(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t stream);
+// K slices across workgroups of a configuration (1 = it needs no scratch).
+int config_k_slices(const tlhip_kernel_config_t& c);
+
+// Set-up of the entry point that allocates nothing (noalloc.hip): resolves the device
+// address of its static scratch array for the current device.
+int noalloc_setup(int device_index);
 
 // Counters.
 void count_gemv_dispatch();

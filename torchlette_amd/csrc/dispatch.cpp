@@ -332,6 +332,19 @@ int autotune_problem(const Problem& p, double* best_us_out) {
 
 }  // namespace
 
+tlhip_kernel_config_t select_gemv_config(const Problem& p) {
+  tlhip_kernel_config_t c = select_config(p);
+  if (c.variant == VARIANT_TILED || c.variant == VARIANT_TILED_DIRECT) c = default_config(p);
+  return c;
+}
+
+int run_kernel_config(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t stream) { return run_config(p, c, stream); }
+
+int config_k_slices(const tlhip_kernel_config_t& c) {
+  if (c.variant == VARIANT_GEMV_MFMA || c.variant == VARIANT_GEMV_XREG) return c.p3 < 1 ? 1 : c.p3;
+  return 1;
+}
+
 int validate_weight(const tlhip_qweight_t* w, const char* who) {
   if (!w) return set_error(TLHIP_ERR_INVALID, "%s: missing packing/scales on B operand", who);
   if (w->format != TLHIP_FMT_INT8_GROUPED && w->format != TLHIP_FMT_INT8_ROW &&
@@ -382,6 +395,7 @@ int make_problem(const tlhip_qweight_t* w, const void* x, int x_dtype, int64_t m
   p->alpha = alpha;
   memset(&p->epi, 0, sizeof p->epi);
   memset(&p->pro, 0, sizeof p->pro);
+  p->scratch = nullptr;
   if (epilogue) {
     if (epilogue->n_ops < 0 || epilogue->n_ops > TLHIP_MAX_EPILOGUE_OPS)
       return set_error(TLHIP_ERR_INVALID, "%s: epilogue has %d ops (max %d)", who, epilogue->n_ops,
@@ -431,9 +445,7 @@ int tlhip_gemv(const tlhip_qweight_t* w, const void* x, int x_dtype, int64_t m, 
   int rc = make_problem(w, x, x_dtype, m, y, y_dtype, alpha, epilogue, &p, "gemv");
   if (rc) return rc;
   if (m > 16) return set_error(TLHIP_ERR_INVALID, "gemv: M=%lld above 16; use tlhip_gemm_prefill", (long long)m);
-  tlhip_kernel_config_t c = select_config(p);
-  if (c.variant == VARIANT_TILED || c.variant == VARIANT_TILED_DIRECT) c = default_config(p);
-  return run_config(p, c, resolve_stream(stream));
+  return run_config(p, select_gemv_config(p), resolve_stream(stream));
 }
 
 int tlhip_gemv_grouped(const tlhip_gemv_problem_t* problems, int count, int x_dtype, int y_dtype, float alpha,

@@ -605,7 +605,7 @@ bool gemv_mfma_config_applicable(const Problem& p, const tlhip_kernel_config_t& 
   if ((iters / ks) % c.p1 != 0) return fail(11);
   if (ks > 1) {
     const int64_t nblocks = (p.n + 15) / 16;
-    if (nblocks > kSplitCounters || (size_t)nblocks * ks * 256 > kSplitWorkspaceFloats) return fail(10);
+    if (nblocks > scratch_counters(p) || (size_t)nblocks * ks * 256 > scratch_tile_floats(p)) return fail(10);
   }
   return true;
 }
@@ -675,7 +675,7 @@ int launch_gemv_mfma(const Problem& p, const tlhip_kernel_config_t& c, hipStream
   a.workspace = nullptr;
   a.counters = nullptr;
   if (a.ks > 1) {
-    const int rc = split_workspace(stream, &a.workspace, &a.counters);
+    const int rc = problem_scratch(p, stream, &a.workspace, &a.counters);
     if (rc) return rc;
   }
   a.nblocks = (int)((p.n + 15) / 16);

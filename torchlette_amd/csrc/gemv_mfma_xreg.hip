@@ -290,7 +290,7 @@ bool gemv_xreg_config_applicable(const Problem& p, const tlhip_kernel_config_t& 
   if (!xreg_geometry(p, c.p0, c.p1, per_cu, ks, &geo, &w)) return fail(w);
   if (ks > 1) {
     const int64_t nblocks = (p.n + 15) / 16;
-    if (nblocks > kSplitCounters || (size_t)nblocks * ks * 256 > kSplitWorkspaceFloats) return fail(8);
+    if (nblocks > scratch_counters(p) || (size_t)nblocks * ks * 256 > scratch_tile_floats(p)) return fail(8);
   }
   return true;
 }
@@ -313,7 +313,7 @@ int launch_gemv_xreg(const Problem& p, const tlhip_kernel_config_t& c, hipStream
   a.workspace = nullptr;
   a.counters = nullptr;
   if (ks > 1) {
-    const int rc = split_workspace(stream, &a.workspace, &a.counters);
+    const int rc = problem_scratch(p, stream, &a.workspace, &a.counters);
     if (rc) return rc;
   }
   a.n = p.n;

@@ -94,6 +94,15 @@ int split_workspace(hipStream_t stream, float** workspace, int** counters) {
   return TLHIP_OK;
 }
 
+int problem_scratch(const Problem& p, hipStream_t stream, float** workspace, int** counters) {
+  if (p.scratch) {
+    *workspace = p.scratch->tiles;
+    *counters = p.scratch->counters;
+    return TLHIP_OK;
+  }
+  return split_workspace(stream, workspace, counters);
+}
+
 int device_cu_count() { return g_init ? g_props.multiProcessorCount : 0; }
 
 void count_gemv_dispatch() { g_gemv_dispatches++; }
@@ -133,6 +142,14 @@ int tlhip_init(int device_index) {
   TLHIP_CHECK_HIP(hipStreamCreateWithFlags(&g_stream, hipStreamNonBlocking));
   g_device = device_index;
   g_init = true;
+  const int rc = noalloc_setup(device_index);
+  if (rc) {
+    (void)hipStreamDestroy(g_stream);
+    g_stream = nullptr;
+    g_init = false;
+    g_device = -1;
+    return rc;
+  }
   clear_error();
   return TLHIP_OK;
 }
