@@ -138,23 +138,26 @@ def test_gemm_against_gemv_on_the_same_rows(be):
     assert rel_l2(full[:16], part) <= 5e-4
 
 
+@pytest.mark.parametrize("act", ["silu", "gelu"])
 @pytest.mark.parametrize("m", [512, 2048])
-def test_config4_full_size(be, m):
-    """M x 4096 x 12288 int4-g32, bias + silu, f16 out: a row sample against the
-    sequential-k oracle, the whole output against numpy float64 (same sums in a
-    different order), and linearity in the activations."""
+def test_config4_full_size(be, m, act):
+    """M x 4096 x 12288 int4-g32, bias + silu or gelu(tanh), f16 out: a row sample
+    against the sequential-k oracle, the whole output against numpy float64 (same
+    sums in a different order), and linearity in the activations."""
     rng = np.random.default_rng(m)
     n, k = 12288, 4096
     packed, scales, deq = make_weight("int4-grouped", n, k, 32, rng)
     x = make_x(m, k, "f16", rng, std=0.5)
     bias = f16_round(rng.standard_normal(n) * 0.1)
-    got = run(be, "int4-grouped", packed, scales, n, k, 32, x, "f16", bias=bias, act="silu")
+    got = run(be, "int4-grouped", packed, scales, n, k, 32, x, "f16", bias=bias, act=act)
     rows = rng.choice(m, 32, replace=False)
-    want_rows = O.linear(x[rows].astype(np.float32), deq, bias.astype(np.float32), "silu", threads=8)
+    want_rows = O.linear(x[rows].astype(np.float32), deq, bias.astype(np.float32), act, threads=8)
     assert rel_l2(got[rows], want_rows) <= REL_L2_TOL, rel_l2(got[rows], want_rows)
     pre = O.np_matmul_nt(x.astype(np.float32), deq)
-    want = O.np_unary("silu", (pre.astype(np.float64) + bias.astype(np.float64)).astype(np.float32))
+    want = O.np_unary(act, (pre.astype(np.float64) + bias.astype(np.float64)).astype(np.float32))
     assert rel_l2(got, want) <= REL_L2_TOL, rel_l2(got, want)
+    if act != "silu":
+        return
     # no epilogue, f32 out: y(2*x) == 2*y(x) exactly (scaling by 2 is exact in f16 and f32)
     y1 = run(be, "int4-grouped", packed, scales, n, k, 32, x, "f32")
     y2 = run(be, "int4-grouped", packed, scales, n, k, 32, f16_round(2 * x.astype(np.float32)), "f32")
