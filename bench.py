@@ -22,6 +22,19 @@ HBM before the timed region.  The printed JSON line carries
                graph), the LM head, the prefill GEMM (TFLOP/s) and config 1
 
 Only one GPU is used; --gpus above 1 exits with a message.
+
+The rocprofv3 summaries under profiles/ are made by this file as well (no GPU
+needed for these three; each prints the table it writes):
+
+    python bench.py --summarise-trace DIR OUT.txt "COMMAND" [run]
+        DIR holds the *_kernel_trace.csv / *_kernel_stats.csv of
+        `rocprofv3 --kernel-trace --stats --output-format csv -d DIR -- python3 bench.py ...`
+    python bench.py --summarise-traffic FETCH.csv WRITE.csv PROBE.log OUT.txt OUT.json
+        the counter_collection.csv files of two `rocprofv3 --pmc FETCH_SIZE` /
+        `--pmc WRITE_SIZE` runs of `python3 bench.py --traffic-probe` and the
+        stdout of one of them; OUT.json is what --traffic-file reads
+    python bench.py --summarise-prefill-counters COUNTERS.csv PROBE.log OUT.txt "COMMAND"
+        one `rocprofv3 --pmc ... -- python3 bench.py --prefill-probe` run
 """
 from __future__ import annotations
 
@@ -152,51 +165,19 @@ class Bench:
         return self.median_time(call, 100)
 
     def tune(self, pool, x, m: int, out, out_dtype: str = "f16", epilogue=None):
-        """Pick the fastest candidate configuration with the weights ROTATING
-        through the pool (the library's own tlhip_autotune times one buffer,
-        which a 256 MB last-level cache keeps resident), and seed the library's
-        per-shape cache with the winner."""
+        """The library's tuner (tlhip_autotune_pool) over this pool: every candidate is
+        timed in batches of back-to-back launches with the weights ROTATING through the
+        pool, the three fastest once more, and the winner lands in the library's
+        per-shape cache.  Returns its time per launch in microseconds."""
         L, be = self.L, self.be
-        qws = [be._qweight(w, False) for w in pool]
+        qws = (L.QWeight * len(pool))(*[be._qweight(w, False) for w in pool])
         xd = L.F16 if x.dtype == "f16" else L.F32
         yd = L.F16 if out_dtype == "f16" else L.F32
         ep = C.byref(epilogue) if epilogue is not None else None
-        fn = L.load().tlhip_matmul_quantized_config
-        best, best_cfg = None, None
-        # untimed launches of the current choice first, so that the first candidates are
-        # not timed at the lower clock the GPU starts from after a pause
-        warm = self.make_call(pool, x, m, out, epilogue=epilogue, out_dtype=out_dtype)
-        spent = 0.0
-        while spent < self.warm_ms * 1e3:
-            spent += self.time_region(warm, 8) * 8
-        timed = []
-        reps = 8 if m > 16 else 24
-
-        def caller(cfg):
-            state = {"i": 0}
-
-            def call():
-                qw = qws[state["i"] % len(qws)]
-                state["i"] += 1
-                return fn(C.byref(qw), x.ptr, xd, m, out.ptr, yd, 1.0, ep, C.byref(cfg), None)
-            return call
-        for cfg in be.candidates(pool[0], x.dtype, m, out_dtype):
-            call = caller(cfg)
-            if call() != 0:
-                continue
-            self.be.synchronize()
-            timed.append((min(self.time_region(call, reps) for _ in range(3)), cfg))
-        # the three fastest once more, longer: candidates within a few per cent of each other
-        # would otherwise change places from run to run
-        timed.sort(key=lambda t: t[0])
-        for _, cfg in timed[:3]:
-            call = caller(cfg)
-            us = min(self.time_region(call, 3 * reps) for _ in range(3))
-            if best is None or us < best:
-                best, best_cfg = us, cfg
-        if best_cfg is not None:
-            be.seedPerShapeMatmulChoice(pool[0], x.dtype, m, out_dtype, best_cfg)
-        return best
+        opts = L.AutotuneOptions(0, 3, 3, 0, self.warm_ms, 0)
+        best = C.c_double()
+        L.call("tlhip_autotune_pool", qws, len(pool), x.ptr, xd, m, out.ptr, yd, ep, C.byref(opts), None, C.byref(best))
+        return best.value
 
 
 def kernel_name_of(cfg) -> str:
@@ -219,7 +200,174 @@ def cpu_step(cases, host_weights, host_x, threads: int) -> float:
     return time.perf_counter() - t0
 
 
+# ---------------------------------------------------------------- profile summaries
+def _short_kernel_name(n: str) -> str:
+    import re
+    m = re.match(r"_ZN5tlhip12_GLOBAL__N_111gemv_kernelILi(\d)E(DF16_|f)Li(\d)ELi(\d)ELi(\d)ELb(\d)E", n)
+    if m:
+        return (f"gemv_kernel<fmt={m.group(1)}, x={'f16' if m.group(2) == 'DF16_' else 'f32'}, rows={m.group(3)}, "
+                f"R={m.group(4)}, U={m.group(5)}{', 4x4x4 mfma' if m.group(6) == '1' else ''}>")
+    n = re.sub(r"tlhip::\(anonymous namespace\)::", "", n)
+    n = re.sub(r"\(anonymous namespace\)::", "", n)
+    n = re.sub(r"\(tlhip::.*", "", n)
+    n = re.sub(r"void ", "", n)
+    return n[:70]
+
+
+def summarise_trace(d: str, out: str, cmd: str, want_run: bool) -> int:
+    """rocprofv3 --kernel-trace --stats CSVs -> the short table kept under profiles/."""
+    import collections
+    import csv
+    import glob
+    import statistics
+
+    def find(pat):
+        r = glob.glob(os.path.join(d, "**", pat), recursive=True)
+        return r[0] if r else None
+    lines = [f"command: {cmd}", f"summary: python bench.py --summarise-trace <its output directory> <this file> \"<command>\"{' run' if want_run else ''}", ""]
+    st = find("*kernel_stats.csv")
+    if st:
+        lines.append("rocprofv3 --stats (per kernel name, all shapes of that name pooled):")
+        lines.append(f"{'kernel':70s} {'calls':>7s} {'total_us':>11s} {'avg_us':>9s} {'min_us':>8s} {'max_us':>9s} {'%':>6s}")
+        for i, r in enumerate(csv.DictReader(open(st))):
+            if i >= 14:
+                break
+            lines.append(f"{_short_kernel_name(r['Name']):70s} {int(r['Calls']):7d} {float(r['TotalDurationNs']) / 1e3:11.1f} "
+                         f"{float(r['AverageNs']) / 1e3:9.2f} {float(r['MinNs']) / 1e3:8.2f} {float(r['MaxNs']) / 1e3:9.2f} "
+                         f"{float(r['Percentage']):6.2f}")
+    tr = find("*kernel_trace.csv")
+    if tr:
+        groups = collections.defaultdict(list)
+        rows = list(csv.DictReader(open(tr)))
+        for r in rows:
+            key = (_short_kernel_name(r["Kernel_Name"]), int(r["Grid_Size_X"]) // max(1, int(r["Workgroup_Size_X"])),
+                   int(r["Workgroup_Size_X"]), int(r["LDS_Block_Size"]))
+            groups[key].append((int(r["End_Timestamp"]) - int(r["Start_Timestamp"])) / 1e3)
+        lines += ["", "kernel trace, dispatches grouped by (kernel, workgroups, threads, LDS bytes) = one shape each:",
+                  f"{'kernel':70s} {'wgs':>6s} {'thr':>5s} {'lds':>7s} {'calls':>6s} {'avg_us':>9s} {'med_us':>9s} {'min_us':>8s}"]
+        for (n, g, t, l), v in sorted(groups.items(), key=lambda kv: -sum(kv[1]))[:40]:
+            lines.append(f"{n:70s} {g:6d} {t:5d} {l:7d} {len(v):6d} {sum(v) / len(v):9.2f} {statistics.median(v):9.2f} {min(v):8.2f}")
+        if want_run:
+            rows.sort(key=lambda r: int(r["Start_Timestamp"]))
+            best, i = (0, 0, None), 0
+            while i < len(rows):
+                j = i
+                while j < len(rows) and rows[j]["Kernel_Name"] == rows[i]["Kernel_Name"]:
+                    j += 1
+                if j - i > best[0]:
+                    best = (j - i, i, rows[i]["Kernel_Name"])
+                i = j
+            n, i0, name = best
+            v = [(int(r["End_Timestamp"]) - int(r["Start_Timestamp"])) / 1e3 for r in rows[i0:i0 + n]]
+            lines += ["", "longest run of consecutive launches of one kernel (bench.py's dominant-kernel timing loop, one shape):",
+                      f"{_short_kernel_name(name)}: {n} launches, avg {sum(v) / n:.2f} us, median {statistics.median(v):.2f} us, "
+                      f"min {min(v):.2f} us"]
+    open(out, "w").write("\n".join(lines) + "\n")
+    print("\n".join(lines))
+    return 0
+
+
+def _probe_record(path: str, key: str):
+    for line in open(path):
+        line = line.strip()
+        if line.startswith("{") and key in line:
+            return json.loads(line)[key]
+    raise SystemExit(f"{path}: no {key} record")
+
+
+def summarise_traffic(fetch_csv: str, write_csv: str, probe_file: str, out_txt: str, out_json: str) -> int:
+    """FETCH_SIZE / WRITE_SIZE counter runs of --traffic-probe -> HBM bytes per launch of
+    each call of the step, each counter scaled by what it reads for the 256 MiB
+    device-to-device copies of the same run."""
+    import csv
+    probe = _probe_record(probe_file, "traffic_probe")
+    cases, nl = probe["cases"], probe["launches"]
+    res, lines = {}, [
+        "commands: rocprofv3 --pmc FETCH_SIZE --output-format csv -d <dir> -o r -- python3 bench.py --traffic-probe",
+        "          rocprofv3 --pmc WRITE_SIZE --output-format csv -d <dir> -o r -- python3 bench.py --traffic-probe",
+        "summary:  python bench.py --summarise-traffic <fetch>/r_counter_collection.csv <write>/r_counter_collection.csv "
+        "<stdout of one run> <this file> <the .json beside it>", ""]
+    for path, counter in ((fetch_csv, "FETCH_SIZE"), (write_csv, "WRITE_SIZE")):
+        rows = [r for r in csv.DictReader(open(path)) if r["Counter_Name"] == counter]
+        rows.sort(key=lambda r: int(r["Start_Timestamp"]))
+        gemv = [float(r["Counter_Value"]) for r in rows if "gemv" in r["Kernel_Name"]][-nl * len(cases):]
+        copy = [float(r["Counter_Value"]) for r in rows if "copyBuffer" in r["Kernel_Name"]][-probe["copies"]:]
+        c_avg = sum(copy) / len(copy)
+        scale = (probe["copy_bytes"] / 1024.0) / c_avg  # known KiB per copy / counted KiB per copy
+        lines.append(f"{counter}: copy kernel (256 MiB each way) avg {c_avg:.1f} KiB/dispatch -> scale {scale:.4f}")
+        for i, c in enumerate(cases):
+            v = gemv[i * nl:(i + 1) * nl]
+            k_avg = sum(v) / len(v)
+            res.setdefault(i, {})[counter] = (k_avg, scale, k_avg * scale * 1024)
+            lines.append(f"  M={c['m']} N={c['n']} K={c['k']} {c['kernel']} config {c['config'][:6]}: avg {k_avg:.1f} KiB/dispatch "
+                         f"over {len(v)} dispatches -> {k_avg * scale * 1024:.0f} bytes")
+    out = {}
+    for i, c in enumerate(cases):
+        f, w = res[i]["FETCH_SIZE"], res[i]["WRITE_SIZE"]
+        traffic = f[2] + w[2]
+        lines.append(f"M={c['m']} N={c['n']} K={c['k']}: traffic (fetch + write, scaled) = {traffic:.0f} bytes per launch; "
+                     f"algorithmic bytes = {c['algorithmic_bytes']}; ratio {traffic / c['algorithmic_bytes']:.3f}")
+        out[f'{c["m"]}_{c["n"]}_{c["k"]}_int4-g32'] = {
+            "config": c["config"], "kernel": c["kernel"], "traffic_bytes": round(traffic), "fetch_bytes": round(f[2]),
+            "write_bytes": round(w[2]), "fetch_scale": round(f[1], 4), "write_scale": round(w[1], 4),
+            "algorithmic_bytes": c["algorithmic_bytes"]}
+    open(out_txt, "w").write("\n".join(lines) + "\n")
+    json.dump(out, open(out_json, "w"), indent=1)
+    print("\n".join(lines))
+    return 0
+
+
+def summarise_prefill_counters(csvf: str, logf: str, out: str, cmd: str) -> int:
+    """One --pmc run of --prefill-probe -> matrix-pipe utilisation and VALU per MFMA."""
+    import collections
+    import csv
+    probe = _probe_record(logf, "prefill_probe")
+    rows = [r for r in csv.DictReader(open(csvf)) if "gemm_direct" in r["Kernel_Name"] or "gemm_prefill" in r["Kernel_Name"]]
+    by_disp = collections.OrderedDict()
+    for r in rows:
+        by_disp.setdefault(int(r["Dispatch_Id"]), {"name": r["Kernel_Name"], "t0": int(r["Start_Timestamp"]),
+                                                   "t1": int(r["End_Timestamp"])})[r["Counter_Name"]] = float(r["Counter_Value"])
+    disp, nl = list(by_disp.values()), probe["launches"]
+    lines = [f"command: {cmd}", "summary: python bench.py --summarise-prefill-counters <dir>/r_counter_collection.csv <stdout of the run> "
+             "<this file> \"<command>\"", "",
+             "one counter run; per case the mean over its 5 launches (durations under the profiler are 5-20 % longer than",
+             "bench.py's own).  An MFMA 32x32x16 f16 occupies its SIMD's matrix pipe for 32 cycles, so",
+             "SQ_VALU_MFMA_BUSY_CYCLES = 32 x MFMA count, and the pipe's utilisation at core clock f is",
+             "busy / (1024 SIMDs x f x duration).  f: 2.4 GHz is the clock the 2.5 PFLOP/s peak is quoted at; rocm-smi",
+             "--showclocks, sampled while the M = 8192 case ran in a loop for 4 s, read sclk = 1.80-1.81 GHz.", ""]
+    for i, c in enumerate(probe["cases"]):
+        ds = disp[i * nl:(i + 1) * nl]
+        if len(ds) < nl:
+            break
+
+        def mean(k):
+            return sum(d[k] for d in ds) / len(ds)
+        dur_us = sum(d["t1"] - d["t0"] for d in ds) / len(ds) / 1e3
+        mf, nm = mean("SQ_VALU_MFMA_BUSY_CYCLES"), c["flops"] / 32768
+        name = ds[0]["name"].replace("void tlhip::(anonymous namespace)::", "").split("(")[0]
+        lines += [f"M={c['m']} N={c['n']} K={c['k']} config {c['config'][:6]} {name}",
+                  f"  duration under the profiler {dur_us:9.1f} us -> {c['flops'] / dur_us / 1e6:7.1f} TFLOP/s = "
+                  f"{c['flops'] / dur_us / 1e6 / F16_MFMA_PEAK_TFLOPS:.3f} of {F16_MFMA_PEAK_TFLOPS:.0f}",
+                  f"  SQ_VALU_MFMA_BUSY_CYCLES   {mf:12.0f}  = 32 x {mf / 32:.0f} (MFMAs the problem needs: {nm:.0f})",
+                  f"  matrix pipe utilisation    {mf / (1024 * 2.4e3 * dur_us):.3f} at 2.4 GHz, {mf / (1024 * 1.8e3 * dur_us):.3f} at 1.8 GHz",
+                  f"  SQ_INSTS_VALU {mean('SQ_INSTS_VALU'):.0f} (MFMA included) -> {(mean('SQ_INSTS_VALU') - nm) / nm:.2f} other VALU "
+                  "instructions per MFMA",
+                  f"  SQ_WAVE_CYCLES {mean('SQ_WAVE_CYCLES'):.0f}  SQ_WAIT_INST_ANY {mean('SQ_WAIT_INST_ANY'):.0f} "
+                  f"({mean('SQ_WAIT_INST_ANY') / mean('SQ_WAVE_CYCLES'):.2f} of the wave cycles)  SQ_ACTIVE_INST_LDS "
+                  f"{mean('SQ_ACTIVE_INST_LDS'):.0f}  SQ_BUSY_CYCLES {mean('SQ_BUSY_CYCLES'):.0f}  GRBM_GUI_ACTIVE "
+                  f"{mean('GRBM_GUI_ACTIVE'):.0f}", ""]
+    open(out, "w").write("\n".join(lines) + "\n")
+    print("\n".join(lines))
+    return 0
+
+
 def main() -> int:
+    if len(sys.argv) > 1 and sys.argv[1] == "--summarise-trace":
+        return summarise_trace(sys.argv[2], sys.argv[3], sys.argv[4], len(sys.argv) > 5 and sys.argv[5] == "run")
+    if len(sys.argv) > 1 and sys.argv[1] == "--summarise-traffic":
+        return summarise_traffic(*sys.argv[2:7])
+    if len(sys.argv) > 1 and sys.argv[1] == "--summarise-prefill-counters":
+        return summarise_prefill_counters(*sys.argv[2:6])
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
@@ -242,7 +390,7 @@ def main() -> int:
                          "three device-to-device copies of 256 MiB (the known size the counters are scaled by), and exit")
     ap.add_argument("--prefill-probe", action="store_true",
                     help="counter runs: only launch the prefill GEMM (M = 512, 2048, 8192; bias + silu), 5 launches each")
-    ap.add_argument("--traffic-file", default=os.path.join(ROOT, "torchlette_amd", "tuning", "mi355x_traffic.json"),
+    ap.add_argument("--traffic-file", default=os.path.join(ROOT, "profiles", "decode_step_qwen3_8b_int4_hbm_traffic.json"),
                     help="measured HBM bytes per launch (from the counter runs), keyed by call; fills roofline.traffic")
     ap.add_argument("--tuning-cache", default=os.path.join(ROOT, "torchlette_amd", "tuning", "mi355x.json"),
                     help="JSON tuning cache to import before the run and to write after --autotune")
@@ -326,14 +474,38 @@ def main() -> int:
         for c in cases:
             c["call"]()
 
-    for _ in range(args.warmup):
-        step()
-    be.synchronize()
+    def timed_step():
+        """One measurement of the step: `--warmup` untimed steps, then the median of
+        five batches of exactly `--steps` steps between events on the launch stream."""
+        for _ in range(args.warmup):
+            step()
+        be.synchronize()
+        return float(np.median([B.time_region(step, args.steps) for _ in range(5)]))
+
+    # `warm_ms` of untimed steps first, like every other section: after the host-side
+    # set-up above the GPU starts from a low clock, and a 20-step batch is over in 3 ms
+    spent = 0.0
+    while spent < B.warm_ms * 1e3:
+        spent += B.time_region(step, 10) * 10
     t0 = time.perf_counter()
-    step_us = B.time_region(step, args.steps)
+    step_us = timed_step()
     be.synchronize()
     wall_s = time.perf_counter() - t0
     value = step_bytes / step_us / 1e3  # GB/s
+
+    # the same step on the heuristic defaults (what a shape without a tuning entry and
+    # without a tuned neighbour of its class gets): the gap to the tuned figure, recorded
+    default_step = None
+    if tuning_source != "heuristic defaults":
+        saved = T.exportTuningCache()
+        T.clearTuningCache()
+        default_configs = [list(be.selectedConfig(pools[(c["n"], c["k"])][0], "f16", c["m"], "f16").as_tuple()) for c in cases]
+        default_us = timed_step()
+        T.importTuningCache(saved)
+        default_step = {"us_per_step": round(default_us, 2), "gbps": round(step_bytes / default_us / 1e3, 1),
+                        "calls_with_another_config": sum(1 for c, d in zip(cases, default_configs) if d != c["config"])}
+        step()  # back on the tuned choices
+        be.synchronize()
 
     # per-call times (each case on its own, back-to-back launches on the one stream)
     for c in cases:
@@ -368,7 +540,11 @@ def main() -> int:
                    "device": info["arch"], "compute_units": info["compute_units"]},
         "roofline": {k: (round(v, 4) if isinstance(v, float) else v) for k, v in roofline.items()},
         "wall_s_timed_region": round(wall_s, 4),
+        "timing": f"{B.warm_ms:g} ms of untimed steps, {args.warmup} warm-up steps, median of 5 batches of {args.steps} steps",
     }
+    if default_step is not None:
+        result["heuristic_defaults"] = default_step
+    result["sum_of_per_call_us"] = round(sum(c["us"] for c in cases), 2)
 
     details = {}
     details["decode_calls"] = [

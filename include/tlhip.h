@@ -119,6 +119,10 @@ typedef struct {
 
 /* ---- runtime: what the WebGPU context/queue provides to the reference
  * backend (src/backend/webgpu/gpu-context.ts; creation.ts:51-87; `read`). ---- */
+/* tlhip_init also imports the tuning file that ships next to the library
+ * (<directory of libtlhip.so>/tuning/mi355x.json; the environment variable
+ * TLHIP_TUNING_FILE names another file, "none" none), as importTuningCache would:
+ * every binding runs the committed kernel choices, re-gated on applicability. */
 int tlhip_init(int device_index);
 int tlhip_shutdown(void);
 const char* tlhip_last_error(void);
@@ -144,8 +148,21 @@ int tlhip_event_elapsed_us(tlhip_event_t start, tlhip_event_t stop, double* host
  * can be replayed with one call.  The reference batches a decode step's
  * dispatches into one command-buffer submission
  * (src/backend/webgpu/shared-encoder.ts); a captured graph is the HIP
- * counterpart.  The compute entry points enqueue kernels only (no memset or
- * allocation), so all of them may be captured; autotuning must be off. */
+ * counterpart.  Rules:
+ *  - the compute entry points enqueue kernels only, so all of them may be captured;
+ *    tlhip_memset returns TLHIP_ERR_STATE on a capturing stream, and lazy autotuning
+ *    is skipped there;
+ *  - a kernel that splits K across workgroups (and tlhip_topk) works through the
+ *    stream's workspace, which is created on the stream's first such call: make that
+ *    call once before capturing, or the call under capture returns TLHIP_ERR_STATE
+ *    (tlhip_gemv_noalloc never needs this);
+ *  - the workspace pointers are part of the captured kernels' arguments: a graph
+ *    replays on the stream it was captured on (another stream: TLHIP_ERR_INVALID),
+ *    in order with that stream's other launches; the workspace stays allocated until
+ *    the stream AND every graph captured on it are destroyed; tlhip_shutdown destroys
+ *    graphs that are still alive;
+ *  - a replay that is aborted half-way (device reset) can leave arrival counters
+ *    non-zero; nothing short of tlhip_shutdown / tlhip_init clears them. */
 int tlhip_graph_begin_capture(tlhip_stream_t stream);
 int tlhip_graph_end_capture(tlhip_stream_t stream, tlhip_graph_t* host_out);
 int tlhip_graph_launch(tlhip_graph_t graph, tlhip_stream_t stream);
@@ -342,8 +359,10 @@ int tlhip_candidate_count(const tlhip_qweight_t* w, int x_dtype, int64_t m, int 
                           int* host_out_count);
 int tlhip_candidate_get(const tlhip_qweight_t* w, int x_dtype, int64_t m, int y_dtype, int index,
                         tlhip_kernel_config_t* host_out);
-/* The configuration tlhip_matmul_quantized would use now (tuned winner if
- * cached, else the heuristic default) — selectMatmulChoice, dispatch.ts:171-192. */
+/* The configuration tlhip_matmul_quantized would use now: the tuned winner of this
+ * exact problem if cached, else the winner of the nearest tuned problem of the same
+ * shape class (autotune.ts:269-300), else the heuristic default — selectMatmulChoice,
+ * dispatch.ts:171-192.  Every level is re-gated on applicability. */
 int tlhip_selected_config(const tlhip_qweight_t* w, int x_dtype, int64_t m, int y_dtype,
                           tlhip_kernel_config_t* host_out);
 
@@ -351,11 +370,36 @@ int tlhip_selected_config(const tlhip_qweight_t* w, int x_dtype, int64_t m, int 
  * on by the environment variable TORCHLETTE_AUTOTUNE=1 (dispatch.ts:559). */
 int tlhip_set_autotune_enabled(int enabled);
 int tlhip_is_autotune_enabled(void);
-/* Benchmark every candidate for this problem (2 warm-up + 3 timed launches
- * each, median, as dispatch.ts:324-397) and cache the winner under the key
- * (m, n, k, format, group, x dtype, y dtype).  Runs on the library stream. */
+/* Benchmark every candidate for this problem (2 warm-up launches + 3 timed batches
+ * each, median, after dispatch.ts:324-397) and cache the winner under the key
+ * (m, n, k, format, group, x dtype, y dtype) and under its shape class.  Runs on the
+ * library stream with the defaults of tlhip_autotune_pool. */
 int tlhip_autotune(const tlhip_qweight_t* w, const void* x, int x_dtype, int64_t m, void* y,
                    int y_dtype, double* host_out_best_us);
+/* The same with the knobs exposed, an epilogue and a caller's stream.
+ * `weights` are `weight_count` buffers of ONE weight shape (format, n, k, group size;
+ * the same or different contents), rotated launch by launch: a 9-28 MB decode weight
+ * stays resident in the 256 MB last-level cache when one buffer is launched over and
+ * over, and the candidates would be ranked by a rate no decode step ever sees.  With
+ * weight_count == 1 the tuner makes alias copies itself, up to options->pool_bytes
+ * (freed before it returns; never under graph capture, where tuning is skipped).
+ * Each candidate: 2 untimed launches, then `batches` event pairs around `reps`
+ * back-to-back launches, median; the `retime_top` fastest are timed once more, three
+ * times as long.  quick = 1 searches only the neighbours of the current choice
+ * (generateNeighborConfigs, autotune.ts:419-465).  options == NULL: the defaults
+ * (reps sized to about 300 us per batch, 3 batches, top 3, 30 ms warm-up, 640 MiB). */
+typedef struct {
+  int32_t reps;       /* launches per event pair; 0 = automatic (20..100) */
+  int32_t batches;    /* 0 = 3 */
+  int32_t retime_top; /* 0 = 3; 1 = no second pass */
+  int32_t quick;
+  double warm_ms;     /* < 0 = 30 */
+  uint64_t pool_bytes;
+} tlhip_autotune_options_t;
+int tlhip_autotune_pool(const tlhip_qweight_t* weights, int weight_count, const void* x, int x_dtype,
+                        int64_t m, void* y, int y_dtype, const tlhip_epilogue_t* epilogue,
+                        const tlhip_autotune_options_t* options, tlhip_stream_t stream,
+                        double* host_out_best_us);
 /* seedPerShapeMatmulChoice (dispatch.ts:99-107): record a winner for this
  * problem without benchmarking (tests, pre-seeded caches, a caller's own
  * timing loop).  Fails if the configuration is not applicable. */
@@ -373,7 +417,8 @@ int tlhip_tune_cache_clear(void);
 
 /* Dispatch counters, the reference's test hooks (dispatch.ts:79-83, 832-864,
  * 943-947): "quant_gemv_dispatches", "quant_gemm_dispatches",
- * "dequant_dispatches", "autotune_runs".  Unknown names return 0. */
+ * "dequant_dispatches", "autotune_runs", and "tuning_entries_loaded" (entries
+ * imported from the tuning file at tlhip_init).  Unknown names return 0. */
 uint64_t tlhip_counter(const char* name);
 int tlhip_counters_reset(void);
 

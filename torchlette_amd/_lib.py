@@ -74,6 +74,11 @@ PRO_NONE, PRO_RMSNORM, PRO_GATED_MUL = 0, 1, 2
 ERR_INVALID, ERR_DEVICE, ERR_STATE, ERR_UNSUPPORTED = 1, 2, 3, 4
 
 
+class AutotuneOptions(C.Structure):
+    _fields_ = [("reps", C.c_int32), ("batches", C.c_int32), ("retime_top", C.c_int32), ("quick", C.c_int32),
+                ("warm_ms", C.c_double), ("pool_bytes", C.c_uint64)]
+
+
 class GemvProblem(C.Structure):
     _fields_ = [("w", QWeight), ("x", C.c_void_p), ("y", C.c_void_p), ("epilogue", C.POINTER(Epilogue))]
 
@@ -132,6 +137,8 @@ SIGNATURES = {
     "tlhip_set_autotune_enabled": (_i, [_i]),
     "tlhip_is_autotune_enabled": (_i, []),
     "tlhip_autotune": (_i, [_QW, _vp, _i, _i64, _vp, _i, C.POINTER(C.c_double)]),
+    "tlhip_autotune_pool": (_i, [_QW, _i, _vp, _i, _i64, _vp, _i, _EP, C.POINTER(AutotuneOptions), _vp,
+                                C.POINTER(C.c_double)]),
     "tlhip_tune_cache_seed": (_i, [_QW, _i, _i64, _i, _KC]),
     "tlhip_pretune_matmul_shapes": (_i, [C.POINTER(_i64), _i]),
     "tlhip_tune_cache_export": (_i, [C.c_char_p, _sz, C.POINTER(_sz)]),

@@ -120,9 +120,28 @@ int run_kernel_config(const Problem& p, const tlhip_kernel_config_t& c, hipStrea
 // K slices across workgroups of a configuration (1 = it needs no scratch).
 int config_k_slices(const tlhip_kernel_config_t& c);
 
+// Imports the tuning file that ships with the library (dispatch.cpp); returns the number
+// of entries added.
+int load_default_tuning();
+void count_tuning_entries_loaded(int n);
+
 // Set-up of the entry point that allocates nothing (noalloc.hip): resolves the device
 // address of its static scratch array for the current device.
 int noalloc_setup(int device_index);
+
+// Launch of a library kernel.  A kernel that takes more than 64 KiB of dynamic LDS needs its
+// limit raised (hipFuncSetAttribute); that is done once per kernel, for every kernel of the
+// library, at tlhip_init (prepare_all_kernels: each translation unit walks its own dispatch
+// tables in "prepare mode", in which launch_kernel raises the limit and launches nothing),
+// so that no launch, and nothing a caller captures into a graph, carries an attribute call.
+int launch_kernel(const void* fn, dim3 grid, dim3 block, void** args, size_t lds_bytes, hipStream_t stream);
+bool prepare_mode();
+int prepare_all_kernels();
+int prepare_gemv_kernels();       // gemv.hip (+ the per-format units)
+int prepare_gemv_mfma_kernels();  // gemv_mfma.hip
+int prepare_gemv_xreg_kernels();  // gemv_mfma_xreg.hip
+int prepare_gemm_kernels();       // gemm_prefill.hip
+int prepare_gemm_direct_kernels();  // gemm_direct.hip
 
 // Counters.
 void count_gemv_dispatch();

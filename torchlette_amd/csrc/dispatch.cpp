@@ -7,13 +7,21 @@
 //    src/backend/webgpu/matmul/dispatch.ts:171-192: explicit config, then the
 //    per-shape tuned winner (re-gated on applicability), then the first
 //    applicable variant's heuristic default;
-//  * the autotuner of dispatch.ts:405-547 (2 warm-up + 3 timed runs per
+//  * the autotuner of dispatch.ts:405-547 (warm-up, then timed runs per
 //    candidate, median) with a per-exact-shape cache that, unlike the
 //    reference's m_n_k_dtype key, also carries the operand format, because the
-//    winner differs per packing;
+//    winner differs per packing; a candidate is timed as a batch of back-to-back
+//    launches per event pair (the kernels take 3-12 us: one launch per event pair
+//    measures the events), with the weight rotating through alias buffers larger
+//    than the last-level cache, and the three fastest are timed once more, longer;
+//  * the per-shape-class level of autotune.ts:269-300: an untuned problem takes
+//    the winner of the nearest tuned problem of its class before the hand
+//    heuristic, and a quick tuning pass searches the neighbours of that choice
+//    (generateNeighborConfigs, autotune.ts:419-465);
 //  * exportTuningCache / importTuningCache (autotune.ts:309-329) as JSON text.
 #include <algorithm>
 #include <array>
+#include <cmath>
 #include <cstdlib>
 #include <cstring>
 #include <map>
@@ -22,13 +30,23 @@
 #include <string>
 #include <vector>
 
+#include <dlfcn.h>
+
 #include "common.h"
 
 namespace tlhip {
 namespace {
 
-std::mutex g_tune_mutex;
+std::mutex g_tune_mutex;      // guards every variable of this block
+std::mutex g_tune_run_mutex;  // held for a whole tuning run: one tuner at a time
 std::map<std::string, tlhip_kernel_config_t> g_tuned;  // per exact problem key
+// The shape-class level (autotune.ts:269-300): every per-shape winner is also filed under
+// its class, with the shape it was found for.
+struct ClassEntry {
+  int64_t m, n, k;
+  tlhip_kernel_config_t config;
+};
+std::map<std::string, std::vector<ClassEntry>> g_class_tuned;
 std::vector<std::array<int64_t, 3>> g_shape_hints;
 int g_autotune_counter = 0;
 bool g_autotuning = false;  // no recursive tuning (dispatch.ts autotuningInProgress)
@@ -50,6 +68,55 @@ std::string problem_key(const Problem& p) {
            format_name(p.format), p.format == TLHIP_FMT_INT8_ROW ? 0 : p.group_size,
            p.x_dtype == TLHIP_F16 ? "f16" : "f32", p.y_dtype == TLHIP_F16 ? "f16" : "f32");
   return buf;
+}
+
+// Shape class of a problem: which kernel family serves it (rows M), what bounds it
+// (bytes of packed weights: launch-, stream- or capacity-bound) and whether the
+// activation rows fit one workgroup's LDS (K), per operand format and types.  The role
+// of classifyShape (src/backend/webgpu/matmul/types.ts:146-200) for this path.
+std::string class_key(const Problem& p) {
+  const char* mc = p.m == 1 ? "m1" : p.m == 2 ? "m2" : p.m <= 4 ? "m4" : p.m <= 16 ? "m16" : p.m < 1024 ? "mid" : "big";
+  const double bytes = (double)p.n * (double)p.k * (p.format == TLHIP_FMT_INT4_GROUPED ? 0.5 : 1.0);
+  const char* sc = bytes < 4e6 ? "small" : bytes < 96e6 ? "medium" : "large";
+  const char* kc = p.k <= 4096 ? "k4k" : p.k <= 8192 ? "k8k" : "klong";
+  char buf[160];
+  snprintf(buf, sizeof buf, "%s_%s_%s_%s_g%d_%s_%s", mc, sc, kc, format_name(p.format),
+           p.format == TLHIP_FMT_INT8_ROW ? 0 : p.group_size, p.x_dtype == TLHIP_F16 ? "f16" : "f32",
+           p.y_dtype == TLHIP_F16 ? "f16" : "f32");
+  return buf;
+}
+
+// Key text -> the shape-determining fields of a Problem (what export writes).
+bool parse_problem_key(const std::string& key, Problem* p) {
+  long long m = 0, n = 0, k = 0;
+  char fmt[32] = "", xd[8] = "", yd[8] = "";
+  int g = 0;
+  if (sscanf(key.c_str(), "%lld_%lld_%lld_%31[^_]_g%d_%7[^_]_%7s", &m, &n, &k, fmt, &g, xd, yd) != 7) return false;
+  memset(p, 0, sizeof *p);
+  if (!strcmp(fmt, "int8-grouped")) p->format = TLHIP_FMT_INT8_GROUPED;
+  else if (!strcmp(fmt, "int8-row")) p->format = TLHIP_FMT_INT8_ROW;
+  else if (!strcmp(fmt, "int4-grouped")) p->format = TLHIP_FMT_INT4_GROUPED;
+  else return false;
+  p->m = m;
+  p->n = n;
+  p->k = k;
+  p->group_size = g;
+  p->x_dtype = !strcmp(xd, "f16") ? TLHIP_F16 : TLHIP_F32;
+  p->y_dtype = !strcmp(yd, "f16") ? TLHIP_F16 : TLHIP_F32;
+  p->alpha = 1.f;
+  return true;
+}
+
+// Caller holds g_tune_mutex.
+void record_winner_locked(const Problem& p, const tlhip_kernel_config_t& c) {
+  g_tuned[problem_key(p)] = c;
+  auto& list = g_class_tuned[class_key(p)];
+  for (auto& e : list)
+    if (e.m == p.m && e.n == p.n && e.k == p.k) {
+      e.config = c;
+      return;
+    }
+  list.push_back({p.m, p.n, p.k, c});
 }
 
 bool env_autotune() {
@@ -241,12 +308,39 @@ std::vector<tlhip_kernel_config_t> candidates(const Problem& p) {
   return out;
 }
 
+// The winner of the nearest tuned problem of the same class (autotune.ts:269-300's
+// per-shape-class cache), re-gated on applicability.  "Near" = N and K each within a
+// factor of two and the same number of rows where the kernel family depends on it;
+// farther than that the hand heuristic knows more than a foreign winner does.
+bool class_config(const Problem& p, tlhip_kernel_config_t* out) {
+  std::lock_guard<std::mutex> lock(g_tune_mutex);
+  auto it = g_class_tuned.find(class_key(p));
+  if (it == g_class_tuned.end()) return false;
+  double best = 1e30;
+  bool found = false;
+  for (const auto& e : it->second) {
+    const double dn = std::fabs(std::log2((double)e.n / (double)p.n));
+    const double dk = std::fabs(std::log2((double)e.k / (double)p.k));
+    const double dm = std::fabs(std::log2((double)e.m / (double)p.m));
+    if (dn > 1.0 || dk > 1.0 || dm > 1.0) continue;
+    const double d = dn + 2.0 * dk + dm;  // K decides whether the activations fit LDS: weigh it
+    if (d < best && config_applicable(p, e.config, nullptr)) {
+      best = d;
+      *out = e.config;
+      found = true;
+    }
+  }
+  return found;
+}
+
 tlhip_kernel_config_t select_config(const Problem& p) {
   {
     std::lock_guard<std::mutex> lock(g_tune_mutex);
     auto it = g_tuned.find(problem_key(p));
     if (it != g_tuned.end() && config_applicable(p, it->second, nullptr)) return it->second;
   }
+  tlhip_kernel_config_t c;
+  if (class_config(p, &c)) return c;
   return default_config(p);
 }
 
@@ -276,57 +370,254 @@ int run_config(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t str
   return launch_gemv(p, c, stream);
 }
 
-int autotune_problem(const Problem& p, double* best_us_out) {
-  if (g_autotuning) return TLHIP_OK;
-  g_autotuning = true;
-  hipStream_t stream = resolve_stream(nullptr);
-  hipEvent_t e0, e1;
-  int rc = TLHIP_OK;
-  if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) {
-    g_autotuning = false;
-    return set_error(TLHIP_ERR_DEVICE, "autotune: hipEventCreate failed");
+int matmul_with(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t stream) {
+  if (c.variant == VARIANT_TILED || c.variant == VARIANT_TILED_DIRECT) return run_config(p, c, stream);
+  if (p.m <= 16) return run_config(p, c, stream);
+  // f32 activations (or a shape the tiled kernel rejects) above 16 rows: GEMV
+  // passes of 16 rows.  Declared, slow: every pass streams the weights again.
+  const int xb = p.x_dtype == TLHIP_F16 ? 2 : 4, yb = p.y_dtype == TLHIP_F16 ? 2 : 4;
+  for (int64_t m0 = 0; m0 < p.m; m0 += 16) {
+    Problem q = p;
+    q.m = std::min<int64_t>(16, p.m - m0);
+    q.x = (const char*)p.x + m0 * p.k * xb;
+    q.y = (char*)p.y + m0 * p.n * yb;
+    int rc = run_config(q, c, stream);
+    if (rc) return rc;
   }
-  double best = 1e30;
-  tlhip_kernel_config_t best_cfg = default_config(p);
-  for (const auto& c : candidates(p)) {
-    bool ok = true;
-    for (int i = 0; i < 2 && ok; ++i) ok = run_config(p, c, stream) == TLHIP_OK;  // warm-up
-    if (!ok) continue;
-    double t[3];
-    for (int i = 0; i < 3 && ok; ++i) {
-      (void)hipEventRecord(e0, stream);
-      ok = run_config(p, c, stream) == TLHIP_OK;
-      (void)hipEventRecord(e1, stream);
-      if (hipEventSynchronize(e1) != hipSuccess) {
-        ok = false;
-        rc = set_error(TLHIP_ERR_DEVICE, "autotune: hipEventSynchronize failed");
-        break;
-      }
-      float ms = 0;
-      (void)hipEventElapsedTime(&ms, e0, e1);
-      t[i] = ms * 1000.0;
+  return TLHIP_OK;
+}
+
+// One-field variations of `base` inside its kernel family, plus the heuristic defaults of
+// the families: the quick search of generateNeighborConfigs (autotune.ts:419-465).
+std::vector<tlhip_kernel_config_t> neighbour_candidates(const Problem& p, const tlhip_kernel_config_t& base) {
+  std::vector<tlhip_kernel_config_t> out;
+  auto same = [](const tlhip_kernel_config_t& a, const tlhip_kernel_config_t& b) { return !memcmp(&a, &b, sizeof a); };
+  auto push = [&](const tlhip_kernel_config_t& c) {
+    if (!config_applicable(p, c, nullptr)) return;
+    for (const auto& o : out)
+      if (same(o, c)) return;
+    out.push_back(c);
+  };
+  push(base);
+  auto vary = [&](int field, std::initializer_list<int> values) {
+    for (int v : values) {
+      tlhip_kernel_config_t c = base;
+      (&c.p0)[field] = v;
+      push(c);
     }
-    if (rc) break;
-    if (!ok) continue;
-    std::sort(t, t + 3);
-    if (t[1] < best) {
-      best = t[1];
-      best_cfg = c;
-    }
+  };
+  switch (base.variant) {
+    case VARIANT_GEMV:
+      vary(0, {16, 32, 64});
+      vary(1, {1, 2, 4});
+      vary(2, {2, 4, 8});
+      vary(3, {1, 2, 4});
+      vary(4, {2, 4, 8});
+      vary(5, {0, 1});
+      break;
+    case VARIANT_GEMV_MFMA:
+      vary(0, {4, 8, 16});
+      vary(1, {1, 2, 4});
+      vary(2, {1, 2, 4, 8, 16});
+      vary(3, {1, 2, 4, 8});
+      vary(5, {0, 1});
+      break;
+    case VARIANT_GEMV_XREG:
+      vary(0, {4, 8, 16});
+      vary(1, {1, 2});
+      vary(2, {1, 2});
+      vary(3, {1, 2, 4, 8, 16});
+      break;
+    default:
+      for (const auto& c : candidates(p))
+        if (c.variant == VARIANT_TILED || c.variant == VARIANT_TILED_DIRECT) push(c);
+      break;
   }
-  (void)hipEventDestroy(e0);
-  (void)hipEventDestroy(e1);
-  g_autotuning = false;
-  if (rc) return rc;
+  push(default_config(p));
+  if (p.m <= 16) push(default_valu_config(p));
+  return out;
+}
+
+struct TuneOptions {
+  int reps = 0;           // launches per event pair; 0 = sized so that a batch takes about 300 us (20..100)
+  int batches = 3;        // timed batches per candidate, median (dispatch.ts:324-397: 3 timed runs)
+  int retime_top = 3;     // the fastest candidates timed once more, three times as long, minimum
+  double warm_ms = 30.0;  // GPU milliseconds of untimed launches first: the clock ramps up after a pause
+  bool quick = false;     // neighbours of the current choice instead of every candidate
+  size_t pool_bytes = (size_t)640 << 20;  // alias copies of the weight the tuner makes when given only one buffer
+};
+
+struct WeightAlias {
+  const void* packed;
+  const void* scales;
+};
+
+size_t packed_bytes(const Problem& p) { return (size_t)p.n * (size_t)p.k / (p.format == TLHIP_FMT_INT4_GROUPED ? 2 : 1); }
+size_t scales_bytes(const Problem& p) {
+  return p.format == TLHIP_FMT_INT8_ROW ? (size_t)p.n * 4 : (size_t)p.n * (size_t)(p.k / p.group_size) * 2;
+}
+
+// Times the candidates for `p` and caches the winner.  `aliases`: the weight in distinct
+// buffers (same contents or not, same shape), rotated launch by launch so that a weight
+// smaller than the 256 MB last-level cache is still timed from HBM; with a single
+// buffer the tuner makes its own copies, up to `pool_bytes`, and frees them afterwards.
+int autotune_problem(const Problem& p0, std::vector<WeightAlias> aliases, const TuneOptions& o, hipStream_t stream,
+                     double* best_us_out) {
   {
     std::lock_guard<std::mutex> lock(g_tune_mutex);
-    g_tuned[problem_key(p)] = best_cfg;
+    if (g_autotuning) return TLHIP_OK;
+  }
+  hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &cap) == hipSuccess && cap != hipStreamCaptureStatusNone) return TLHIP_OK;
+  std::lock_guard<std::mutex> run_lock(g_tune_run_mutex);
+  {
+    std::lock_guard<std::mutex> lock(g_tune_mutex);
+    g_autotuning = true;
+  }
+  struct Done {
+    ~Done() {
+      std::lock_guard<std::mutex> lock(g_tune_mutex);
+      g_autotuning = false;
+    }
+  } done;
+
+  if (aliases.empty()) aliases.push_back({p0.packed, p0.scales});
+  std::vector<void*> owned;
+  struct FreeOwned {
+    std::vector<void*>& v;
+    hipStream_t s;
+    ~FreeOwned() {
+      if (v.empty()) return;
+      (void)hipStreamSynchronize(s);
+      for (void* q : v) (void)hipFree(q);
+    }
+  } free_owned{owned, stream};
+  const size_t pb = packed_bytes(p0), sb = scales_bytes(p0);
+  if (aliases.size() == 1 && o.pool_bytes > pb + sb && pb + sb < ((size_t)256 << 20)) {
+    size_t want = o.pool_bytes / (pb + sb);
+    if (want > 95) want = 95;
+    for (size_t i = 0; i < want; ++i) {
+      void *wp = nullptr, *sp = nullptr;
+      if (hipMalloc(&wp, pb) != hipSuccess) break;
+      if (hipMalloc(&sp, sb) != hipSuccess) {
+        (void)hipFree(wp);
+        break;
+      }
+      owned.push_back(wp);
+      owned.push_back(sp);
+      if (hipMemcpyAsync(wp, p0.packed, pb, hipMemcpyDeviceToDevice, stream) != hipSuccess ||
+          hipMemcpyAsync(sp, p0.scales, sb, hipMemcpyDeviceToDevice, stream) != hipSuccess)
+        break;
+      aliases.push_back({wp, sp});
+    }
+    (void)hipGetLastError();  // a failed allocation only means fewer aliases
+  }
+
+  hipEvent_t e0, e1;
+  if (hipEventCreate(&e0) != hipSuccess) return set_error(TLHIP_ERR_DEVICE, "autotune: hipEventCreate failed");
+  if (hipEventCreate(&e1) != hipSuccess) {
+    (void)hipEventDestroy(e0);
+    return set_error(TLHIP_ERR_DEVICE, "autotune: hipEventCreate failed");
+  }
+  struct FreeEvents {
+    hipEvent_t a, b;
+    ~FreeEvents() {
+      (void)hipEventDestroy(a);
+      (void)hipEventDestroy(b);
+    }
+  } free_events{e0, e1};
+
+  size_t turn = 0;
+  auto launch = [&](const tlhip_kernel_config_t& c) {
+    Problem q = p0;
+    const WeightAlias& a = aliases[turn++ % aliases.size()];
+    q.packed = a.packed;
+    q.scales = a.scales;
+    return matmul_with(q, c, stream) == TLHIP_OK;
+  };
+  // microseconds per launch of `reps` back-to-back launches; < 0: the candidate failed
+  int device_error = 0;
+  auto time_batch = [&](const tlhip_kernel_config_t& c, int reps) -> double {
+    if (hipEventRecord(e0, stream) != hipSuccess) return -1.0;
+    for (int i = 0; i < reps; ++i)
+      if (!launch(c)) {
+        (void)hipStreamSynchronize(stream);
+        return -1.0;
+      }
+    if (hipEventRecord(e1, stream) != hipSuccess || hipEventSynchronize(e1) != hipSuccess) {
+      device_error = 1;
+      return -1.0;
+    }
+    float ms = 0;
+    (void)hipEventElapsedTime(&ms, e0, e1);
+    return (double)ms * 1000.0 / reps;
+  };
+
+  const tlhip_kernel_config_t current = select_config(p0);
+  // warm-up on the current choice, and the batch length from its time
+  double cur_us = time_batch(current, 20);
+  if (device_error) return set_error(TLHIP_ERR_DEVICE, "autotune: a timing event failed");
+  if (cur_us <= 0) cur_us = 10.0;
+  int reps = o.reps > 0 ? o.reps : (int)(300.0 / cur_us);
+  if (o.reps <= 0) reps = reps < 20 ? 20 : (reps > 100 ? 100 : reps);
+  for (double spent = 0; spent < o.warm_ms * 1e3;) {
+    const double us = time_batch(current, reps);
+    if (us <= 0) break;
+    spent += us * reps;
+  }
+
+  const std::vector<tlhip_kernel_config_t> cands = o.quick ? neighbour_candidates(p0, current) : candidates(p0);
+  std::vector<std::pair<double, tlhip_kernel_config_t>> timed;
+  const int batches = o.batches < 1 ? 1 : (o.batches > 9 ? 9 : o.batches);
+  for (const auto& c : cands) {
+    if (!launch(c) || !launch(c)) {  // two untimed launches (dispatch.ts:324-397: 2 warm-up runs)
+      (void)hipStreamSynchronize(stream);
+      continue;
+    }
+    double t[9];
+    bool ok = true;
+    for (int i = 0; i < batches && ok; ++i) {
+      t[i] = time_batch(c, reps);
+      ok = t[i] > 0;
+    }
+    if (device_error) return set_error(TLHIP_ERR_DEVICE, "autotune: a timing event failed");
+    if (!ok) continue;
+    std::sort(t, t + batches);
+    timed.push_back({t[batches / 2], c});
+  }
+  if (timed.empty()) return set_error(TLHIP_ERR_INVALID, "autotune: no candidate configuration ran for %s", problem_key(p0).c_str());
+  std::sort(timed.begin(), timed.end(), [](const auto& a, const auto& b) { return a.first < b.first; });
+  double best = timed[0].first;
+  tlhip_kernel_config_t best_cfg = timed[0].second;
+  // candidates within a few per cent of each other change places from run to run: the
+  // fastest few once more, three times as long, the minimum of three batches
+  if (o.retime_top > 1 && timed.size() > 1) {
+    best = 1e30;
+    const size_t top = std::min<size_t>(timed.size(), (size_t)o.retime_top);
+    for (size_t i = 0; i < top; ++i) {
+      double us = 1e30;
+      for (int r = 0; r < 3; ++r) {
+        const double v = time_batch(timed[i].second, 3 * reps);
+        if (v > 0 && v < us) us = v;
+      }
+      if (device_error) return set_error(TLHIP_ERR_DEVICE, "autotune: a timing event failed");
+      if (us < best) {
+        best = us;
+        best_cfg = timed[i].second;
+      }
+    }
+  }
+  {
+    std::lock_guard<std::mutex> lock(g_tune_mutex);
+    record_winner_locked(p0, best_cfg);
   }
   count_autotune_run();
   if (best_us_out) *best_us_out = best;
   if (getenv("TORCHLETTE_DEBUG_AUTOTUNE"))
-    fprintf(stderr, "[tlhip autotune] %s -> variant %d (%d,%d,%d,%d,%d) %.2f us\n", problem_key(p).c_str(),
-            best_cfg.variant, best_cfg.p0, best_cfg.p1, best_cfg.p2, best_cfg.p3, best_cfg.p4, best);
+    fprintf(stderr, "[tlhip autotune] %s: %zu candidates, %zu weight buffers, %d launches per batch -> variant %d "
+                    "(%d,%d,%d,%d,%d,%d) %.2f us\n",
+            problem_key(p0).c_str(), cands.size(), aliases.size(), reps, best_cfg.variant, best_cfg.p0, best_cfg.p1,
+            best_cfg.p2, best_cfg.p3, best_cfg.p4, best_cfg.p5, best);
   return TLHIP_OK;
 }
 
@@ -339,6 +630,43 @@ tlhip_kernel_config_t select_gemv_config(const Problem& p) {
 }
 
 int run_kernel_config(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t stream) { return run_config(p, c, stream); }
+
+// The tuning file that ships next to the library: <directory of libtlhip.so>/tuning/
+// mi355x.json, or the file TLHIP_TUNING_FILE names ("none" = load nothing).  Called by
+// tlhip_init, so every binding gets the committed winners, not only the benchmark.
+// A missing or malformed file is not an error: the heuristic defaults serve.
+int load_default_tuning() {
+  std::string path;
+  if (const char* e = getenv("TLHIP_TUNING_FILE")) {
+    if (!strcmp(e, "none") || !*e) return 0;
+    path = e;
+  } else {
+    Dl_info info;
+    if (!dladdr((const void*)&load_default_tuning, &info) || !info.dli_fname) return 0;
+    path = info.dli_fname;
+    const size_t slash = path.rfind('/');
+    path = (slash == std::string::npos ? std::string(".") : path.substr(0, slash)) + "/tuning/mi355x.json";
+  }
+  FILE* f = fopen(path.c_str(), "rb");
+  if (!f) return 0;
+  std::string text;
+  char buf[4096];
+  size_t got;
+  while ((got = fread(buf, 1, sizeof buf, f)) > 0) text.append(buf, got);
+  fclose(f);
+  size_t before;
+  {
+    std::lock_guard<std::mutex> lock(g_tune_mutex);
+    before = g_tuned.size();
+  }
+  if (tlhip_tune_cache_import(text.c_str()) != TLHIP_OK) {
+    if (getenv("TORCHLETTE_DEBUG_AUTOTUNE")) fprintf(stderr, "[tlhip] tuning file %s ignored: %s\n", path.c_str(), tlhip_last_error());
+    clear_error();
+    return 0;
+  }
+  std::lock_guard<std::mutex> lock(g_tune_mutex);
+  return (int)(g_tuned.size() - before);
+}
 
 int config_k_slices(const tlhip_kernel_config_t& c) {
   if (c.variant == VARIANT_GEMV_MFMA || c.variant == VARIANT_GEMV_XREG) return c.p3 < 1 ? 1 : c.p3;
@@ -435,8 +763,6 @@ int tlhip_dequant(const tlhip_qweight_t* w, float* out, tlhip_stream_t stream) {
   if (((uintptr_t)out & 15) != 0) return set_error(TLHIP_ERR_INVALID, "dequant: output must be 16-byte aligned");
   return launch_dequant(*w, out, resolve_stream(stream));
 }
-
-static int matmul_with(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t stream);
 
 int tlhip_gemv(const tlhip_qweight_t* w, const void* x, int x_dtype, int64_t m, void* y, int y_dtype,
                float alpha, const tlhip_epilogue_t* epilogue, tlhip_stream_t stream) {
@@ -559,23 +885,6 @@ int tlhip_gemm_prefill(const tlhip_qweight_t* w, const void* x, int x_dtype, int
   return run_config(p, c, resolve_stream(stream));
 }
 
-static int matmul_with(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t stream) {
-  if (c.variant == VARIANT_TILED || c.variant == VARIANT_TILED_DIRECT) return run_config(p, c, stream);
-  if (p.m <= 16) return run_config(p, c, stream);
-  // f32 activations (or a shape the tiled kernel rejects) above 16 rows: GEMV
-  // passes of 16 rows.  Declared, slow: every pass streams the weights again.
-  const int xb = p.x_dtype == TLHIP_F16 ? 2 : 4, yb = p.y_dtype == TLHIP_F16 ? 2 : 4;
-  for (int64_t m0 = 0; m0 < p.m; m0 += 16) {
-    Problem q = p;
-    q.m = std::min<int64_t>(16, p.m - m0);
-    q.x = (const char*)p.x + m0 * p.k * xb;
-    q.y = (char*)p.y + m0 * p.n * yb;
-    int rc = run_config(q, c, stream);
-    if (rc) return rc;
-  }
-  return TLHIP_OK;
-}
-
 int tlhip_matmul_quantized(const tlhip_qweight_t* w, const void* x, int x_dtype, int64_t m, void* y,
                            int y_dtype, float alpha, const tlhip_epilogue_t* epilogue, tlhip_stream_t stream) {
   TLHIP_REQUIRE_INIT();
@@ -583,18 +892,21 @@ int tlhip_matmul_quantized(const tlhip_qweight_t* w, const void* x, int x_dtype,
   int rc = make_problem(w, x, x_dtype, m, y, y_dtype, alpha, epilogue, &p, "matmulQuantizedB");
   if (rc) return rc;
   if (p.m == 0 || p.n == 0) return TLHIP_OK;
-  if ((g_autotune_counter > 0 || env_autotune()) && !g_autotuning) {
-    bool have;
-    {
-      std::lock_guard<std::mutex> lock(g_tune_mutex);
-      have = g_tuned.count(problem_key(p)) != 0;
-    }
-    if (!have) {
-      // Tuning launches write y; the real launch below overwrites it.
-      (void)hipStreamSynchronize(resolve_stream(stream));
-      rc = autotune_problem(p, nullptr);
-      if (rc) return rc;
-    }
+  bool tune;
+  {
+    std::lock_guard<std::mutex> lock(g_tune_mutex);
+    tune = (g_autotune_counter > 0 || env_autotune()) && !g_autotuning && g_tuned.count(problem_key(p)) == 0;
+  }
+  if (tune) {
+    // Lazy tuning at first dispatch (dispatch.ts:559-578), on the caller's stream; the
+    // tuning launches write y, which the real launch below overwrites.  A problem whose
+    // class already has a winner nearby gets the quick neighbour search.
+    hipStream_t s = resolve_stream(stream);
+    TuneOptions o;
+    tlhip_kernel_config_t near;
+    o.quick = class_config(p, &near);
+    rc = autotune_problem(p, {}, o, s, nullptr);
+    if (rc) return rc;
   }
   return matmul_with(p, select_config(p), resolve_stream(stream));
 }
@@ -670,27 +982,56 @@ int tlhip_tune_cache_seed(const tlhip_qweight_t* w, int x_dtype, int64_t m, int 
   if (!config_applicable(p, *config, &why))
     return set_error(TLHIP_ERR_INVALID, "tune_cache_seed: config not applicable: %s", why ? why : "?");
   std::lock_guard<std::mutex> lock(g_tune_mutex);
-  g_tuned[problem_key(p)] = *config;
+  record_winner_locked(p, *config);
   return TLHIP_OK;
 }
 
 int tlhip_set_autotune_enabled(int enabled) {
   // dispatch.ts:128-134: true increments (nested regions), false resets to 0.
+  std::lock_guard<std::mutex> lock(g_tune_mutex);
   if (enabled) g_autotune_counter++;
   else g_autotune_counter = 0;
   return TLHIP_OK;
 }
 
-int tlhip_is_autotune_enabled(void) { return g_autotune_counter > 0 || env_autotune(); }
+int tlhip_is_autotune_enabled(void) {
+  std::lock_guard<std::mutex> lock(g_tune_mutex);
+  return g_autotune_counter > 0 || env_autotune();
+}
 
 int tlhip_autotune(const tlhip_qweight_t* w, const void* x, int x_dtype, int64_t m, void* y, int y_dtype,
                    double* best_us) {
+  return tlhip_autotune_pool(w, 1, x, x_dtype, m, y, y_dtype, nullptr, nullptr, nullptr, best_us);
+}
+
+int tlhip_autotune_pool(const tlhip_qweight_t* weights, int weight_count, const void* x, int x_dtype, int64_t m,
+                        void* y, int y_dtype, const tlhip_epilogue_t* epilogue, const tlhip_autotune_options_t* options,
+                        tlhip_stream_t stream, double* best_us) {
   TLHIP_REQUIRE_INIT();
+  if (weight_count < 1 || !weights) return set_error(TLHIP_ERR_INVALID, "autotune: no weight");
   Problem p;
-  int rc = make_problem(w, x, x_dtype, m, y, y_dtype, 1.f, nullptr, &p, "autotune");
+  int rc = make_problem(&weights[0], x, x_dtype, m, y, y_dtype, 1.f, epilogue, &p, "autotune");
   if (rc) return rc;
   if (p.m == 0 || p.n == 0 || p.k == 0) return set_error(TLHIP_ERR_INVALID, "autotune: empty problem");
-  return autotune_problem(p, best_us);
+  std::vector<WeightAlias> aliases;
+  for (int i = 0; i < weight_count; ++i) {
+    rc = validate_weight(&weights[i], "autotune");
+    if (rc) return rc;
+    if (weights[i].format != p.format || weights[i].n != p.n || weights[i].k != p.k ||
+        (p.format != TLHIP_FMT_INT8_ROW && weights[i].group_size != p.group_size))
+      return set_error(TLHIP_ERR_INVALID, "autotune: weight %d differs in format or shape from weight 0", i);
+    aliases.push_back({weights[i].packed, weights[i].scales});
+  }
+  TuneOptions o;
+  if (options) {
+    if (options->reps > 0) o.reps = options->reps;
+    if (options->batches > 0) o.batches = options->batches;
+    if (options->retime_top > 0) o.retime_top = options->retime_top;
+    if (options->warm_ms >= 0) o.warm_ms = options->warm_ms;
+    o.quick = options->quick != 0;
+    o.pool_bytes = (size_t)options->pool_bytes;
+  }
+  return autotune_problem(p, aliases, o, resolve_stream(stream), best_us);
 }
 
 int tlhip_pretune_matmul_shapes(const int64_t* mnk, int count) {
@@ -758,13 +1099,18 @@ int tlhip_tune_cache_import(const char* json) {
     parsed[key] = c;
   }
   std::lock_guard<std::mutex> lock(g_tune_mutex);
-  for (auto& kv : parsed) g_tuned[kv.first] = kv.second;
+  for (auto& kv : parsed) {
+    Problem q;
+    if (parse_problem_key(kv.first, &q)) record_winner_locked(q, kv.second);  // the shape-class level too
+    else g_tuned[kv.first] = kv.second;
+  }
   return TLHIP_OK;
 }
 
 int tlhip_tune_cache_clear(void) {
   std::lock_guard<std::mutex> lock(g_tune_mutex);
   g_tuned.clear();
+  g_class_tuned.clear();
   g_shape_hints.clear();
   return TLHIP_OK;
 }

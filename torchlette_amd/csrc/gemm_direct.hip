@@ -34,6 +34,7 @@
 //   * 4 or 8 waves per workgroup, two waves per SIMD resident.
 // MFMA-bound by design: per MFMA a wave reads 1 KB / TN from LDS and spends
 // 14 / TM VALU instructions on dequantisation.
+#include <cstring>
 #include <type_traits>
 
 #include "gemm_common.h"
@@ -330,14 +331,11 @@ int launch_direct_tile(const DirectArgs& a, bool g32, hipStream_t stream) {
   size_t lds_bytes = (size_t)(2 * BM * HROW_UNITS + BN * 4) * 16;
   const size_t patch_bytes = (size_t)WM * WN * 32 * (TN * 32 + 4) * sizeof(float);
   if (lds_bytes < patch_bytes) lds_bytes = patch_bytes;
-  if (lds_bytes > 64 * 1024)
-    TLHIP_CHECK_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
   DirectArgs b = a;
   int grid = 0;
   b.map = make_tile_map((a.m + BM - 1) / BM, (a.n + BN - 1) / BN, &grid);
   void* args[] = {(void*)&b};
-  TLHIP_CHECK_HIP(hipLaunchKernel(fn, dim3(grid), dim3(WM * WN * 64), args, lds_bytes, stream));
-  return TLHIP_OK;
+  return launch_kernel(fn, dim3(grid), dim3(WM * WN * 64), args, lds_bytes, stream);
 }
 
 struct DirectTile {
@@ -415,6 +413,24 @@ int launch_gemm_direct(const Problem& p, const tlhip_kernel_config_t& c, hipStre
   if (rc) return rc;
   TLHIP_CHECK_HIP(hipGetLastError());
   count_gemm_dispatch();
+  return TLHIP_OK;
+}
+
+// Every instance launch_gemm_direct can reach, in prepare mode (see launch_kernel).
+int prepare_gemm_direct_kernels() {
+  DirectArgs a;
+  memset(&a, 0, sizeof a);
+  a.m = a.n = 1;
+  for (bool g32 : {true, false}) {
+    int rc = launch_direct_tile<2, 2, 4, 4>(a, g32, nullptr);
+    if (!rc) rc = launch_direct_tile<2, 4, 4, 2>(a, g32, nullptr);
+    if (!rc) rc = launch_direct_tile<2, 4, 4, 1>(a, g32, nullptr);
+    if (!rc) rc = launch_direct_tile<1, 4, 4, 2>(a, g32, nullptr);
+    if (!rc) rc = launch_direct_tile<2, 4, 2, 2>(a, g32, nullptr);
+    if (!rc) rc = launch_direct_tile<2, 2, 2, 2>(a, g32, nullptr);
+    if (!rc) rc = launch_direct_tile<4, 2, 2, 2>(a, g32, nullptr);
+    if (rc) return rc;
+  }
   return TLHIP_OK;
 }
 

@@ -22,6 +22,8 @@
 // traffic only, not for the global loads in flight).
 // Epilogue: acc*alpha -> ops in order (bias indexed by n, unary) -> cast, the
 // order of applyBlockEpilogue (matmul-skeleton.ts:916-966).
+#include <cstring>
+
 #include "gemm_common.h"
 
 namespace tlhip {
@@ -239,14 +241,11 @@ int launch_tile(const GemmArgs& a, hipStream_t stream) {
   size_t lds_bytes = (size_t)2 * (BM + BN) * ROW_BYTES;
   const size_t patch_bytes = (size_t)4 * 32 * (BN / 64 * 32 + 4) * sizeof(float);
   if (lds_bytes < patch_bytes) lds_bytes = patch_bytes;
-  if (lds_bytes > 64 * 1024)
-    TLHIP_CHECK_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
   GemmArgs b = a;
   int grid = 0;
   b.map = make_tile_map((a.m + BM - 1) / BM, (a.n + BN - 1) / BN, &grid);
   void* args[] = {(void*)&b};
-  TLHIP_CHECK_HIP(hipLaunchKernel(fn, dim3(grid), dim3(256), args, lds_bytes, stream));
-  return TLHIP_OK;
+  return launch_kernel(fn, dim3(grid), dim3(256), args, lds_bytes, stream);
 }
 
 template <int FMT>
@@ -323,6 +322,21 @@ int launch_gemm(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t st
   if (rc) return rc;
   TLHIP_CHECK_HIP(hipGetLastError());
   count_gemm_dispatch();
+  return TLHIP_OK;
+}
+
+// Every instance launch_gemm can reach, in prepare mode (see launch_kernel).
+int prepare_gemm_kernels() {
+  GemmArgs a;
+  memset(&a, 0, sizeof a);
+  a.m = a.n = 1;
+  static const int tiles[][2] = {{256, 256}, {128, 256}, {256, 128}, {128, 128}, {64, 128}};
+  for (auto& t : tiles) {
+    int rc = launch_fmt<TLHIP_FMT_INT4_GROUPED>(t[0], t[1], a, nullptr);
+    if (!rc && t[0] * t[1] != 256 * 256) rc = launch_fmt<TLHIP_FMT_INT8_GROUPED>(t[0], t[1], a, nullptr);
+    if (!rc && t[0] * t[1] != 256 * 256) rc = launch_fmt<TLHIP_FMT_INT8_ROW>(t[0], t[1], a, nullptr);
+    if (rc) return rc;
+  }
   return TLHIP_OK;
 }
 

@@ -3,6 +3,8 @@
 // geometry, the single and the grouped launch.  The kernel is in gemv_kernel.h and
 // is instantiated per weight format in gemv_int4.hip, gemv_int8_grouped.hip and
 // gemv_int8_row.hip.
+#include <cstring>
+
 #include "gemv_args.h"
 
 namespace tlhip {
@@ -206,6 +208,36 @@ int launch_gemv_grouped(const Problem* ps, int count, const tlhip_kernel_config_
   if (rc) return rc;
   TLHIP_CHECK_HIP(hipGetLastError());
   for (int i = 0; i < g.count; ++i) count_gemv_dispatch();
+  return TLHIP_OK;
+}
+
+// Every instance the launch tables above can reach, in prepare mode (see launch_kernel).
+int prepare_gemv_kernels() {
+  GemvArgs a;
+  memset(&a, 0, sizeof a);
+  GroupedGemvArgs g;
+  memset(&g, 0, sizeof g);
+  g.count = 1;
+  g.first[1] = 1;
+  static const int ru[][2] = {{1, 2}, {1, 4}, {1, 8}, {2, 2}, {2, 4}, {4, 2}};
+  for (int xd : {TLHIP_F16, TLHIP_F32})
+    for (int mt : {1, 2, 4})
+      for (auto& c : ru) {
+        int rc = launch_gemv_int4(xd, mt, c[0], c[1], a, 64, 1, 0, nullptr);
+        if (!rc) rc = launch_gemv_int8_grouped(xd, mt, c[0], c[1], a, 64, 1, 0, nullptr);
+        if (!rc) rc = launch_gemv_int8_row(xd, mt, c[0], c[1], a, 64, 1, 0, nullptr);
+        if (rc) return rc;
+      }
+  for (int u : {2, 4, 8}) {
+    const int rc = launch_gemv_mf4_int4(u, a, 64, 1, 0, nullptr);
+    if (rc) return rc;
+  }
+  for (int r : {1, 2}) {
+    int rc = launch_gemv_grouped_int4(r, g, 64, 0, nullptr);
+    if (!rc) rc = launch_gemv_grouped_int8_grouped(r, g, 64, 0, nullptr);
+    if (!rc) rc = launch_gemv_grouped_int8_row(r, g, 64, 0, nullptr);
+    if (rc) return rc;
+  }
   return TLHIP_OK;
 }
 

@@ -649,11 +649,8 @@ __global__ __launch_bounds__(512) void gemv_grouped_kernel(const GroupedGemvArgs
 template <int FMT, typename XT, int MT, int R, int U, bool MF4 = false>
 int launch_t(const GemvArgs& a, int threads, int grid, size_t lds_bytes, hipStream_t stream) {
   const void* fn = (const void*)gemv_kernel<FMT, XT, MT, R, U, MF4>;
-  if (lds_bytes > 64 * 1024)
-    TLHIP_CHECK_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
   void* args[] = {(void*)&a};
-  TLHIP_CHECK_HIP(hipLaunchKernel(fn, dim3(grid), dim3(threads), args, lds_bytes, stream));
-  return TLHIP_OK;
+  return launch_kernel(fn, dim3(grid), dim3(threads), args, lds_bytes, stream);
 }
 
 // (rows per lane group, chunks in flight) pairs that are instantiated: R*U <= 8.
@@ -691,11 +688,8 @@ int launch_x(int x_dtype, int mt, int r, int u, const GemvArgs& a, int threads, 
 template <int FMT, int R>
 int launch_grouped_t(const GroupedGemvArgs& g, int threads, size_t lds_bytes, hipStream_t stream) {
   const void* fn = (const void*)gemv_grouped_kernel<FMT, _Float16, 1, R, 2>;
-  if (lds_bytes > 64 * 1024)
-    TLHIP_CHECK_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
   void* args[] = {(void*)&g};
-  TLHIP_CHECK_HIP(hipLaunchKernel(fn, dim3(g.first[g.count]), dim3(threads), args, lds_bytes, stream));
-  return TLHIP_OK;
+  return launch_kernel(fn, dim3(g.first[g.count]), dim3(threads), args, lds_bytes, stream);
 }
 
 

@@ -24,6 +24,8 @@
 // LDS; with kw = 1 a wave owns a row block alone and nothing is combined.  The
 // weight loads of all row blocks of a workgroup form one software pipeline, as
 // in the VALU kernel.
+#include <cstring>
+
 #include "gemv_mfma_common.h"
 
 namespace tlhip {
@@ -623,11 +625,8 @@ static int launch_mfma_u(int unroll, const MfmaArgs& a, int grid, int threads, s
       default: fn = (const void*)gemv_mfma_kernel<FMT, 4, WIDE, 512>; break;
     }
   }
-  if (lds_bytes > 64 * 1024)
-    TLHIP_CHECK_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
   void* args[] = {(void*)&a};
-  TLHIP_CHECK_HIP(hipLaunchKernel(fn, dim3(grid), dim3(threads), args, lds_bytes, stream));
-  return TLHIP_OK;
+  return launch_kernel(fn, dim3(grid), dim3(threads), args, lds_bytes, stream);
 }
 
 // The form with whole-line weight loads (2 or 4 iterations in flight).
@@ -637,11 +636,8 @@ static int launch_mfma_line(int unroll, const MfmaArgs& a, int grid, int threads
   if (threads > 512) fn = (const void*)gemv_mfma_kernel<FMT, 2, WIDE, 1024, true>;
   else if (unroll == 2) fn = (const void*)gemv_mfma_kernel<FMT, 2, WIDE, 512, true>;
   else fn = (const void*)gemv_mfma_kernel<FMT, 4, WIDE, 512, true>;
-  if (lds_bytes > 64 * 1024)
-    TLHIP_CHECK_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
   void* args[] = {(void*)&a};
-  TLHIP_CHECK_HIP(hipLaunchKernel(fn, dim3(grid), dim3(threads), args, lds_bytes, stream));
-  return TLHIP_OK;
+  return launch_kernel(fn, dim3(grid), dim3(threads), args, lds_bytes, stream);
 }
 
 int launch_gemv_mfma(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t stream) {
@@ -717,6 +713,27 @@ int launch_gemv_mfma(const Problem& p, const tlhip_kernel_config_t& c, hipStream
   if (rc) return rc;
   TLHIP_CHECK_HIP(hipGetLastError());
   count_gemv_dispatch();
+  return TLHIP_OK;
+}
+
+// Every instance launch_gemv_mfma can reach, in prepare mode (see launch_kernel).
+int prepare_gemv_mfma_kernels() {
+  MfmaArgs a;
+  memset(&a, 0, sizeof a);
+  for (int threads : {512, 1024})
+    for (int unroll : {1, 2, 4}) {
+      int rc = launch_mfma_u<TLHIP_FMT_INT4_GROUPED, true>(unroll, a, 1, threads, 0, nullptr);
+      if (!rc) rc = launch_mfma_u<TLHIP_FMT_INT4_GROUPED, false>(unroll, a, 1, threads, 0, nullptr);
+      if (!rc) rc = launch_mfma_u<TLHIP_FMT_INT8_GROUPED, false>(unroll, a, 1, threads, 0, nullptr);
+      if (!rc) rc = launch_mfma_u<TLHIP_FMT_INT8_ROW, false>(unroll, a, 1, threads, 0, nullptr);
+      if (unroll != 1) {
+        if (!rc) rc = launch_mfma_line<TLHIP_FMT_INT4_GROUPED, true>(unroll, a, 1, threads, 0, nullptr);
+        if (!rc) rc = launch_mfma_line<TLHIP_FMT_INT8_GROUPED, true>(unroll, a, 1, threads, 0, nullptr);
+        if (!rc) rc = launch_mfma_line<TLHIP_FMT_INT8_GROUPED, false>(unroll, a, 1, threads, 0, nullptr);
+        if (!rc) rc = launch_mfma_line<TLHIP_FMT_INT8_ROW, false>(unroll, a, 1, threads, 0, nullptr);
+      }
+      if (rc) return rc;
+    }
   return TLHIP_OK;
 }
 

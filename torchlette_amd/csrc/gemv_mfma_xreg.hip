@@ -342,12 +342,24 @@ int launch_gemv_xreg(const Problem& p, const tlhip_kernel_config_t& c, hipStream
     default: break;
   }
   if (!fn) return set_error(TLHIP_ERR_INVALID, "gemv_mfma_xreg: no kernel instance for this configuration");
-  if (geo.lds_bytes > 64 * 1024)
-    TLHIP_CHECK_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)geo.lds_bytes));
   void* args[] = {(void*)&a};
-  TLHIP_CHECK_HIP(hipLaunchKernel(fn, dim3(geo.grid), dim3(threads), args, geo.lds_bytes, stream));
+  const int rc = launch_kernel(fn, dim3(geo.grid), dim3(threads), args, geo.lds_bytes, stream);
+  if (rc) return rc;
   TLHIP_CHECK_HIP(hipGetLastError());
   count_gemv_dispatch();
+  return TLHIP_OK;
+}
+
+// Every instance launch_gemv_xreg can reach, in prepare mode (see launch_kernel).
+int prepare_gemv_xreg_kernels() {
+  const void* fns[] = {xreg_fn<1, 1>(512), xreg_fn<1, 2>(512), xreg_fn<1, 3>(512), xreg_fn<1, 4>(512), xreg_fn<1, 6>(512),
+                       xreg_fn<2, 1>(512), xreg_fn<2, 2>(512), xreg_fn<2, 3>(512), xreg_fn<1, 1>(1024),
+                       xreg_fn<1, 2>(1024), xreg_fn<2, 1>(1024)};
+  for (const void* fn : fns) {
+    if (!fn) continue;
+    const int rc = launch_kernel(fn, dim3(1), dim3(64), nullptr, 0, nullptr);
+    if (rc) return rc;
+  }
   return TLHIP_OK;
 }
 

@@ -8,6 +8,7 @@
 #include <mutex>
 #include <string>
 #include <unordered_map>
+#include <unordered_set>
 
 #include "common.h"
 
@@ -25,6 +26,7 @@ std::atomic<uint64_t> g_gemv_dispatches{0};
 std::atomic<uint64_t> g_gemm_dispatches{0};
 std::atomic<uint64_t> g_dequant_dispatches{0};
 std::atomic<uint64_t> g_autotune_runs{0};
+std::atomic<uint64_t> g_tuning_entries_loaded{0};
 }  // namespace
 
 int set_error(int code, const char* fmt, ...) {
@@ -42,15 +44,25 @@ bool is_initialised() { return g_init; }
 hipStream_t resolve_stream(tlhip_stream_t s) { return s ? static_cast<hipStream_t>(s) : g_stream; }
 
 namespace {
+// One workspace per stream.  A captured graph has the pointers of its capture stream's
+// workspace baked into its kernel arguments, so the workspace outlives the stream for as
+// long as a graph captured on it is alive: `graphs` counts those, `stream_alive` says
+// whether tlhip_stream_destroy has been called.
 struct SplitWorkspace {
   float* workspace;
   int* counters;
+  int graphs;
+  bool stream_alive;
 };
 std::mutex g_ws_mutex;
 std::unordered_map<hipStream_t, SplitWorkspace> g_workspaces;
+std::unordered_map<hipGraphExec_t, hipStream_t> g_graphs;  // live graph -> its capture stream
+std::unordered_set<hipStream_t> g_live_streams;            // the library stream and tlhip_stream_create's
 
 void free_workspaces() {
   std::lock_guard<std::mutex> lock(g_ws_mutex);
+  for (auto& kv : g_graphs) (void)hipGraphExecDestroy(kv.first);  // graphs first: they reference the workspaces
+  g_graphs.clear();
   for (auto& kv : g_workspaces) {
     (void)hipFree(kv.second.workspace);
     (void)hipFree(kv.second.counters);
@@ -58,13 +70,21 @@ void free_workspaces() {
   g_workspaces.clear();
 }
 
+// Caller holds g_ws_mutex.
+void release_if_unused(hipStream_t stream) {
+  auto it = g_workspaces.find(stream);
+  if (it == g_workspaces.end() || it->second.stream_alive || it->second.graphs > 0) return;
+  (void)hipFree(it->second.workspace);
+  (void)hipFree(it->second.counters);
+  g_workspaces.erase(it);
+}
+
 void free_workspace_of(hipStream_t stream) {
   std::lock_guard<std::mutex> lock(g_ws_mutex);
   auto it = g_workspaces.find(stream);
   if (it == g_workspaces.end()) return;
-  (void)hipFree(it->second.workspace);
-  (void)hipFree(it->second.counters);
-  g_workspaces.erase(it);
+  it->second.stream_alive = false;
+  release_if_unused(stream);
 }
 }  // namespace
 
@@ -78,7 +98,7 @@ int split_workspace(hipStream_t stream, float** workspace, int** counters) {
       return set_error(TLHIP_ERR_STATE,
                        "split-K workspace of this stream does not exist yet and cannot be created during "
                        "capture: run the same call once on this stream before capturing");
-    SplitWorkspace w{nullptr, nullptr};
+    SplitWorkspace w{nullptr, nullptr, 0, true};
     TLHIP_CHECK_HIP(hipMalloc((void**)&w.workspace, kSplitWorkspaceFloats * sizeof(float)));
     hipError_t e = hipMalloc((void**)&w.counters, kSplitCounters * sizeof(int));
     if (e == hipSuccess) e = hipMemset(w.counters, 0, kSplitCounters * sizeof(int));
@@ -92,6 +112,48 @@ int split_workspace(hipStream_t stream, float** workspace, int** counters) {
   *workspace = it->second.workspace;
   *counters = it->second.counters;
   return TLHIP_OK;
+}
+
+namespace {
+thread_local bool t_prepare_mode = false;
+std::mutex g_lds_mutex;
+std::unordered_set<const void*> g_lds_raised;
+
+// Raises fn's dynamic-LDS limit to what the hardware leaves next to its static LDS, once.
+int ensure_max_lds(const void* fn) {
+  std::lock_guard<std::mutex> lock(g_lds_mutex);
+  if (g_lds_raised.count(fn)) return TLHIP_OK;
+  hipFuncAttributes attr;
+  TLHIP_CHECK_HIP(hipFuncGetAttributes(&attr, fn));
+  const int limit = 160 * 1024 - (int)attr.sharedSizeBytes;
+  TLHIP_CHECK_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, limit));
+  g_lds_raised.insert(fn);
+  return TLHIP_OK;
+}
+}  // namespace
+
+bool prepare_mode() { return t_prepare_mode; }
+
+int launch_kernel(const void* fn, dim3 grid, dim3 block, void** args, size_t lds_bytes, hipStream_t stream) {
+  if (t_prepare_mode) return ensure_max_lds(fn);
+  if (lds_bytes > 64 * 1024) {
+    // already raised at tlhip_init; this is a set lookup
+    const int rc = ensure_max_lds(fn);
+    if (rc) return rc;
+  }
+  TLHIP_CHECK_HIP(hipLaunchKernel(fn, grid, block, args, lds_bytes, stream));
+  return TLHIP_OK;
+}
+
+int prepare_all_kernels() {
+  t_prepare_mode = true;
+  int rc = prepare_gemv_kernels();
+  if (!rc) rc = prepare_gemv_mfma_kernels();
+  if (!rc) rc = prepare_gemv_xreg_kernels();
+  if (!rc) rc = prepare_gemm_kernels();
+  if (!rc) rc = prepare_gemm_direct_kernels();
+  t_prepare_mode = false;
+  return rc;
 }
 
 int problem_scratch(const Problem& p, hipStream_t stream, float** workspace, int** counters) {
@@ -109,6 +171,7 @@ void count_gemv_dispatch() { g_gemv_dispatches++; }
 void count_gemm_dispatch() { g_gemm_dispatches++; }
 void count_dequant_dispatch() { g_dequant_dispatches++; }
 void count_autotune_run() { g_autotune_runs++; }
+void count_tuning_entries_loaded(int n) { g_tuning_entries_loaded += (uint64_t)(n > 0 ? n : 0); }
 
 }  // namespace tlhip
 
@@ -140,9 +203,14 @@ int tlhip_init(int device_index) {
   }
   // Default priority only: mixed stream priorities are not used anywhere.
   TLHIP_CHECK_HIP(hipStreamCreateWithFlags(&g_stream, hipStreamNonBlocking));
+  {
+    std::lock_guard<std::mutex> ws_lock(g_ws_mutex);
+    g_live_streams.insert(g_stream);
+  }
   g_device = device_index;
   g_init = true;
-  const int rc = noalloc_setup(device_index);
+  int rc = noalloc_setup(device_index);
+  if (!rc) rc = prepare_all_kernels();
   if (rc) {
     (void)hipStreamDestroy(g_stream);
     g_stream = nullptr;
@@ -150,6 +218,7 @@ int tlhip_init(int device_index) {
     g_device = -1;
     return rc;
   }
+  count_tuning_entries_loaded(load_default_tuning());
   clear_error();
   return TLHIP_OK;
 }
@@ -159,10 +228,18 @@ int tlhip_shutdown(void) {
   if (!g_init) return TLHIP_OK;
   (void)hipStreamSynchronize(g_stream);
   free_workspaces();
+  {
+    std::lock_guard<std::mutex> ws_lock(g_ws_mutex);
+    g_live_streams.clear();
+  }
   (void)hipStreamDestroy(g_stream);
   g_stream = nullptr;
   g_init = false;
   g_device = -1;
+  {
+    std::lock_guard<std::mutex> lds_lock(g_lds_mutex);
+    g_lds_raised.clear();
+  }
   return TLHIP_OK;
 }
 
@@ -202,6 +279,12 @@ int tlhip_free(void* ptr) {
 int tlhip_memset(void* ptr, int value, size_t bytes, tlhip_stream_t stream) {
   TLHIP_REQUIRE_INIT();
   if (bytes == 0) return TLHIP_OK;
+  // not into a graph: memset nodes have given wrong results on replays after the first
+  hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+  TLHIP_CHECK_HIP(hipStreamIsCapturing(resolve_stream(stream), &status));
+  if (status != hipStreamCaptureStatusNone)
+    return set_error(TLHIP_ERR_STATE, "tlhip_memset: the stream is being captured; clear memory before the capture "
+                                      "or with a kernel");
   TLHIP_CHECK_HIP(hipMemsetAsync(ptr, value, bytes, resolve_stream(stream)));
   return TLHIP_OK;
 }
@@ -246,6 +329,10 @@ int tlhip_stream_create(tlhip_stream_t* out) {
   if (!out) return set_error(TLHIP_ERR_INVALID, "tlhip_stream_create: null output");
   hipStream_t s;
   TLHIP_CHECK_HIP(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+  {
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    g_live_streams.insert(s);
+  }
   *out = s;
   return TLHIP_OK;
 }
@@ -255,6 +342,10 @@ int tlhip_stream_destroy(tlhip_stream_t stream) {
   if (!stream) return TLHIP_OK;
   TLHIP_CHECK_HIP(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
   free_workspace_of(static_cast<hipStream_t>(stream));
+  {
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    g_live_streams.erase(static_cast<hipStream_t>(stream));
+  }
   TLHIP_CHECK_HIP(hipStreamDestroy(static_cast<hipStream_t>(stream)));
   return TLHIP_OK;
 }
@@ -311,12 +402,19 @@ int tlhip_graph_begin_capture(tlhip_stream_t stream) {
 int tlhip_graph_end_capture(tlhip_stream_t stream, tlhip_graph_t* out) {
   TLHIP_REQUIRE_INIT();
   if (!out) return set_error(TLHIP_ERR_INVALID, "tlhip_graph_end_capture: null output");
+  hipStream_t s = resolve_stream(stream);
   hipGraph_t graph = nullptr;
-  TLHIP_CHECK_HIP(hipStreamEndCapture(resolve_stream(stream), &graph));
+  TLHIP_CHECK_HIP(hipStreamEndCapture(s, &graph));
   hipGraphExec_t exec = nullptr;
   hipError_t e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
   (void)hipGraphDestroy(graph);
   if (e != hipSuccess) return set_error(TLHIP_ERR_DEVICE, "hipGraphInstantiate failed: %s", hipGetErrorString(e));
+  {
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    g_graphs[exec] = s;
+    auto it = g_workspaces.find(s);
+    if (it != g_workspaces.end()) it->second.graphs++;
+  }
   *out = exec;
   return TLHIP_OK;
 }
@@ -324,14 +422,47 @@ int tlhip_graph_end_capture(tlhip_stream_t stream, tlhip_graph_t* out) {
 int tlhip_graph_launch(tlhip_graph_t graph, tlhip_stream_t stream) {
   TLHIP_REQUIRE_INIT();
   if (!graph) return set_error(TLHIP_ERR_INVALID, "tlhip_graph_launch: null graph");
-  TLHIP_CHECK_HIP(hipGraphLaunch(static_cast<hipGraphExec_t>(graph), resolve_stream(stream)));
+  hipStream_t s = resolve_stream(stream);
+  {
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    auto it = g_graphs.find(static_cast<hipGraphExec_t>(graph));
+    if (it == g_graphs.end()) return set_error(TLHIP_ERR_INVALID, "tlhip_graph_launch: unknown or destroyed graph");
+    // the captured kernels use the capture stream's K-slice workspace; on another stream a
+    // replay could run next to that stream's own launches on the same tiles and counters
+    if (it->second != s)
+      return set_error(TLHIP_ERR_INVALID, "tlhip_graph_launch: a graph replays on the stream it was captured on");
+  }
+  TLHIP_CHECK_HIP(hipGraphLaunch(static_cast<hipGraphExec_t>(graph), s));
   return TLHIP_OK;
 }
 
 int tlhip_graph_destroy(tlhip_graph_t graph) {
   TLHIP_REQUIRE_INIT();
   if (!graph) return TLHIP_OK;
-  TLHIP_CHECK_HIP(hipGraphExecDestroy(static_cast<hipGraphExec_t>(graph)));
+  hipGraphExec_t exec = static_cast<hipGraphExec_t>(graph);
+  hipStream_t origin = nullptr;
+  {
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    auto it = g_graphs.find(exec);
+    if (it == g_graphs.end()) return TLHIP_OK;  // idempotent, like destroy() in the reference
+    origin = it->second;
+    g_graphs.erase(it);
+  }
+  // a replay may still be in flight on the capture stream (the library stream is never destroyed
+  // before shutdown; a caller's stream that is already gone has been synchronised by its destroy)
+  bool alive;
+  {
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    alive = g_live_streams.count(origin) != 0;
+  }
+  if (alive) (void)hipStreamSynchronize(origin);
+  TLHIP_CHECK_HIP(hipGraphExecDestroy(exec));
+  std::lock_guard<std::mutex> lock(g_ws_mutex);
+  auto w = g_workspaces.find(origin);
+  if (w != g_workspaces.end() && w->second.graphs > 0) {
+    w->second.graphs--;
+    release_if_unused(origin);
+  }
   return TLHIP_OK;
 }
 
@@ -341,6 +472,7 @@ uint64_t tlhip_counter(const char* name) {
   if (!strcmp(name, "quant_gemm_dispatches")) return g_gemm_dispatches.load();
   if (!strcmp(name, "dequant_dispatches")) return g_dequant_dispatches.load();
   if (!strcmp(name, "autotune_runs")) return g_autotune_runs.load();
+  if (!strcmp(name, "tuning_entries_loaded")) return g_tuning_entries_loaded.load();
   return 0;
 }
 
