@@ -234,6 +234,14 @@ typedef struct {
 } tlhip_gemv_problem_t;
 int tlhip_gemv_grouped(const tlhip_gemv_problem_t* problems, int count, int x_dtype, int y_dtype, float alpha,
                        tlhip_stream_t stream);
+/* The same for a batched decode step: every problem has `m` (<= 16) activation rows.
+ * Problems that share ONE activation pointer (q/k/v on the normed hidden state,
+ * gate/up; packages/qwen3-browser/src/model.ts:341-361) run as one launch of the
+ * matrix-core kernels when the configuration selected for their combined rows is one of
+ * theirs (variants gemv_mfma and gemv_mfma_xreg: f16 activations); anything else runs as
+ * separate launches (m = 1: as the VALU kernel's grouped launch).  Results are those of `count` tlhip_gemv calls. */
+int tlhip_gemv_grouped_rows(const tlhip_gemv_problem_t* problems, int count, int x_dtype, int64_t m,
+                            int y_dtype, float alpha, tlhip_stream_t stream);
 
 /* Prefill GEMM with dequant fused into the LDS stage: same contract as
  * tlhip_gemv for any m >= 1; x must be f16.  Stands in for the explicit
@@ -331,7 +339,10 @@ int tlhip_topk(const float* logits, int64_t offset, int64_t length, int k, float
  * 128x256 1x4),
  * 4 = "gemv_mfma_xreg" (skinny MFMA for int4 g32 with the activations held in
  * registers: p0 waves per workgroup, p1 iterations in flight, p2 workgroups per
- * CU, p3 K slices across workgroups).  Unused fields are 0. */
+ * CU, p3 K slices across workgroups, p4 = 1: every weight load of a wave issued
+ * before the first is consumed (at most 4 row blocks per workgroup), p5 = 1: a
+ * workgroup barrier between the activation loads and the weight loads).  Unused
+ * fields are 0. */
 typedef struct {
   int32_t variant;
   int32_t p0; /* gemv: lanes per row (16/32/64)   gemv_mfma: waves per workgroup   tiled: tile M */

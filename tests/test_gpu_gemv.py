@@ -465,10 +465,65 @@ def test_grouped_gemv_rejects_mixed_shapes(be):
     assert outs[0].numpy().shape == (1, 64)
     with pytest.raises(ValueError, match="1..4"):
         be.linearGrouped(x, [w1] * 5)
-    x2 = be.ops.tensorFromArray(make_x(2, 256, "f16", rng), [2, 256], "f16")
-    with pytest.raises(ValueError, match="one f16 activation row"):
-        be.linearGrouped(x2, [w1])
+    x17 = be.ops.tensorFromArray(make_x(17, 256, "f16", rng), [17, 256], "f16")
+    with pytest.raises(ValueError, match="1..16 rows"):
+        be.linearGrouped(x17, [w1])
     del w2
+
+
+@pytest.mark.parametrize("m", [2, 4, 8, 16])
+@pytest.mark.parametrize("fmt,g,k,ns,cfg", [
+    ("int4-grouped", 32, 4096, [1024, 256, 256], None),                 # q, k, v: whatever is selected for their sum
+    ("int4-grouped", 32, 2048, [1000, 37, 515, 2048], (1, 8, 2, 8, 1)),    # ragged N, four problems, LDS-staged matrix-core kernel
+    ("int4-grouped", 32, 2048, [3072, 3072], (1, 8, 2, 4, 2, 0, 1)),        # gate, up: K slices across workgroups, whole-line loads
+    ("int4-grouped", 32, 2048, [1536, 512], (4, 8, 2, 1, 1)),           # activations in registers
+    ("int4-grouped", 32, 2048, [1536, 520], (4, 8, 1, 1, 2, 1, 1)),     # ... every load upfront, K slices, barrier
+    ("int8-row", 0, 2304, [1000, 515], (1, 8, 2, 1, 1, 0, 1)),
+    ("int8-grouped", 64, 2048, [768, 512], (1, 4, 2, 4, 1)),
+])
+def test_grouped_batched_decode_equals_the_oracle_and_separate_launches(be, fmt, g, k, ns, cfg, m):
+    """q/k/v (or gate/up) of a batched decode step (M <= 16 rows on the same activations)
+    in one launch of a matrix-core kernel: per problem within tolerance of the oracle, and
+    bit-identical to the same configuration launched on that problem alone wherever the
+    per-row-block arithmetic does not depend on the launch geometry (no K split across
+    waves of different workgroups)."""
+    rng = np.random.default_rng(sum(ns) + k + m)
+    x = make_x(m, k, "f16", rng)
+    xt = be.ops.tensorFromArray(x, [m, k], "f16")
+    ws, deqs, biases, bts = [], [], [], []
+    for n in ns:
+        packed, scales, deq = make_weight(fmt, n, k, g, rng)
+        ws.append(be.createQuantizedWeight(packed, scales, n, k, T.resolveWeightFormat(fmt_name(fmt, g), "f32")))
+        deqs.append(deq)
+        b = rng.standard_normal(n).astype(np.float32)
+        biases.append(b)
+        bts.append(be.ops.tensorFromArray(b, [n], "f32"))
+    # the group is chosen like ONE problem with all the rows: seed that problem's winner
+    total = be.createQuantizedWeight(np.zeros(sum(ns) * k // (8 if fmt.startswith("int4") else 4), np.uint32),
+                                     np.zeros(sum(ns) * (k // g if g else 1), np.float32 if fmt == "int8-row" else np.uint16),
+                                     sum(ns), k, T.resolveWeightFormat(fmt_name(fmt, g), "f32"))
+    saved = T.exportTuningCache()
+    try:
+        if cfg is not None:
+            be.seedPerShapeMatmulChoice(total, "f16", m, "f32", L.KernelConfig.of(*cfg))
+        sel = be.selectedConfig(total, "f16", m, "f32")
+        before = T.getQuantGemvDispatchCount()
+        outs = be.linearGrouped(xt, ws, bts, "silu")
+        assert T.getQuantGemvDispatchCount() == before + len(ns)
+        for w, bt, b, deq, o in zip(ws, bts, biases, deqs, outs):
+            got = o.numpy()
+            want = O.linear(x.astype(np.float32), deq, b, "silu")
+            assert got.shape == want.shape
+            assert rel_l2(got, want) <= 2e-6, (sel.as_tuple(), rel_l2(got, want))
+            if cfg is not None:
+                try:
+                    sep = be.linear(xt, w, bt, "silu", fused=True, config=L.KernelConfig.of(*cfg)).numpy()
+                except L.TlhipError:
+                    continue  # the configuration fits the group's rows but not this problem's alone
+                assert np.array_equal(got, sep), sel.as_tuple()
+    finally:
+        T.clearTuningCache()
+        T.importTuningCache(saved)
 
 
 def test_k_slices_are_stable_over_many_back_to_back_launches(be):

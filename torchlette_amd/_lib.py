@@ -119,6 +119,7 @@ SIGNATURES = {
     "tlhip_gemv": (_i, [_QW, _vp, _i, _i64, _vp, _i, _f, _EP, _vp]),
     "tlhip_gemv_noalloc": (_i, [_QW, _vp, _i, _i64, _vp, _i, _f, _EP, _vp]),
     "tlhip_gemv_grouped": (_i, [C.POINTER(GemvProblem), _i, _i, _i, _f, _vp]),
+    "tlhip_gemv_grouped_rows": (_i, [C.POINTER(GemvProblem), _i, _i, _i64, _i, _f, _vp]),
     "tlhip_gemv_prologue": (_i, [_QW, C.POINTER(Prologue), _vp, _i, _i64, _vp, _i, _f, _EP, _vp]),
     "tlhip_gemv_grouped_prologue": (_i, [C.POINTER(GemvProblem), _i, C.POINTER(Prologue), _i, _i, _f, _vp]),
     "tlhip_rmsnorm": (_i, [_vp, _i, _vp, _vp, _i, _i64, _i64, _f, _vp]),

@@ -545,16 +545,17 @@ class HipBackend:
     def linearGrouped(self, input: HipTensor, weights: Sequence[HipTensor],
                       biases: Optional[Sequence[Optional[HipTensor]]] = None,
                       activation: Optional[str] = None, _prologue: Optional[L.Prologue] = None) -> List[HipTensor]:
-        """Up to four decode Linears on the same activation row (q/k/v, or gate/up)
-        in one launch: the results of ``[linear(input, w, b, activation, fused=True)
-        for w, b in zip(weights, biases)]``.  M = 1 and f16 activations."""
+        """Up to four decode Linears on the same activations (q/k/v, or gate/up) in
+        one launch: the results of ``[linear(input, w, b, activation, fused=True)
+        for w, b in zip(weights, biases)]``.  f16 activations, at most 16 rows (with a
+        prologue: one row)."""
         if not 1 <= len(weights) <= 4:
             raise ValueError("linearGrouped: a group holds 1..4 weights")
         biases = list(biases) if biases is not None else [None] * len(weights)
         qws = [self._qweight(w, transposed=False) for w in weights]
         m = input.size // qws[0].k
-        if m != 1 or input.dtype != "f16":
-            raise ValueError("linearGrouped: one f16 activation row")
+        if input.dtype != "f16" or not 1 <= m <= 16 or (m != 1 and _prologue is not None):
+            raise ValueError("linearGrouped: f16 activations, 1..16 rows (one row with a prologue)")
         out_dtype = "f16" if all(w.format.elementType == "f16" for w in weights) else "f32"
         outs = [self._alloc(list(input.shape[:-1]) + [qw.n], out_dtype) for qw in qws]
         eps = [self.makeEpilogue(b, activation) for b in biases]
@@ -568,7 +569,7 @@ class HipBackend:
             L.call("tlhip_gemv_grouped_prologue", probs, len(weights), C.byref(_prologue), _DT_CODE[input.dtype],
                    _DT_CODE[out_dtype], 1.0, self.stream)
         else:
-            L.call("tlhip_gemv_grouped", probs, len(weights), _DT_CODE[input.dtype], _DT_CODE[out_dtype], 1.0,
+            L.call("tlhip_gemv_grouped_rows", probs, len(weights), _DT_CODE[input.dtype], m, _DT_CODE[out_dtype], 1.0,
                    self.stream)
         return outs
 

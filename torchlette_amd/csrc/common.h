@@ -91,8 +91,13 @@ bool gemv_group_compatible(const Problem* ps, int count, const tlhip_kernel_conf
 int launch_gemv_grouped(const Problem* ps, int count, const tlhip_kernel_config_t& c, hipStream_t stream);
 bool gemv_mfma_config_applicable(const Problem& p, const tlhip_kernel_config_t& c, const char** why);
 int launch_gemv_mfma(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t stream);
+bool gemv_mfma_group_applicable(const Problem* ps, int count, const tlhip_kernel_config_t& c, const char** why);
+int launch_gemv_mfma_group(const Problem* ps, int count, const tlhip_kernel_config_t& c, hipStream_t stream);
 bool gemv_xreg_config_applicable(const Problem& p, const tlhip_kernel_config_t& c, const char** why);
 int launch_gemv_xreg(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t stream);
+// up to 4 problems that share activations, rows and shape class in one launch
+bool gemv_xreg_group_applicable(const Problem* ps, int count, const tlhip_kernel_config_t& c, const char** why);
+int launch_gemv_xreg_group(const Problem* ps, int count, const tlhip_kernel_config_t& c, hipStream_t stream);
 bool gemm_config_applicable(const Problem& p, const tlhip_kernel_config_t& c, const char** why);
 int launch_gemm(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t stream);
 bool gemm_direct_config_applicable(const Problem& p, const tlhip_kernel_config_t& c, const char** why);

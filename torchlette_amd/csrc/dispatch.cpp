@@ -147,7 +147,7 @@ tlhip_kernel_config_t mfma_cfg(int waves, int unroll, int kw, int ks = 1) {
   return c;
 }
 
-tlhip_kernel_config_t xreg_cfg(int waves, int unroll, int per_cu, int ks) {
+tlhip_kernel_config_t xreg_cfg(int waves, int unroll, int per_cu, int ks, int upfront = 0, int xbar = 0) {
   tlhip_kernel_config_t c;
   memset(&c, 0, sizeof c);
   c.variant = VARIANT_GEMV_XREG;
@@ -155,6 +155,8 @@ tlhip_kernel_config_t xreg_cfg(int waves, int unroll, int per_cu, int ks) {
   c.p1 = unroll;
   c.p2 = per_cu;
   c.p3 = ks;
+  c.p4 = upfront;
+  c.p5 = xbar;
   return c;
 }
 
@@ -285,10 +287,12 @@ std::vector<tlhip_kernel_config_t> candidates(const Problem& p) {
     for (int waves : {4, 8, 16})
       for (int unroll : {1, 2})
         for (int per_cu : {1, 2})
-          for (int ks : {1, 2, 4, 8, 16}) {
-            tlhip_kernel_config_t c = xreg_cfg(waves, unroll, per_cu, ks);
-            if (gemv_xreg_config_applicable(p, c, nullptr)) out.push_back(c);
-          }
+          for (int ks : {1, 2, 4, 8, 16})
+            for (int upfront : {0, 1})
+              for (int xbar : {0, 1}) {
+                tlhip_kernel_config_t c = xreg_cfg(waves, unroll, per_cu, ks, upfront, xbar);
+                if (gemv_xreg_config_applicable(p, c, nullptr)) out.push_back(c);
+              }
   }
   if (p.x_dtype == TLHIP_F16 && p.m >= 16) {
     static const int tiles[][5] = {
@@ -427,6 +431,8 @@ std::vector<tlhip_kernel_config_t> neighbour_candidates(const Problem& p, const 
       vary(1, {1, 2});
       vary(2, {1, 2});
       vary(3, {1, 2, 4, 8, 16});
+      vary(4, {0, 1});
+      vary(5, {0, 1});
       break;
     default:
       for (const auto& c : candidates(p))
@@ -776,27 +782,55 @@ int tlhip_gemv(const tlhip_qweight_t* w, const void* x, int x_dtype, int64_t m, 
 
 int tlhip_gemv_grouped(const tlhip_gemv_problem_t* problems, int count, int x_dtype, int y_dtype, float alpha,
                        tlhip_stream_t stream) {
+  return tlhip_gemv_grouped_rows(problems, count, x_dtype, 1, y_dtype, alpha, stream);
+}
+
+int tlhip_gemv_grouped_rows(const tlhip_gemv_problem_t* problems, int count, int x_dtype, int64_t m, int y_dtype,
+                            float alpha, tlhip_stream_t stream) {
   TLHIP_REQUIRE_INIT();
   if (count < 0 || (count > 0 && !problems)) return set_error(TLHIP_ERR_INVALID, "gemv_grouped: bad problem list");
   if (count > 4) return set_error(TLHIP_ERR_INVALID, "gemv_grouped: a group holds at most 4 problems, got %d", count);
+  if (m < 0 || m > 16) return set_error(TLHIP_ERR_INVALID, "gemv_grouped: M=%lld outside 0..16", (long long)m);
   Problem ps[4];
   for (int i = 0; i < count; ++i) {
-    int rc = make_problem(&problems[i].w, problems[i].x, x_dtype, 1, problems[i].y, y_dtype, alpha,
+    int rc = make_problem(&problems[i].w, problems[i].x, x_dtype, m, problems[i].y, y_dtype, alpha,
                           problems[i].epilogue, &ps[i], "gemv_grouped");
     if (rc) return rc;
   }
-  if (count == 0) return TLHIP_OK;
+  if (count == 0 || m == 0) return TLHIP_OK;
   hipStream_t s = resolve_stream(stream);
-  // the configuration of the largest problem, in its grouped form when there is one
-  int big = 0;
-  for (int i = 1; i < count; ++i)
-    if (ps[i].n > ps[big].n) big = i;
-  // (one grouped launch of the VALU kernel beats separate launches of whichever kernel is
-  // fastest for a single problem: every launch costs 2-3 us)
-  const tlhip_kernel_config_t c = grouped_config(ps[big]);
-  if (count > 1 && gemv_group_compatible(ps, count, c, nullptr)) return launch_gemv_grouped(ps, count, c, s);
+  if (m == 1 && count > 1) {
+    // one activation row: the configuration of the largest problem, in the VALU kernel's
+    // grouped form (one grouped launch beats separate launches of whichever kernel is
+    // fastest for a single problem: every launch costs 2-3 us)
+    int big = 0;
+    for (int i = 1; i < count; ++i)
+      if (ps[i].n > ps[big].n) big = i;
+    const tlhip_kernel_config_t c = grouped_config(ps[big]);
+    if (gemv_group_compatible(ps, count, c, nullptr)) return launch_gemv_grouped(ps, count, c, s);
+  }
+  if (count > 1) {
+    // Problems on the SAME activations (q/k/v, gate/up): one launch of a matrix-core
+    // kernel, chosen as for one problem with all the rows (its tuned winner, or the winner
+    // of the nearest tuned problem of its class).
+    bool shared = true;
+    int64_t rows = 0;
+    for (int i = 0; i < count; ++i) {
+      shared = shared && ps[i].x == ps[0].x && ps[i].k == ps[0].k;
+      rows += ps[i].n;
+    }
+    if (shared && rows > 0) {
+      Problem all = ps[0];
+      all.n = rows;
+      tlhip_kernel_config_t c = select_config(all);
+      if (c.variant == VARIANT_GEMV_MFMA && gemv_mfma_group_applicable(ps, count, c, nullptr))
+        return launch_gemv_mfma_group(ps, count, c, s);
+      if (c.variant == VARIANT_GEMV_XREG && gemv_xreg_group_applicable(ps, count, c, nullptr))
+        return launch_gemv_xreg_group(ps, count, c, s);
+    }
+  }
   for (int i = 0; i < count; ++i) {
-    int rc = matmul_with(ps[i], select_config(ps[i]), s);
+    int rc = matmul_with(ps[i], select_gemv_config(ps[i]), s);
     if (rc) return rc;
   }
   return TLHIP_OK;

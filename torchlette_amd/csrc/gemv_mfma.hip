@@ -31,14 +31,25 @@
 namespace tlhip {
 namespace {
 
-struct MfmaArgs {
+// Up to four problems that share their activations (q/k/v, gate/up of a decode step) run
+// as one launch: their 16-row blocks form one index space, a row block finds its problem
+// through this table.
+constexpr int kMfmaMaxGroup = 4;
+struct MfmaProblem {
   const u32x4* packed;
   const void* scales;
-  const _Float16* x;
   void* y;
+  int64_t n;
+  int first_block;  // index of this problem's first 16-row block in the launch's block space
+  DevEpilogue epi;
+};
+
+struct MfmaArgs {
+  MfmaProblem p[kMfmaMaxGroup];
+  int count;
+  const _Float16* x;
   float* workspace;   // split-K partial tiles: [(row block * ks + slice) * 256]
   int* counters;      // split-K arrival counters, one per row block; zero between launches
-  int64_t n;
   int k;
   int m;
   int nchunks;        // 16-byte chunks per weight row
@@ -52,12 +63,11 @@ struct MfmaArgs {
   int kw_shift;
   int blocks_per_wg;  // 16-row blocks a workgroup works on at a time = waves / kw
   int nsteps;         // batches (U consecutive iterations each) per row block per wave
-  int nblocks;        // 16-row blocks
+  int nblocks;        // 16-row blocks of all problems together
   int nwgblocks;      // ceil(nblocks / blocks_per_wg)
   float alpha;
   float scale_mul;
   int y_dtype;
-  DevEpilogue epi;
   int patch_unit;     // whole-line form: first 16-byte LDS unit of the waves' patches
 };
 
@@ -144,20 +154,31 @@ __global__ __launch_bounds__(MAXT) void gemv_mfma_kernel(const MfmaArgs a) {
   };
   const int nbatches = a.slice_iters / U;  // U divides the iterations of a slice
 
+  // row block of the launch -> its problem (wave-uniform)
+  auto problem_of = [&](int rb) {
+    int pi = 0;
+#pragma unroll
+    for (int j = 1; j < kMfmaMaxGroup; ++j)
+      if (j < a.count && rb >= a.p[j].first_block) pi = j;
+    return pi;
+  };
+
   auto load_batch = [&](Batch& b, int wb, int step) {
     const int rb = min(wb * a.blocks_per_wg + bw_idx, a.nblocks - 1);
-    const int64_t row = min((int64_t)rb * 16 + nl, a.n - 1);
-    const u32x4* wrow = a.packed + row * a.nchunks;
-    const uint16_t* srow = (const uint16_t*)a.scales + row * a.groups_per_row;
+    const MfmaProblem& P = a.p[problem_of(rb)];
+    const int64_t r0 = (int64_t)(rb - P.first_block) * 16;  // first row of the block inside its problem
+    const int64_t row = min(r0 + nl, P.n - 1);
+    const u32x4* wrow = P.packed + row * a.nchunks;
+    const uint16_t* srow = (const uint16_t*)P.scales + row * a.groups_per_row;
     const int itb = it_begin + min(kw_idx + step * a.kw, nbatches - 1) * U;
     if constexpr (LINE) {
       // pair p of the batch = 128 k = one line per row: rows 0..7 of the block in
       // register 2p, rows 8..15 in register 2p+1, lane = 8 * row + 16-byte chunk
       const int r8 = lane >> 3, c8 = lane & 7;
-      const int64_t row_lo = min((int64_t)rb * 16 + r8, a.n - 1);
-      const int64_t row_hi = min((int64_t)rb * 16 + 8 + r8, a.n - 1);
-      const u32x4* wlo = a.packed + row_lo * a.nchunks + c8;
-      const u32x4* whi = a.packed + row_hi * a.nchunks + c8;
+      const int64_t row_lo = min(r0 + r8, P.n - 1);
+      const int64_t row_hi = min(r0 + 8 + r8, P.n - 1);
+      const u32x4* wlo = P.packed + row_lo * a.nchunks + c8;
+      const u32x4* whi = P.packed + row_hi * a.nchunks + c8;
 #pragma unroll
       for (int p2 = 0; p2 < U / 2; ++p2) {
         b.w[2 * p2] = __builtin_nontemporal_load(wlo + (itb + 2 * p2) * 4);
@@ -337,16 +358,17 @@ __global__ __launch_bounds__(MAXT) void gemv_mfma_kernel(const MfmaArgs a) {
       }
     }
     if (owner) {
-      const int64_t orow = (int64_t)rb * 16 + nl;
-      if (orow < a.n) {
+      const MfmaProblem& P = a.p[problem_of(rb)];
+      const int64_t orow = (int64_t)(rb - P.first_block) * 16 + nl;
+      if (orow < P.n) {
         float rs = a.scale_mul * a.alpha;
-        if (!GROUPED) rs *= ((const float*)a.scales)[orow];
+        if (!GROUPED) rs *= ((const float*)P.scales)[orow];
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const int m = 4 * g + r;
           if (m < mrows) {
-            const float v = apply_epilogue(a.epi, t[r] * rs, orow);
-            store_out(a.y, a.y_dtype, (int64_t)m * a.n + orow, v);
+            const float v = apply_epilogue(P.epi, t[r] * rs, orow);
+            store_out(P.y, a.y_dtype, (int64_t)m * P.n + orow, v);
           }
         }
       }
@@ -526,9 +548,8 @@ struct MfmaGeometry {
   size_t lds_bytes;
   size_t patch_offset;  // bytes of activations and parked tiles in front of the patches
 };
-static bool mfma_geometry(int64_t n, int64_t k, int64_t m, int waves, int kw, int ks, size_t patch_bytes, MfmaGeometry* out) {
+static bool mfma_geometry(int64_t nblocks, int64_t k, int64_t m, int waves, int kw, int ks, size_t patch_bytes, MfmaGeometry* out) {
   const int threads = waves * 64;
-  const int64_t nblocks = (n + 15) / 16;
   const int blocks_per_wg = waves / kw;
   const int64_t nwgblocks = (nblocks + blocks_per_wg - 1) / blocks_per_wg;
   const size_t x_bytes = (size_t)m * (k / ks * 2 + 16);
@@ -560,7 +581,8 @@ static size_t line_patch_bytes(const tlhip_kernel_config_t& c) {
   return c.p5 == 1 ? (size_t)c.p0 * c.p1 * 1024 : 0;
 }
 
-bool gemv_mfma_config_applicable(const Problem& p, const tlhip_kernel_config_t& c, const char** why) {
+// `nblocks`: 16-row blocks of the launch (of all problems of a group together).
+static bool mfma_applicable(const Problem& p, int64_t nblocks, const tlhip_kernel_config_t& c, const char** why) {
   static const char* reasons[] = {
       "not the gemv_mfma variant",
       "waves per workgroup must be 4, 8 or 16 (16: at most two iterations in flight)",
@@ -603,13 +625,33 @@ bool gemv_mfma_config_applicable(const Problem& p, const tlhip_kernel_config_t& 
     if (!(c.p5 == 1 && fmt_ok && (c.p1 == 2 || c.p1 == 4) && (iters / ks) % 2 == 0)) return fail(12);
   }
   MfmaGeometry geo;
-  if (!mfma_geometry(p.n, p.k, p.m, c.p0, kw, ks, line_patch_bytes(c), &geo)) return fail(8);
+  if (!mfma_geometry(nblocks, p.k, p.m, c.p0, kw, ks, line_patch_bytes(c), &geo)) return fail(8);
   if ((iters / ks) % c.p1 != 0) return fail(11);
-  if (ks > 1) {
-    const int64_t nblocks = (p.n + 15) / 16;
-    if (nblocks > scratch_counters(p) || (size_t)nblocks * ks * 256 > scratch_tile_floats(p)) return fail(10);
-  }
+  if (ks > 1 && (nblocks > scratch_counters(p) || (size_t)nblocks * ks * 256 > scratch_tile_floats(p))) return fail(10);
   return true;
+}
+
+bool gemv_mfma_config_applicable(const Problem& p, const tlhip_kernel_config_t& c, const char** why) {
+  return mfma_applicable(p, (p.n + 15) / 16, c, why);
+}
+
+// The problems of a group: same activations and rows, one shape class; N, pointers and
+// epilogues per problem.  The configuration is checked against the group's total rows.
+bool gemv_mfma_group_applicable(const Problem* ps, int count, const tlhip_kernel_config_t& c, const char** why) {
+  if (count < 1 || count > kMfmaMaxGroup) {
+    if (why) *why = "a group holds 1..4 problems";
+    return false;
+  }
+  int64_t nblocks = 0;
+  for (int i = 0; i < count; ++i) {
+    if (ps[i].x != ps[0].x || ps[i].m != ps[0].m || ps[i].format != ps[0].format || ps[i].group_size != ps[0].group_size ||
+        ps[i].k != ps[0].k || ps[i].x_dtype != ps[0].x_dtype || ps[i].y_dtype != ps[0].y_dtype || ps[i].alpha != ps[0].alpha) {
+      if (why) *why = "the problems of a group share activations, rows, format, group size, K, output type and alpha";
+      return false;
+    }
+    nblocks += (ps[i].n + 15) / 16;
+  }
+  return mfma_applicable(ps[0], nblocks > 0 ? nblocks : 1, c, why);
 }
 
 template <int FMT, bool WIDE>
@@ -640,20 +682,30 @@ static int launch_mfma_line(int unroll, const MfmaArgs& a, int grid, int threads
   return launch_kernel(fn, dim3(grid), dim3(threads), args, lds_bytes, stream);
 }
 
-int launch_gemv_mfma(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t stream) {
+int launch_gemv_mfma_group(const Problem* ps, int count, const tlhip_kernel_config_t& c, hipStream_t stream) {
   const char* why = nullptr;
-  if (!gemv_mfma_config_applicable(p, c, &why))
+  if (!gemv_mfma_group_applicable(ps, count, c, &why))
     return set_error(TLHIP_ERR_INVALID, "gemv_mfma: config not applicable: %s", why);
-  if (p.n == 0 || p.m == 0) return TLHIP_OK;
+  const Problem& p = ps[0];
   const bool int4 = p.format == TLHIP_FMT_INT4_GROUPED;
   const int cw = int4 ? 32 : 16;
   const int waves = c.p0, unroll = c.p1;
   MfmaArgs a;
-  a.packed = (const u32x4*)p.packed;
-  a.scales = p.scales;
+  memset(&a, 0, sizeof a);
+  int64_t nblocks = 0;
+  for (int i = 0; i < count; ++i) {
+    if (ps[i].n == 0) continue;
+    MfmaProblem& P = a.p[a.count++];
+    P.packed = (const u32x4*)ps[i].packed;
+    P.scales = ps[i].scales;
+    P.y = ps[i].y;
+    P.n = ps[i].n;
+    P.first_block = (int)nblocks;
+    P.epi = ps[i].epi;
+    nblocks += (ps[i].n + 15) / 16;
+  }
+  if (a.count == 0 || p.m == 0) return TLHIP_OK;
   a.x = (const _Float16*)p.x;
-  a.y = p.y;
-  a.n = p.n;
   a.k = (int)p.k;
   a.m = (int)p.m;
   a.nchunks = (int)(p.k / cw);
@@ -674,14 +726,13 @@ int launch_gemv_mfma(const Problem& p, const tlhip_kernel_config_t& c, hipStream
     const int rc = problem_scratch(p, stream, &a.workspace, &a.counters);
     if (rc) return rc;
   }
-  a.nblocks = (int)((p.n + 15) / 16);
+  a.nblocks = (int)nblocks;
   a.nwgblocks = (a.nblocks + a.blocks_per_wg - 1) / a.blocks_per_wg;
   a.alpha = p.alpha;
   a.scale_mul = p.format == TLHIP_FMT_INT8_GROUPED ? (1.0f / 127.0f) : 1.0f;
   a.y_dtype = p.y_dtype;
-  a.epi = p.epi;
   MfmaGeometry geo;
-  if (!mfma_geometry(p.n, p.k, p.m, waves, a.kw, a.ks, line_patch_bytes(c), &geo))
+  if (!mfma_geometry(nblocks, p.k, p.m, waves, a.kw, a.ks, line_patch_bytes(c), &geo))
     return set_error(TLHIP_ERR_INVALID, "gemv_mfma: launch geometry does not close");
   const size_t lds_bytes = geo.lds_bytes;
   a.patch_unit = (int)(geo.patch_offset / 16);
@@ -712,8 +763,16 @@ int launch_gemv_mfma(const Problem& p, const tlhip_kernel_config_t& c, hipStream
   }
   if (rc) return rc;
   TLHIP_CHECK_HIP(hipGetLastError());
-  count_gemv_dispatch();
+  for (int i = 0; i < a.count; ++i) count_gemv_dispatch();
   return TLHIP_OK;
+}
+
+int launch_gemv_mfma(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t stream) {
+  const char* why = nullptr;
+  if (!gemv_mfma_config_applicable(p, c, &why))
+    return set_error(TLHIP_ERR_INVALID, "gemv_mfma: config not applicable: %s", why);
+  if (p.n == 0 || p.m == 0) return TLHIP_OK;
+  return launch_gemv_mfma_group(&p, 1, c, stream);
 }
 
 // Every instance launch_gemv_mfma can reach, in prepare mode (see launch_kernel).
