@@ -561,6 +561,85 @@ def main() -> int:
             probe[f"{n}x{k}"] = {"bytes": nbytes, "us": round(us, 2), "gbps": round(nbytes / us / 1e3, 1)}
         details["read_only_probe"] = probe
 
+        # one Qwen3-8B-shaped decoder layer's Linears (q 4096, k 1024, v 1024, o 4096, gate 12288,
+        # up 12288 from K = 4096; down 4096 from K = 12288): 7 launches, or 4 with the Linears
+        # that share their activations (q/k/v, gate/up) grouped into one launch each
+        # (packages/qwen3-browser/src/model.ts:341-361 issues them back to back)
+        kv_pool, _ = B.weight_pool("int4", 1024, 4096, 32, "f16", pool_bytes=300e6)
+        qkv_cat, _ = B.weight_pool("int4", 6144, 4096, 32, "f16")     # stand-ins of the groups' combined
+        gu_cat, _ = B.weight_pool("int4", 24576, 4096, 32, "f16")     # rows, for the tuner only
+        gfn = L.load().tlhip_gemv_grouped_rows
+        layer_rows = []
+        for m in (1, 8, 16):
+            x4, x12 = xs[(m, 4096)], xs[(m, 12288)]
+            y = {key: be._alloc([m, n], "f16") for key, n in
+                 (("q", 4096), ("k", 1024), ("v", 1024), ("o", 4096), ("gate", 12288), ("up", 12288), ("down", 4096))}
+            ycat = be._alloc([m, 24576], "f16")
+            if not args.no_autotune:
+                B.tune(kv_pool, x4, m, y["k"])
+                B.tune(qkv_cat, x4, m, ycat)
+                B.tune(gu_cat, x4, m, ycat)
+            p44, p124, p412 = pools[(4096, 4096)], pools[(12288, 4096)], pools[(4096, 12288)]
+            nlayers = 12  # distinct weight sets: 12 x 97 MB, far above the last-level cache
+
+            def probs_of(items):
+                arr = (L.GemvProblem * len(items))()
+                for i, (w, x, out) in enumerate(items):
+                    arr[i].w = be._qweight(w, False)
+                    arr[i].x = x.ptr
+                    arr[i].y = out.ptr
+                    arr[i].epilogue = None
+                return arr, len(items)
+            sep, grp, gu_only = [], [], []
+            for li in range(nlayers):
+                wq, wo = p44[(2 * li) % len(p44)], p44[(2 * li + 1) % len(p44)]
+                wk, wv = kv_pool[(2 * li) % len(kv_pool)], kv_pool[(2 * li + 1) % len(kv_pool)]
+                wg, wu = p124[(2 * li) % len(p124)], p124[(2 * li + 1) % len(p124)]
+                wd = p412[li % len(p412)]
+                linears = [(wq, x4, y["q"]), (wk, x4, y["k"]), (wv, x4, y["v"]), (wo, x4, y["o"]), (wg, x4, y["gate"]),
+                           (wu, x4, y["up"]), (wd, x12, y["down"])]
+                sep.append([probs_of([t]) for t in linears])
+                grp.append([probs_of(linears[0:3]), probs_of(linears[3:4]), probs_of(linears[4:6]), probs_of(linears[6:7])])
+                gu_only.append(probs_of(linears[4:6]))
+            state = {"i": 0}
+
+            def runner(table):
+                def call():
+                    for arr, cnt in table[state["i"] % nlayers]:
+                        rc = gfn(arr, cnt, L.F16, m, L.F16, 1.0, None)
+                        if rc:
+                            L.check(rc)
+                    state["i"] += 1
+                return call
+
+            def gate_up():
+                arr, cnt = gu_only[state["i"] % nlayers]
+                state["i"] += 1
+                rc = gfn(arr, cnt, L.F16, m, L.F16, 1.0, None)
+                if rc:
+                    L.check(rc)
+            layer_bytes = sum(algorithmic_bytes("int4", n, k, 32, m, 2, 2) for (n, k) in
+                              ((4096, 4096), (1024, 4096), (1024, 4096), (4096, 4096), (12288, 4096), (12288, 4096), (4096, 12288)))
+            gu_bytes = 2 * algorithmic_bytes("int4", 12288, 4096, 32, m, 2, 2) - m * 4096 * 2
+            us_sep = B.median_time(runner(sep), 40)
+            us_grp = B.median_time(runner(grp), 40)
+            us_gu = B.median_time(gate_up, 100)
+            layer_rows.append({
+                "m": m, "bytes": layer_bytes, "us_7_launches": round(us_sep, 2), "us_4_launches": round(us_grp, 2),
+                "gbps_4_launches": round(layer_bytes / us_grp / 1e3, 1),
+                "frac_of_peak_4_launches": round(layer_bytes / us_grp / 1e3 / HBM_PEAK_GBPS, 4),
+                "gate_up_grouped_us": round(us_gu, 2), "gate_up_grouped_gbps": round(gu_bytes / us_gu / 1e3, 1),
+                "gate_up_grouped_frac_of_peak": round(gu_bytes / us_gu / 1e3 / HBM_PEAK_GBPS, 4),
+                "config_qkv": list(be.selectedConfig(qkv_cat[0], "f16", m, "f16").as_tuple()),
+                "config_gate_up": list(be.selectedConfig(gu_cat[0], "f16", m, "f16").as_tuple())})
+            for t in list(y.values()) + [ycat]:
+                t.destroy()
+        details["qwen3_8b_decode_layer"] = layer_rows
+        for pool_ in (kv_pool, qkv_cat, gu_cat):
+            for w in pool_[1:]:
+                w._base.destroy()
+                w.scales.destroy()
+
         # config 5: LM head 256000 x 2304 int8-row (f32 logits) and the MLP GEMVs
         lm_pool, _ = B.weight_pool("int8-row", 256000, 2304, 0, "f32", pool_bytes=1.25e9)
         lm = []

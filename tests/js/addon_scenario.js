@@ -47,19 +47,19 @@ for (const c of manifest.cases) {
     r.gemm = H.getQuantGemmDispatchCount() - m0;
     r.shape = y.shape;
     r.dtype = y.dtype;
-    save(c.out, be.ops.read(y));
+    save(c.out, be.readSync(y));
   } else if (c.kind === "quantize") {
     const q = H.quantizeLinearWeight(load(c.weight, "f32"), c.n, c.k, c.g);
     save(c.out_packed, q.packed);
     save(c.out_scales, q.scales);
     const w = be.createQuantizedWeight(q.packed, q.scales, c.n, c.k, H.resolveWeightFormat(c.g === 64 ? "int8-64" : "int8-128", "f32"));
     const d0 = H.getDequantI8DispatchCount();
-    save(c.out_dequant, be.ops.read(be.dequantizeToF32(w)));
+    save(c.out_dequant, be.readSync(be.dequantizeToF32(w)));
     r.dequant = H.getDequantI8DispatchCount() - d0;
     // and on the device, from the f32 weight uploaded as it is
     const wdev = be.ops.tensorFromArray(load(c.weight, "f32"), [c.n, c.k], "f32");
     const qd = be.quantizeLinearWeightOnDevice(wdev, c.g, "f32");
-    save(c.out_dequant_device, be.ops.read(be.dequantizeToF32(qd)));
+    save(c.out_dequant_device, be.readSync(be.dequantizeToF32(qd)));
   } else if (c.kind === "rmsnorm_linear" || c.kind === "gated_linear") {
     const w = weightOf(be, c);
     const x = tensor(be, c.x, [c.m, c.k], c.xdtype);
@@ -67,23 +67,27 @@ for (const c of manifest.cases) {
     if (c.kind === "rmsnorm_linear") {
       const nw = tensor(be, c.norm_weight, [c.k], "f32");
       const normed = be.ops.fusedRMSNormForward(x, nw, { numRows: c.m, featureDim: c.k, eps: c.eps });
-      save(c.out_norm, be.ops.read(normed));
+      save(c.out_norm, be.readSync(normed));
       y = be.linearAfterRMSNorm(x, nw, c.eps, w);
       apart = be.linear(normed, w, null, "none", true);
     } else {
       const up = tensor(be, c.up, [c.m, c.k], c.xdtype);
       const prod = be.ops.mul(be.ops.silu(x), up);   // the model's two ops
-      save(c.out_prod, be.ops.read(prod));
+      save(c.out_prod, be.readSync(prod));
       y = be.linearAfterGatedMul(x, up, "silu", w);
       apart = be.linear(prod, w, null, "none", true);
     }
-    save(c.out, be.ops.read(y));
-    save(c.out_apart, be.ops.read(apart));
+    save(c.out, be.readSync(y));
+    save(c.out_apart, be.readSync(apart));
   } else if (c.kind === "grouped") {
-    const x = tensor(be, c.x, [1, c.k], "f16");
+    const x = tensor(be, c.x, [c.m, c.k], "f16");
     const ws = c.weights.map((wc) => weightOf(be, Object.assign({ k: c.k, format: c.format, element: "f16" }, wc)));
     const outs = be.linearGrouped(x, ws);
-    outs.forEach((o, i) => save(c.weights[i].out, be.ops.read(o)));
+    outs.forEach((o, i) => save(c.weights[i].out, be.readSync(o)));
+    if (c.out_noalloc) {
+      const out = be.ops.zeros([c.m, c.weights[0].n], "f16");
+      save(c.out_noalloc, be.readSync(be.linearInto(out, x, ws[0], null, "none")));
+    }
   } else if (c.kind === "side_door") {
     // the fused path's call for matmul -> bias -> unary (-> cast): executor.ts:2959-3049
     const w = weightOf(be, c);
@@ -102,7 +106,7 @@ for (const c of manifest.cases) {
       outputDtype: c.out_dtype, epilogueConfig: epilogue, epilogueBuffers: [bias], packing: w.format.packing, scales: w.scales });
     r.dtype = y1.dtype;
     r.plan = D.planBareMatmul(x, be.ops.transpose(w));
-    [y1, y2, y3, y4].forEach((y, i) => save(c.out + i, be.ops.read(y)));
+    [y1, y2, y3, y4].forEach((y, i) => save(c.out + i, be.readSync(y)));
     try {
       D.dispatchMatmul(x, be.ops.transpose(w), false, false, undefined,
         { epilogue: { ops: [{ kind: "binary", op: "mul", inputIndex: 0 }], additionalInputCount: 1, outputDtype: "f32" }, epilogueInputs: [bias] });
@@ -117,7 +121,7 @@ for (const c of manifest.cases) {
       save(c.out_indices, t.indices);
     });
     const packed = be.ops.deviceTopK(logits, c.k);
-    save(c.out_packed, be.ops.read(packed));
+    save(c.out_packed, be.readSync(packed));
   }
   results.cases[c.name] = r;
 }
@@ -165,7 +169,45 @@ function expectThrow(name, fn) {
   results.autotune_runs = H.getAutotuneRunCount() - a0;
   H.setAutotuneEnabled(false);
 }
+/* the Backend contract (src/backend/types.ts:340-696): every required op is there (the list is
+ * the mock backend's, src/backend/mock/index.ts:150-176), `read` is a Promise of numbers, and
+ * the ops outside this path are declared delegates to a cpu backend */
+const pending = [];
+{
+  const conf = {};
+  conf.required = H.REQUIRED_OPS.slice();
+  conf.missing = H.REQUIRED_OPS.filter((n) => typeof be.ops[n] !== "function");
+  conf.name = be.name;
+  const a = be.ops.tensorFromArray([1, 2, 3, 4, 5, 6], [2, 3], "f32");
+  const b = be.ops.tensorFromArray([6, 5, 4, 3, 2, 1], [2, 3], "f32");
+  const p = be.ops.read(a);
+  conf.read_is_promise = p instanceof Promise;
+  pending.push(p.then((v) => {
+    conf.read_value = v;
+    conf.read_is_array = Array.isArray(v);
+  }));
+  expectThrow("delegated_without_cpu", () => be.ops.sub(a, b));
+  // a stand-in for getBackend("cpu"): tensors are {shape, toArray()}, as BackendTensor requires
+  const cpuTensor = (shape, data) => ({ shape, toArray: () => data });
+  be.setCpuDelegate({ name: "cpu", ops: {
+    tensorFromArray: (values, shape) => cpuTensor(shape, Array.from(values)),
+    sub: (x, y) => cpuTensor(x.shape, x.toArray().map((v, i) => v - y.toArray()[i])),
+    sum: (x) => cpuTensor([], [x.toArray().reduce((s, v) => s + v, 0)]),
+  } });
+  const d = be.ops.sub(a, b);
+  conf.sub = Array.from(be.readSync(d));
+  conf.sub_shape = d.shape;
+  conf.sum = Array.from(be.readSync(be.ops.sum(a)));
+  expectThrow("delegated_unknown_to_cpu", () => be.ops.gather(a, 0, b));
+  // a strided view is materialised through the host
+  const at = be.ops.transpose(a);
+  conf.transposed_contiguous = at.isContiguous;
+  conf.transposed = Array.from(be.readSync(be.ops.contiguous(at)));
+  conf.transposed_to_array = at.toArray();
+  be.setCpuDelegate(null);
+  results.conformance = conf;
+}
 be.synchronize();
-setImmediate(() => {
+Promise.all(pending).then(() => setImmediate(() => {
   fs.writeFileSync(path.join(dir, "results.json"), JSON.stringify(results));
-});
+}));

@@ -178,3 +178,22 @@ def test_gemm_rejects_f32_activations_and_falls_back_to_gemv_passes(be):
     y = be.linear(xt, w).numpy()
     assert T.getQuantGemvDispatchCount() == v0 + 3      # 16 + 16 + 8 rows
     assert rel_l2(y, O.linear(x, deq)) <= 2e-6
+
+
+@pytest.mark.parametrize("lo,hi", [(200.0, 4000.0), (2e-3, 8e-3)])
+@pytest.mark.parametrize("cfg", [None, (2, 128, 128, 64, 2, 2)])
+def test_prefill_scale_range(be, lo, hi, cfg):
+    """The prefill GEMMs round q*s once to f16 before the matrix cores: inside the stated
+    scale range (|q*s| within f16's normal range) the result keeps the 1e-3 bar."""
+    rng = np.random.default_rng(int(hi))
+    m, n, k = 64, 256, 512
+    q = rng.integers(-8, 8, (n, k)).astype(np.int8)
+    packed = O.np_pack_int4(q)
+    scales = f16_round(rng.uniform(lo, hi, n * (k // 32))).view(np.uint16)
+    deq = O.dequant_int4_grouped(packed, scales, n, k, 32)
+    x = make_x(m, k, "f16", rng, std=0.5)
+    got = run(be, "int4-grouped", packed, scales, n, k, 32, x, "f32",
+              config=L.KernelConfig.of(*cfg) if cfg else None)
+    want = O.linear(x.astype(np.float32), deq, threads=8)
+    assert np.isfinite(got).all()
+    assert rel_l2(got, want) <= REL_L2_TOL, rel_l2(got, want)

@@ -102,8 +102,20 @@ def run(tmp_path_factory):
         gw.append({"n": n, "packed": put(f"g{i}.packed", packed), "scales": put(f"g{i}.scales", scales),
                    "out": f"g{i}.y"})
         want[f"grouped{i}"] = O.linear(x.astype(np.float32), deq)
-    cases.append({"kind": "grouped", "name": "grouped", "format": "int4-32", "k": k,
+    cases.append({"kind": "grouped", "name": "grouped", "format": "int4-32", "k": k, "m": 1,
                   "x": put("g.x", x.astype(np.float32)), "weights": gw})
+    # the same group for a batched decode step (8 rows), and one Linear through the entry point
+    # that allocates nothing
+    x8 = make_x(8, k, "f16", rng)
+    gw8 = []
+    for i in range(3):
+        gw8.append(dict(gw[i], out=f"g8_{i}.y"))
+        n = gw[i]["n"]
+        deq = O.dequant_int4_grouped(np.fromfile(os.path.join(d, gw[i]["packed"]), np.uint32),
+                                     np.fromfile(os.path.join(d, gw[i]["scales"]), np.uint16), n, k, 32)
+        want[f"grouped8_{i}"] = O.linear(x8.astype(np.float32), deq)
+    cases.append({"kind": "grouped", "name": "grouped8", "format": "int4-32", "k": k, "m": 8,
+                  "x": put("g8.x", x8.astype(np.float32)), "weights": gw8, "out_noalloc": "g8.noalloc"})
 
     for name, m, xdt, out_dtype in (("door_m1", 1, "f32", "f32"), ("door_m64", 64, "f16", "f16")):
         rng = seeded("addon", name)
@@ -195,6 +207,14 @@ def test_grouped_launch(run):
         assert rel_l2(run["get"](f"g{i}.y").reshape(want.shape), want) <= 1e-3
 
 
+def test_grouped_launch_of_a_batched_step_and_the_no_alloc_entry_point(run):
+    for i in range(3):
+        want = run["want"][f"grouped8_{i}"]
+        assert rel_l2(run["get"](f"g8_{i}.y").reshape(want.shape), want) <= 1e-3
+    want = run["want"]["grouped8_0"]
+    assert rel_l2(run["get"]("g8.noalloc").reshape(want.shape), want) <= 1e-3
+
+
 def test_topk(run):
     logits = run["want"]["topk"]
     order = np.argsort(-logits, kind="stable")[:40]
@@ -219,3 +239,24 @@ def test_tuning_cache_and_autotune_hooks(run):
     assert t["selected_after_import"] == t["seeded"]
     assert run["results"]["autotune_enabled"] is True
     assert run["results"]["autotune_runs"] == 1
+
+
+def test_backend_object_conforms_to_the_required_ops(run):
+    """The Backend contract (src/backend/types.ts:340-696): every op the smallest conforming
+    backend has (src/backend/mock/index.ts:150-176) is a function, `read` is a Promise of
+    numbers (types.ts:666), and the ops outside the path are declared cpu delegates."""
+    c = run["results"]["conformance"]
+    mock_ops = ["tensorFromArray", "add", "sub", "div", "mul", "matmul", "sqrt", "relu", "expand", "reshape", "transpose",
+                "permute", "contiguous", "max", "where", "stridedScatterCopy", "stridedScatterAdd", "gather", "scatterAdd",
+                "sum", "mean", "read"]
+    assert sorted(c["required"]) == sorted(mock_ops)
+    assert c["missing"] == [] and c["name"] == "hip"
+    assert c["read_is_promise"] and c["read_is_array"] and c["read_value"] == [1, 2, 3, 4, 5, 6]
+    e = run["results"]["errors"]
+    assert "sub is outside the quantized-weight linear path" in e["delegated_without_cpu"]["message"]
+    assert "setCpuDelegate" in e["delegated_without_cpu"]["message"]
+    assert "gather is outside" in e["delegated_unknown_to_cpu"]["message"]
+    assert c["sub"] == [-5, -3, -1, 1, 3, 5] and c["sub_shape"] == [2, 3]
+    assert c["sum"] == [21]
+    assert c["transposed_contiguous"] is False
+    assert c["transposed"] == [1, 4, 2, 5, 3, 6] and c["transposed_to_array"] == [1, 4, 2, 5, 3, 6]

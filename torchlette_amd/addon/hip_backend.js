@@ -18,7 +18,16 @@
  *   linear                                         frontend/torchlette.ts:878-894
  *   setAutotuneEnabled, exportTuningCache, ...     matmul/dispatch.ts:99-141, autotune.ts:309-329
  *
- * There is no CPU fallback: without a gfx950 device `getBackend()` throws. */
+ *   ops.sub / div / sqrt / expand / gather / scatterAdd / sum / max / mean / where /
+ *   stridedScatterCopy / stridedScatterAdd / contiguous (of a strided view)
+ *                                                  the rest of the required BackendOps
+ *                                                  (types.ts:340-679; the smallest conforming
+ *                                                  backend is mock/index.ts:150-176): OUTSIDE
+ *                                                  this path, declared host-copy delegates to
+ *                                                  the cpu backend given to setCpuDelegate()
+ *
+ * There is no CPU fallback for the path itself: without a gfx950 device `getBackend()`
+ * throws, and the delegated ops throw with the op's name until a cpu backend is set. */
 const path = require("path");
 const tl = require(path.join(__dirname, "tlhip_napi.node"));
 
@@ -27,6 +36,14 @@ const DT = { f32: 0, f16: 1, i32: 2 };
 const BYTES = { f32: 4, f16: 2, u32: 4, i32: 4 };
 const UNARY = { none: 0, relu: 1, silu: 2, gelu: 3, gelu_tanh: 3, gelu_erf: 4, sigmoid: 5, tanh: 6 };
 const PRO_RMSNORM = 1, PRO_GATED_MUL = 2;
+/* BackendOps that every backend must have (types.ts:340-679; mock/index.ts:150-176) and that
+ * are not part of the quantized-weight linear path. */
+const DELEGATED_OPS = ["sub", "div", "sqrt", "expand", "gather", "scatterAdd", "sum", "max", "mean", "where",
+                       "stridedScatterCopy", "stridedScatterAdd"];
+/* ... and the whole required set, for conformance checks. */
+const REQUIRED_OPS = ["tensorFromArray", "add", "sub", "div", "mul", "matmul", "sqrt", "relu", "expand", "reshape", "transpose",
+                      "permute", "contiguous", "gather", "scatterAdd", "sum", "max", "mean", "where", "stridedScatterCopy",
+                      "stridedScatterAdd", "read"];
 
 function sizeOf(shape) {
   return shape.reduce((p, c) => p * c, 1);
@@ -82,7 +99,7 @@ class HipTensor {
   }
   /** BackendTensor.toArray: a host copy as plain numbers. */
   toArray() {
-    return Array.from(this.backend.ops.read(this));
+    return Array.from(this.backend.readSync(this));
   }
   destroy() {
     if (this.ownsBuffer && this.ptr) {
@@ -117,26 +134,16 @@ class HipBackend {
         if (t.nbytes) tl.memset(t.ptr, 0, t.nbytes);
         return t;
       },
-      /** `read`: f16 tensors come back as f32 values, as the reference's read does. */
+      /** read(a): Promise<number[]> (types.ts:666): the one op that waits.  f16 tensors come
+       *  back as f32 values, as the reference's read does. */
       read(a) {
-        const t = a.isContiguous ? a : self.ops.contiguous(a);
-        const n = t.size;
-        let out;
-        if (t.dtype === "f32") {
-          out = new Float32Array(n);
-          tl.memcpyD2H(out, t.ptr);
-        } else if (t.dtype === "f16") {
-          const bits = new Uint16Array(n);
-          tl.memcpyD2H(bits, t.ptr);
-          out = fromF16Bits(bits);
-        } else if (t.dtype === "u32") {
-          out = new Uint32Array(n);
-          tl.memcpyD2H(out, t.ptr);
-        } else {
-          out = new Int32Array(n);
-          tl.memcpyD2H(out, t.ptr);
-        }
-        return out;
+        return new Promise((resolve, reject) => {
+          try {
+            resolve(Array.from(self.readSync(a)));
+          } catch (e) {
+            reject(e);
+          }
+        });
       },
       permute(a, dims) {
         const v = new HipTensor(self, dims.map((d) => a.shape[d]), a.dtype, a.ptr, a.nbytes, false, a._base || a);
@@ -165,9 +172,12 @@ class HipBackend {
         v.scales = a.scales;
         return v;
       },
+      /** A strided view is materialised through a host copy (outside the path: the
+       *  Linear's transposed weight view is consumed by matmul as a view, never copied). */
       contiguous(a) {
         if (a.isContiguous) return a;
-        throw new Error("hip backend contiguous: materialising a strided view is outside the quantized-weight linear path");
+        if (a.format && a.format.packing) throw new Error("hip backend contiguous: a packed weight view is not materialised");
+        return self.ops.tensorFromArray(self.readSync(a), a.shape, a.dtype === "f16" ? "f16" : a.dtype);
       },
       /** matmul-ops.ts:42-59: a packed B operand goes to matmulQuantizedB. */
       matmul(a, b) {
@@ -232,12 +242,75 @@ class HipBackend {
         return { values, indices };
       },
       /** types.ts:632-634: [2k] f32 on the device, values then indices (as f32). */
-      deviceTopK(logits, k) {
+      deviceTopK(logits, config) {
+        const k = typeof config === "number" ? config : config.k;
         const out = self._alloc([2 * k], "f32");
         tl.topk(logits.ptr, 0, logits.size, k, out.ptr, out.ptr + BigInt(4 * k), DT.f32);
         return out;
       },
     };
+    /* The required BackendOps that are not on the quantized-weight linear path: declared
+     * host-copy delegates.  Each downloads its tensor arguments, runs the cpu backend's op
+     * of the same name and uploads the result. */
+    for (const name of DELEGATED_OPS) {
+      if (!(name in this.ops)) this.ops[name] = (...args) => self._viaHost(name, args);
+    }
+    this._cpu = null;
+  }
+
+  /** The cpu backend (`getBackend("cpu")` of a torchlette checkout) the delegated ops run on. */
+  setCpuDelegate(cpuBackend) {
+    this._cpu = cpuBackend;
+  }
+
+  _viaHost(name, args) {
+    const cpu = this._cpu;
+    if (!cpu || !cpu.ops || typeof cpu.ops[name] !== "function")
+      throw new Error(`hip backend: ${name} is outside the quantized-weight linear path; it runs on the cpu backend ` +
+                      "through a host copy once setCpuDelegate(cpuBackend) has been called");
+    let dtype = "f32";
+    const onCpu = [];
+    const lower = (v) => {
+      if (v instanceof HipTensor) {
+        if (v.dtype === "f16") dtype = "f16";
+        // the cpu backend holds every dtype as f32 values (src/backend/cpu/numeric.ts:29-117)
+        const t = cpu.ops.tensorFromArray(Array.from(this.readSync(v)), v.shape.slice());
+        onCpu.push(t);
+        return t;
+      }
+      return Array.isArray(v) && v.some((e) => e instanceof HipTensor) ? v.map(lower) : v;
+    };
+    const out = cpu.ops[name].apply(cpu.ops, args.map(lower));
+    const up = this.ops.tensorFromArray(out.toArray(), out.shape.slice(), dtype);
+    for (const t of onCpu.concat([out])) if (t.destroy) t.destroy();
+    return up;
+  }
+
+  /** Synchronous host copy of a tensor as a typed array (f16 -> f32 values); a strided
+   *  view is gathered on the host from its base buffer. */
+  readSync(a) {
+    const TYPES = { f32: Float32Array, u32: Uint32Array, i32: Int32Array };
+    const fetch = (ptr, n, dtype) => {
+      if (dtype === "f16") {
+        const bits = new Uint16Array(n);
+        if (n) tl.memcpyD2H(bits, ptr);
+        return fromF16Bits(bits);
+      }
+      const out = new TYPES[dtype](n);
+      if (n) tl.memcpyD2H(out, ptr);
+      return out;
+    };
+    if (a.isContiguous) return fetch(a.ptr, a.size, a.dtype);
+    const base = fetch(a.ptr, a.nbytes / BYTES[a.dtype], a.dtype);
+    const out = new base.constructor(a.size);
+    const idx = new Array(a.shape.length).fill(0);
+    for (let i = 0; i < out.length; i++) {
+      let off = 0;
+      for (let d = 0; d < idx.length; d++) off += idx[d] * a.strides[d];
+      out[i] = base[off];
+      for (let d = idx.length - 1; d >= 0 && ++idx[d] === a.shape[d]; d--) idx[d] = 0;
+    }
+    return out;
   }
 
   _alloc(shape, dtype) {
@@ -348,23 +421,27 @@ class HipBackend {
     return y;
   }
 
-  /** Up to four decode Linears on one f16 activation row in one launch (q/k/v, gate/up). */
+  /** Up to four decode Linears on the same f16 activations (1..16 rows; one row with a
+   *  prologue) in one launch (q/k/v, gate/up). */
   linearGrouped(input, weights, biases, activation, prologue) {
     if (weights.length < 1 || weights.length > 4) throw new Error("linearGrouped: a group holds 1..4 weights");
-    if (input.dtype !== "f16") throw new Error("linearGrouped: one f16 activation row");
+    if (input.dtype !== "f16") throw new Error("linearGrouped: f16 activations");
+    const rows = input.size / this._weightArgs(weights[0], false)[3];
+    if (!(rows >= 1 && rows <= 16) || (prologue && rows !== 1)) throw new Error("linearGrouped: 1..16 activation rows (one row with a prologue)");
     const outDtype = weights.every((w) => w.format.elementType === "f16") ? "f16" : "f32";
     const act = UNARY[activation === "gelu" ? "gelu_tanh" : activation || "none"];
     const outs = [];
     const probs = weights.map((w, i) => {
       const wa = this._weightArgs(w, false);
-      if (input.size !== wa[3]) throw new Error("linearGrouped: one f16 activation row");
+      if (input.size !== rows * wa[3]) throw new Error("linearGrouped: the weights of a group share K");
       const out = this._alloc(input.shape.slice(0, -1).concat([wa[2]]), outDtype);
       outs.push(out);
       const b = biases && biases[i];
       return wa.concat([input.ptr, out.ptr, b ? b.ptr : null, b ? DT[b.dtype] : 0, act]);
     });
     if (prologue) tl.gemvGrouped(probs, DT[input.dtype], DT[outDtype], prologue.kind, prologue.operand, prologue.unary, prologue.eps);
-    else tl.gemvGrouped(probs, DT[input.dtype], DT[outDtype]);
+    else if (rows === 1) tl.gemvGrouped(probs, DT[input.dtype], DT[outDtype]);
+    else tl.gemvGroupedRows(probs, DT[input.dtype], rows, DT[outDtype]);
     return outs;
   }
 
@@ -414,6 +491,17 @@ class HipBackend {
 
   linearGroupedAfterRMSNorm(input, normWeight, eps, weights, biases, activation) {
     return this.linearGrouped(input, weights, biases, activation, { kind: PRO_RMSNORM, operand: normWeight.ptr, unary: 0, eps });
+  }
+
+  /** linear(input, weight, bias, activation) for M <= 16 through the entry point that allocates no
+   *  device memory (tlhip_gemv_noalloc; `out` is the caller's): for code under graph capture. */
+  linearInto(out, input, weight, bias, activation) {
+    const wa = this._weightArgs(weight, false);
+    const m = input.size / wa[3];
+    const act = UNARY[activation === "gelu" ? "gelu_tanh" : activation || "none"];
+    tl.gemvNoalloc.apply(null, wa.concat([input.ptr, DT[input.dtype], m, out.ptr, DT[out.dtype], bias ? bias.ptr : null,
+                                          bias ? DT[bias.dtype] : 0, act]));
+    return out;
   }
 
   /** Explicit dequantisation to f32 [N,K] (dispatchDequantizeInt8Grouped, dispatch.ts:949-1037). */
@@ -500,5 +588,7 @@ module.exports = {
     tl.tuneCacheClear();
     tl.countersReset();
   },
+  REQUIRED_OPS,
+  DELEGATED_OPS,
   native: tl,
 };

@@ -438,38 +438,48 @@ static napi_value GemvPrologue(napi_env env, napi_callback_info info) {
   napi_get_boolean(env, true, &b);
   return b;
 }
-/* gemvGrouped([ [format, groupSize, n, k, packed, scales, xPtr, yPtr, biasPtr|null, biasDtype, unary], ... ],
- *             xDtype, yDtype [, kind, operandPtr, proUnary, eps]) */
-static napi_value GemvGrouped(napi_env env, napi_callback_info info) {
-  ARGS(3);
+/* A JavaScript array of problems [format, groupSize, n, k, packed, scales, xPtr, yPtr, biasPtr|null,
+ * biasDtype, unary] -> tlhip_gemv_problem_t[count]; NULL (with a pending exception) on a bad one. */
+static const char* parse_problems(napi_env env, napi_value arr, tlhip_gemv_problem_t* probs, tlhip_epilogue_t* eps,
+                                  uint32_t* count_out) {
   uint32_t count = 0;
   bool is_array = false;
-  if (napi_is_array(env, a[0], &is_array) != napi_ok || !is_array) return throw_type(env, "tlhip: gemvGrouped needs an array of problems");
-  napi_get_array_length(env, a[0], &count);
-  if (count > 4) return throw_type(env, "tlhip: a group holds at most 4 problems");
-  I32(1, xd);
-  I32(2, yd);
-  tlhip_gemv_problem_t probs[4];
-  tlhip_epilogue_t eps[4];
+  if (napi_is_array(env, arr, &is_array) != napi_ok || !is_array) return "tlhip: gemvGrouped needs an array of problems";
+  napi_get_array_length(env, arr, &count);
+  if (count > 4) return "tlhip: a group holds at most 4 problems";
   for (uint32_t i = 0; i < count; ++i) {
     napi_value row, f[11];
     uint32_t len = 0;
-    napi_get_element(env, a[0], i, &row);
-    if (napi_is_array(env, row, &is_array) != napi_ok || !is_array) return throw_type(env, "tlhip: a problem is an array of 11");
+    napi_get_element(env, arr, i, &row);
+    if (napi_is_array(env, row, &is_array) != napi_ok || !is_array) return "tlhip: a problem is an array of 11";
     napi_get_array_length(env, row, &len);
-    if (len != 11) return throw_type(env, "tlhip: a problem is an array of 11");
+    if (len != 11) return "tlhip: a problem is an array of 11";
     for (uint32_t j = 0; j < 11; ++j) napi_get_element(env, row, j, &f[j]);
-    if (!get_weight(env, f, &probs[i].w)) return throw_type(env, "tlhip: bad weight in problem");
+    if (!get_weight(env, f, &probs[i].w)) return "tlhip: bad weight in problem";
     void *x, *y, *bias;
     int32_t bd, un;
     if (!get_ptr(env, f[6], &x) || !get_ptr(env, f[7], &y) || !get_ptr(env, f[8], &bias) || !get_i32(env, f[9], &bd) ||
         !get_i32(env, f[10], &un))
-      return throw_type(env, "tlhip: bad problem fields");
+      return "tlhip: bad problem fields";
     make_epilogue(bias, bd, un, &eps[i]);
     probs[i].x = x;
     probs[i].y = y;
     probs[i].epilogue = eps[i].n_ops ? &eps[i] : NULL;
   }
+  *count_out = count;
+  return NULL;
+}
+/* gemvGrouped([ [format, groupSize, n, k, packed, scales, xPtr, yPtr, biasPtr|null, biasDtype, unary], ... ],
+ *             xDtype, yDtype [, kind, operandPtr, proUnary, eps]) */
+static napi_value GemvGrouped(napi_env env, napi_callback_info info) {
+  ARGS(3);
+  I32(1, xd);
+  I32(2, yd);
+  tlhip_gemv_problem_t probs[4];
+  tlhip_epilogue_t eps[4];
+  uint32_t count = 0;
+  const char* bad = parse_problems(env, a[0], probs, eps, &count);
+  if (bad) return throw_type(env, bad);
   if (argc >= 7) {
     I32(3, kind);
     PTR(4, operand);
@@ -485,6 +495,38 @@ static napi_value GemvGrouped(napi_env env, napi_callback_info info) {
   } else {
     CHECK(tlhip_gemv_grouped(probs, (int)count, xd, yd, 1.0f, NULL));
   }
+  return undefined(env);
+}
+/* gemvGroupedRows(problems as for gemvGrouped, xDtype, m, yDtype): m <= 16 rows on shared activations */
+static napi_value GemvGroupedRows(napi_env env, napi_callback_info info) {
+  ARGS(4);
+  I32(1, xd);
+  I64(2, m);
+  I32(3, yd);
+  tlhip_gemv_problem_t probs[4];
+  tlhip_epilogue_t eps[4];
+  uint32_t count = 0;
+  const char* bad = parse_problems(env, a[0], probs, eps, &count);
+  if (bad) return throw_type(env, bad);
+  CHECK(tlhip_gemv_grouped_rows(probs, (int)count, xd, m, yd, 1.0f, NULL));
+  return undefined(env);
+}
+/* gemvNoalloc(format, groupSize, n, k, packed, scales, xPtr, xDtype, m, yPtr, yDtype, biasPtr | null, biasDtype, unary):
+ * tlhip_gemv without any allocation (for callers under graph capture) */
+static napi_value GemvNoalloc(napi_env env, napi_callback_info info) {
+  ARGS(14);
+  WEIGHT(0, w);
+  PTR(6, x);
+  I32(7, xd);
+  I64(8, m);
+  PTR(9, y);
+  I32(10, yd);
+  PTR(11, bias);
+  I32(12, bd);
+  I32(13, un);
+  tlhip_epilogue_t ep;
+  make_epilogue(bias, bd, un, &ep);
+  CHECK(tlhip_gemv_noalloc(&w, x, xd, m, y, yd, 1.0f, ep.n_ops ? &ep : NULL, NULL));
   return undefined(env);
 }
 /* biasAdd(inPtr, dtype, biasPtr, biasDtype, outPtr, m, n) */
@@ -717,7 +759,7 @@ NAPI_MODULE_INIT() {
       FN("f32ToF16Bits", F32ToF16Bits), FN("f16BitsToF32", F16BitsToF32),
       FN("quantizeInt8Grouped", QuantizeInt8Grouped), FN("quantizeInt8GroupedDevice", QuantizeInt8GroupedDevice),
       FN("dequant", Dequant), FN("matmulQuantized", MatmulQuantized), FN("matmulQuantizedOps", MatmulQuantizedOps), FN("gemvPrologue", GemvPrologue),
-      FN("gemvGrouped", GemvGrouped), FN("biasAdd", BiasAdd), FN("unary", Unary), FN("cast", Cast),
+      FN("gemvGrouped", GemvGrouped), FN("gemvGroupedRows", GemvGroupedRows), FN("gemvNoalloc", GemvNoalloc), FN("biasAdd", BiasAdd), FN("unary", Unary), FN("cast", Cast),
       FN("rmsnorm", RmsNorm), FN("gatedMul", GatedMul), FN("topk", TopK), FN("selectedConfig", SelectedConfig),
       FN("candidates", Candidates), FN("autotune", Autotune), FN("tuneCacheSeed", TuneCacheSeed),
       FN("setAutotuneEnabled", SetAutotuneEnabled), FN("isAutotuneEnabled", IsAutotuneEnabled),

@@ -702,6 +702,9 @@ int validate_weight(const tlhip_qweight_t* w, const char* who) {
                      (long long)w->n, (long long)w->k);
   if (((uintptr_t)w->packed & 15) != 0)
     return set_error(TLHIP_ERR_INVALID, "%s: packed weights must be 16-byte aligned", who);
+  // the kernels load the scales of consecutive groups as 4-, 8- and 16-byte vectors
+  if (((uintptr_t)w->scales & 15) != 0)
+    return set_error(TLHIP_ERR_INVALID, "%s: scales must be 16-byte aligned", who);
   return TLHIP_OK;
 }
 

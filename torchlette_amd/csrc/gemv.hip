@@ -26,6 +26,7 @@ bool gemv_config_applicable(const Problem& p, const tlhip_kernel_config_t& c, co
       "M above 16",
       "chunks in flight must be 2, 4 or 8 with rows*chunks <= 8",
       "the 4x4x4 matrix-core form (p5 = 1) is built for int4 weights, f16 activations, M <= 4, 16 lanes per row, one row per lane group",
+      "the activation rows of one pass (K x 2 or 4 bytes each; four rows in the 4x4x4 form) do not fit LDS",
   };
   auto fail = [&](int i) {
     if (why) *why = reasons[i];
@@ -45,6 +46,11 @@ bool gemv_config_applicable(const Problem& p, const tlhip_kernel_config_t& c, co
   if (c.p5 != 0 && (c.p5 != 1 || p.format != TLHIP_FMT_INT4_GROUPED || p.x_dtype != TLHIP_F16 || p.m > 4 || c.p0 != 16 ||
                     c.p1 != 1))
     return fail(9);
+  // LDS: one activation row must fit next to the partials (more rows per pass only if they
+  // fit: see launch_gemv); the 4x4x4 form always stages four
+  const size_t xbytes = p.x_dtype == TLHIP_F16 ? 2 : 4;
+  const size_t rows = c.p5 == 1 ? 4 : 1;
+  if (rows * (size_t)p.k * xbytes + 16 * 1024 > (size_t)kLdsBudget) return fail(10);
   return true;
 }
 
@@ -106,8 +112,7 @@ int launch_gemv(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t st
   // activation rows per pass: as many (4, 2 or 1) as fit LDS next to the partials
   int pass = 4;
   while (pass > 1 && (size_t)pass * p.k * xbytes + 16 * 1024 > (size_t)kLdsBudget) pass >>= 1;
-  if ((size_t)pass * p.k * xbytes + 16 * 1024 > (size_t)kLdsBudget)
-    return set_error(TLHIP_ERR_INVALID, "gemv: K=%lld is too long for the LDS-resident activation row", (long long)p.k);
+  if (c.p5 == 1) pass = 4;  // the 4x4x4 form: four rows per pass (checked above)
 
   for (int64_t m0 = 0; m0 < p.m; m0 += pass) {
     const int mrows = (int)(p.m - m0 < pass ? p.m - m0 : pass);

@@ -130,12 +130,26 @@ __global__ __launch_bounds__(MAXT) void gemv_xreg_kernel(const XregArgs a) {
     u32x4 w[NSTEPS][U];
     uint32_t sv[NSTEPS][2 * U];  // scale 4u+t of batch s in half (t & 1) of word 2u + t/2
   };
+  // In the hot loop a problem's fields are SELECTED from the four table entries, each read
+  // with a constant index (scalar registers from the start of the kernel): a run-time index
+  // into the kernel arguments would put scalar loads and their waits into every round.
   auto load_round = [&](Round& b, int r) {
     const int rb = min(rb0 + r * sets, a.nblocks - 1);  // a round past the end reloads the last block; never consumed
-    const XregProblem& P = a.p[problem_of(rb)];
-    const int64_t row = min((int64_t)(rb - P.first_block) * 16 + nl, P.n - 1);  // tail rows reload the last row; never stored
-    const u32x4* wrow = P.packed + row * a.nchunks;
-    const uint16_t* srow = P.scales + row * a.groups_per_row;
+    const u32x4* packed = a.p[0].packed;
+    const uint16_t* scales = a.p[0].scales;
+    int64_t pn = a.p[0].n;
+    int first = 0;
+#pragma unroll
+    for (int j = 1; j < kXMaxGroup; ++j) {
+      const bool here = j < a.count && rb >= a.p[j].first_block;
+      packed = here ? a.p[j].packed : packed;
+      scales = here ? a.p[j].scales : scales;
+      pn = here ? a.p[j].n : pn;
+      first = here ? a.p[j].first_block : first;
+    }
+    const int64_t row = min((int64_t)(rb - first) * 16 + nl, pn - 1);  // tail rows reload the last row; never stored
+    const u32x4* wrow = packed + row * a.nchunks;
+    const uint16_t* srow = scales + row * a.groups_per_row;
 #pragma unroll
     for (int s = 0; s < NSTEPS; ++s) {
       const int it = itb(s);
