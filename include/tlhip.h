@@ -342,7 +342,7 @@ int tlhip_topk(const float* logits, int64_t offset, int64_t length, int k, float
  * 3 = "tiled_direct" (prefill MFMA GEMM for int4, weights dequantised in
  * registers; fields as "tiled" with tile K 128; tiles (M, N, waves M, waves N):
  * 256x256 2x4, 256x128 2x4, 128x256 2x4, 256x128 4x2, 128x128 2x2, 256x256 2x2,
- * 128x256 1x4),
+ * 128x256 1x4, 128x192 2x2),
  * 4 = "gemv_mfma_xreg" (skinny MFMA for int4 g32 with the activations held in
  * registers: p0 waves per workgroup, p1 iterations in flight, p2 workgroups per
  * CU, p3 K slices across workgroups, p4 = 1: every weight load of a wave issued

@@ -59,7 +59,7 @@ def test_every_tile_config_ragged_shapes(be, fmt, g, bm, bn):
 
 
 DIRECT_TILES = [(256, 256, 2, 4), (256, 128, 2, 4), (128, 256, 2, 4), (256, 128, 4, 2), (128, 128, 2, 2), (256, 256, 2, 2),
-                (128, 256, 1, 4)]
+                (128, 256, 1, 4), (128, 192, 2, 2)]
 
 
 @pytest.mark.parametrize("bm,bn,wm,wn", DIRECT_TILES)

@@ -303,7 +303,7 @@ std::vector<tlhip_kernel_config_t> candidates(const Problem& p) {
       tlhip_kernel_config_t c = tiled_cfg(t[0], t[1], t[2], t[3], t[4]);
       if (gemm_config_applicable(p, c, nullptr)) out.push_back(c);
     }
-    static const int direct[][4] = {{256, 256, 2, 4}, {256, 128, 2, 4}, {128, 256, 2, 4}, {256, 128, 4, 2}, {128, 128, 2, 2}, {256, 256, 2, 2}, {128, 256, 1, 4}};
+    static const int direct[][4] = {{256, 256, 2, 4}, {256, 128, 2, 4}, {128, 256, 2, 4}, {256, 128, 4, 2}, {128, 128, 2, 2}, {256, 256, 2, 2}, {128, 256, 1, 4}, {128, 192, 2, 2}};
     for (auto& t : direct) {
       tlhip_kernel_config_t c = direct_cfg(t[0], t[1], t[2], t[3]);
       if (gemm_direct_config_applicable(p, c, nullptr)) out.push_back(c);

@@ -72,7 +72,8 @@ __device__ __forceinline__ void wave_epilogue(float* patch, const float16_t (&ac
                                               int col0, const OutArgs& o) {
   constexpr int PW = TN * 32 + 4;
   constexpr int LPR = TN * 4;     // lanes per row, 8 columns each
-  constexpr int RPP = 64 / LPR;   // rows per pass
+  constexpr int RPP = 64 / LPR;   // rows per pass (TN = 3: 5 rows on 60 lanes, four lanes idle)
+  constexpr int PASSES = (32 + RPP - 1) / RPP;
   const int lrow = lane & 31, lk = lane >> 5;
 #pragma unroll
   for (int j = 0; j < TN; ++j)
@@ -80,6 +81,7 @@ __device__ __forceinline__ void wave_epilogue(float* patch, const float16_t (&ac
     for (int r = 0; r < 16; ++r) patch[(8 * (r >> 2) + 4 * lk + (r & 3)) * PW + j * 32 + lrow] = acc[j][r];
   __builtin_amdgcn_s_waitcnt(0xc07f);  // this wave's LDS writes have landed (lgkmcnt(0))
   const int rr0 = lane / LPR, cc = (lane % LPR) * 8;
+  const bool lane_used = rr0 < RPP;
   const int col = col0 + cc;
   const bool vec = o.vec_ok && col + 8 <= o.n;
   // The common chain, [bias] then [unary], keeps the lane's 8 bias values in
@@ -100,13 +102,13 @@ __device__ __forceinline__ void wave_epilogue(float* patch, const float16_t (&ac
     }
   }
 #pragma unroll 1
-  for (int p = 0; p < 32 / RPP; ++p) {
-    const int rr = p * RPP + rr0;
+  for (int p = 0; p < PASSES; ++p) {
+    const int rr = min(p * RPP + rr0, 31);
     const int row = row0 + rr;
     const float4_t a = *(const float4_t*)(patch + rr * PW + cc);
     const float4_t b = *(const float4_t*)(patch + rr * PW + cc + 4);
     float v[8] = {a[0], a[1], a[2], a[3], b[0], b[1], b[2], b[3]};
-    if (row < o.m) {
+    if (row < o.m && lane_used && p * RPP + rr0 < 32) {
       if (simple) {
 #pragma unroll
         for (int e = 0; e < 8; ++e) v[e] = apply_unary(unary, v[e] * o.alpha + bias[e]);

@@ -350,6 +350,7 @@ constexpr DirectTile kDirectTiles[] = {
     {128, 128, 2, 2},  // wave tile 64 x 64, 4 waves: two workgroups share a CU
     {256, 256, 2, 2},  // wave tile 128 x 128, 4 waves, one per SIMD
     {128, 256, 1, 4},  // wave tile 128 x 64, 4 waves, 48 KB of LDS: two workgroups share a CU
+    {128, 192, 2, 2},  // wave tile 64 x 96, 4 waves: M = 512 x N = 12288 makes exactly 256 tiles, one per CU
 };
 
 }  // namespace
@@ -361,7 +362,7 @@ bool gemm_direct_config_applicable(const Problem& p, const tlhip_kernel_config_t
       "activations must be f16",
       "K must be a multiple of 128",
       "group size must be a multiple of 32",
-      "tile (M, N, waves M, waves N) must be one of 256x256 2x4, 256x128 2x4, 128x256 2x4, 256x128 4x2, 128x128 2x2, 256x256 2x2, 128x256 1x4 with tile K 128",
+      "tile (M, N, waves M, waves N) must be one of 256x256 2x4, 256x128 2x4, 128x256 2x4, 256x128 4x2, 128x128 2x2, 256x256 2x2, 128x256 1x4, 128x192 2x2 with tile K 128",
   };
   auto fail = [&](int i) {
     if (why) *why = reasons[i];
@@ -409,6 +410,7 @@ int launch_gemm_direct(const Problem& p, const tlhip_kernel_config_t& c, hipStre
   else if (c.p0 == 128 && c.p1 == 256 && c.p3 == 1) rc = launch_direct_tile<1, 4, 4, 2>(a, g32, stream);
   else if (c.p0 == 128 && c.p1 == 256) rc = launch_direct_tile<2, 4, 2, 2>(a, g32, stream);
   else if (c.p0 == 128 && c.p1 == 128) rc = launch_direct_tile<2, 2, 2, 2>(a, g32, stream);
+  else if (c.p0 == 128 && c.p1 == 192) rc = launch_direct_tile<2, 2, 2, 3>(a, g32, stream);
   else rc = launch_direct_tile<4, 2, 2, 2>(a, g32, stream);
   if (rc) return rc;
   TLHIP_CHECK_HIP(hipGetLastError());
@@ -428,6 +430,7 @@ int prepare_gemm_direct_kernels() {
     if (!rc) rc = launch_direct_tile<1, 4, 4, 2>(a, g32, nullptr);
     if (!rc) rc = launch_direct_tile<2, 4, 2, 2>(a, g32, nullptr);
     if (!rc) rc = launch_direct_tile<2, 2, 2, 2>(a, g32, nullptr);
+    if (!rc) rc = launch_direct_tile<2, 2, 2, 3>(a, g32, nullptr);
     if (!rc) rc = launch_direct_tile<4, 2, 2, 2>(a, g32, nullptr);
     if (rc) return rc;
   }
