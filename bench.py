@@ -851,6 +851,18 @@ def main() -> int:
                             "config": list(cfg.as_tuple())})
             out.destroy()
         details["prefill_gemm_int4_4096x12288"] = pre
+        # the same GEMM on f32 activations with f32 output (the reference's default
+        # dtype): one cast launch into the stream's workspace + the f16 problem's kernel
+        pre32 = []
+        for m in (512, 2048):
+            x, _ = B.activations(m, k, dtype="f32", std=0.5)
+            out = be._alloc([m, n], "f32")
+            us = B.median_time(B.make_call([w], x, m, out, epilogue=be.makeEpilogue(bias, "silu"), out_dtype="f32"), 20)
+            fl = 2.0 * m * n * k
+            pre32.append({"m": m, "epilogue": "bias+silu", "us": round(us, 1), "tflops": round(fl / us / 1e6, 1),
+                          "config": list(be.selectedConfig(w, "f32", m, "f32").as_tuple())})
+            out.destroy()
+        details["prefill_gemm_int4_4096x12288_f32_activations"] = pre32
 
         # config 1: int8-row 1024 x 1024, f32 activations and output, M = 1
         pool, _ = B.weight_pool("int8-row", 1024, 1024, 0, "f32", pool_bytes=64e6)

@@ -260,7 +260,12 @@ int tlhip_gemm_prefill(const tlhip_qweight_t* w, const void* x, int x_dtype, int
 
 /* The matmul seam for a packed B operand: matmulQuantizedB
  * (matmul-ops.ts:113-182).  Routes small m to the GEMV kernels and larger m to
- * the prefill GEMM (or, for f32 activations, to GEMV passes of <= 16 rows). */
+ * the prefill GEMM.  f32 activations: up to 63 rows run as GEMV passes of <= 16
+ * rows in f32 arithmetic; from 64 rows on they are rounded to f16 (the operand
+ * type of the matrix cores; |x| above 65504 becomes inf) by a cast launch into
+ * the stream's workspace and take the prefill GEMM of the f16 problem, which is
+ * the configuration tlhip_selected_config then reports.  Like a K-sliced GEMV,
+ * a stream's first such call must not happen under graph capture. */
 int tlhip_matmul_quantized(const tlhip_qweight_t* w, const void* x, int x_dtype, int64_t m,
                            void* y, int y_dtype, float alpha, const tlhip_epilogue_t* epilogue,
                            tlhip_stream_t stream);

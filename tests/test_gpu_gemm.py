@@ -180,6 +180,45 @@ def test_gemm_rejects_f32_activations_and_falls_back_to_gemv_passes(be):
     assert rel_l2(y, O.linear(x, deq)) <= 2e-6
 
 
+@pytest.mark.parametrize("fmt,g,m,n,k,ydt", [
+    ("int4-grouped", 32, 64, 256, 512, "f32"),
+    ("int4-grouped", 32, 300, 384, 1024, "f32"),       # ragged rows and tiles
+    ("int4-grouped", 128, 2304, 256, 4096, "f32"),     # more rows than one workspace chunk holds (2048 at K = 4096)
+    ("int8-grouped", 64, 96, 256, 512, "f32"),
+    ("int8-row", 0, 130, 192, 768, "f32"),
+])
+def test_f32_activations_from_64_rows_take_the_matrix_cores(be, fmt, g, m, n, k, ydt):
+    """f32 activations, 64 rows or more: rounded to f16 once, then the prefill GEMM of
+    the f16 problem (no GEMV dispatch).  Checked against the oracle on the ORIGINAL f32
+    activations at the stated bar (rel-L2 <= 1e-3: the rounding of x to f16 costs about
+    3e-4), and against the oracle on the rounded activations at the prefill kernels' own
+    accuracy."""
+    rng = np.random.default_rng(m * 7 + k)
+    packed, scales, deq = make_weight(fmt, n, k, g, rng)
+    x = make_x(m, k, "f32", rng, std=0.5)
+    w = be.createQuantizedWeight(packed, scales, n, k, T.resolveWeightFormat(fmt_name(fmt, g), "f32"))
+    xt = be.ops.tensorFromArray(x, [m, k], "f32")
+    sel = be.selectedConfig(w, "f32", m, ydt)
+    assert sel.variant in (2, 3), sel.as_tuple()        # a tiled kernel
+    gemms = lambda: int(L.load().tlhip_counter(b"quant_gemm_dispatches"))
+    v0, d0 = T.getQuantGemvDispatchCount(), gemms()
+    y = be.linear(xt, w)
+    got = y.numpy()
+    assert T.getQuantGemvDispatchCount() == v0
+    assert gemms() == d0 + (2 if m > 2048 else 1)      # one launch per workspace chunk
+    want = O.linear(x, deq, threads=8)
+    assert rel_l2(got, want) <= REL_L2_TOL, rel_l2(got, want)
+    want16 = O.linear(f16_round(x).astype(np.float32), deq, threads=8)
+    assert rel_l2(got, want16) <= 4e-4, rel_l2(got, want16)
+    # the f16 problem on the same rounded rows gives the same bits
+    x16 = be.ops.tensorFromArray(f16_round(x), [m, k], "f16")
+    y16 = be.linear(x16, w, config=sel)
+    assert np.array_equal(y16.numpy(), got)
+    for t in (y, y16, x16, xt):
+        t.destroy()
+    w.destroy()
+
+
 @pytest.mark.parametrize("lo,hi", [(200.0, 4000.0), (2e-3, 8e-3)])
 @pytest.mark.parametrize("cfg", [None, (2, 128, 128, 64, 2, 2)])
 def test_prefill_scale_range(be, lo, hi, cfg):

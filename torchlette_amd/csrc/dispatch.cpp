@@ -374,11 +374,55 @@ int run_config(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t str
   return launch_gemv(p, c, stream);
 }
 
+// From this many rows on, f32 activations take the matrix-core route below; fewer rows
+// stay on the f32 arithmetic of the GEMV passes (at most four of them).
+constexpr int64_t kF32TiledFromRows = 64;
+
+// The problem an f32-activation prefill runs as: the same one on f16 activations.
+Problem as_f16_activations(const Problem& p) {
+  Problem q = p;
+  q.x_dtype = TLHIP_F16;
+  return q;
+}
+
+// f32 activations, many rows: the matrix cores take f16 operands, so the rows are
+// rounded to f16 once (a cast launch into the stream's workspace, as many rows at a time
+// as it holds) and go through the tiled kernel selected for the f16 problem.  Returns
+// false when this route does not apply (no tiled kernel for the shape, K too long for
+// the workspace) and nothing was launched.
+bool f32_rows_through_tiled(const Problem& p, hipStream_t stream, int* rc) {
+  if (p.x_dtype != TLHIP_F32 || p.m < kF32TiledFromRows || p.pro.kind != TLHIP_PRO_NONE) return false;
+  Problem q = as_f16_activations(p);
+  const tlhip_kernel_config_t c = select_config(q);
+  if (c.variant != VARIANT_TILED && c.variant != VARIANT_TILED_DIRECT) return false;
+  const int64_t capacity = (int64_t)(kSplitWorkspaceFloats * sizeof(float) / sizeof(_Float16));
+  int64_t rows = capacity / std::max<int64_t>(p.k, 1);
+  if (rows >= 256) rows -= rows % 256;  // whole tiles per chunk
+  if (rows < 32) return false;
+  float* workspace = nullptr;
+  int* counters = nullptr;
+  *rc = split_workspace(stream, &workspace, &counters);
+  if (*rc) return true;
+  const int yb = p.y_dtype == TLHIP_F16 ? 2 : 4;
+  for (int64_t m0 = 0; m0 < p.m; m0 += rows) {
+    q.m = std::min<int64_t>(rows, p.m - m0);
+    *rc = tlhip_cast((const float*)p.x + m0 * p.k, TLHIP_F32, workspace, TLHIP_F16, q.m * p.k, (tlhip_stream_t)stream);
+    if (*rc) return true;
+    q.x = workspace;
+    q.y = (char*)p.y + m0 * p.n * yb;
+    *rc = run_config(q, c, stream);
+    if (*rc) return true;
+  }
+  return true;
+}
+
 int matmul_with(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t stream) {
   if (c.variant == VARIANT_TILED || c.variant == VARIANT_TILED_DIRECT) return run_config(p, c, stream);
   if (p.m <= 16) return run_config(p, c, stream);
-  // f32 activations (or a shape the tiled kernel rejects) above 16 rows: GEMV
-  // passes of 16 rows.  Declared, slow: every pass streams the weights again.
+  int rc = TLHIP_OK;
+  if (f32_rows_through_tiled(p, stream, &rc)) return rc;
+  // f32 activations below kF32TiledFromRows rows (or a shape the tiled kernels reject):
+  // GEMV passes of 16 rows.  Declared, slow: every pass streams the weights again.
   const int xb = p.x_dtype == TLHIP_F16 ? 2 : 4, yb = p.y_dtype == TLHIP_F16 ? 2 : 4;
   for (int64_t m0 = 0; m0 < p.m; m0 += 16) {
     Problem q = p;
@@ -934,6 +978,8 @@ int tlhip_matmul_quantized(const tlhip_qweight_t* w, const void* x, int x_dtype,
     std::lock_guard<std::mutex> lock(g_tune_mutex);
     tune = (g_autotune_counter > 0 || env_autotune()) && !g_autotuning && g_tuned.count(problem_key(p)) == 0;
   }
+  // f32 activations on the matrix-core route run the f16 problem's winner: nothing to tune here
+  if (p.x_dtype == TLHIP_F32 && p.m >= kF32TiledFromRows) tune = false;
   if (tune) {
     // Lazy tuning at first dispatch (dispatch.ts:559-578), on the caller's stream; the
     // tuning launches write y, which the real launch below overwrites.  A problem whose
@@ -1006,6 +1052,11 @@ int tlhip_selected_config(const tlhip_qweight_t* w, int x_dtype, int64_t m, int 
   if (rc) return rc;
   if (!out) return set_error(TLHIP_ERR_INVALID, "selected_config: null output");
   *out = select_config(p);
+  if (p.x_dtype == TLHIP_F32 && p.m >= kF32TiledFromRows) {
+    // what tlhip_matmul_quantized launches for these rows: the f16 problem's tiled kernel
+    const tlhip_kernel_config_t c = select_config(as_f16_activations(p));
+    if (c.variant == VARIANT_TILED || c.variant == VARIANT_TILED_DIRECT) *out = c;
+  }
   return TLHIP_OK;
 }
 
