@@ -128,7 +128,10 @@ typedef struct {
 /* tlhip_init also imports the tuning file that ships next to the library
  * (<directory of libtlhip.so>/tuning/mi355x.json; the environment variable
  * TLHIP_TUNING_FILE names another file, "none" none), as importTuningCache would:
- * every binding runs the committed kernel choices, re-gated on applicability. */
+ * every binding runs the committed kernel choices, re-gated on applicability.
+ * The library serves ONE device per process, the one given here, and makes it the
+ * calling thread's current HIP device; a thread that calls the library later must
+ * have the same device current (allocations and launches go to the current device). */
 int tlhip_init(int device_index);
 int tlhip_shutdown(void);
 const char* tlhip_last_error(void);

@@ -18,6 +18,7 @@ void clear_error();
 bool is_initialised();
 hipStream_t resolve_stream(tlhip_stream_t s);  // NULL -> library stream
 int device_cu_count();
+int device_index();  // the device tlhip_init selected, -1 before
 
 #define TLHIP_CHECK_HIP(expr)                                                            \
   do {                                                                                   \

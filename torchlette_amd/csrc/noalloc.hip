@@ -63,6 +63,11 @@ extern "C" int tlhip_gemv_noalloc(const tlhip_qweight_t* w, const void* x, int x
   if (p.m == 0 || p.n == 0) return TLHIP_OK;
   int dev = -1;
   TLHIP_CHECK_HIP(hipGetDevice(&dev));
+  // the array's address differs from GPU to GPU: the one of the library's device is only
+  // right while that device is the calling thread's current one (as every launch needs)
+  if (dev != device_index())
+    return set_error(TLHIP_ERR_STATE, "gemv_noalloc: device %d is current, the library was initialised on device %d",
+                     dev, device_index());
   if (dev < 0 || dev >= kMaxDevices || !g_scratch_ptr[dev])
     return set_error(TLHIP_ERR_STATE, "gemv_noalloc: the scratch of device %d was not set up by tlhip_init", dev);
   // the kernel and configuration tlhip_gemv would run for this problem

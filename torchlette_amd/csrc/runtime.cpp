@@ -56,7 +56,11 @@ struct SplitWorkspace {
 };
 std::mutex g_ws_mutex;
 std::unordered_map<hipStream_t, SplitWorkspace> g_workspaces;
-std::unordered_map<hipGraphExec_t, hipStream_t> g_graphs;  // live graph -> its capture stream
+struct GraphRecord {
+  hipStream_t stream;  // the capture stream
+  bool holds_workspace;  // counted in that stream's SplitWorkspace::graphs
+};
+std::unordered_map<hipGraphExec_t, GraphRecord> g_graphs;  // live graphs
 std::unordered_set<hipStream_t> g_live_streams;            // the library stream and tlhip_stream_create's
 
 void free_workspaces() {
@@ -101,7 +105,9 @@ int split_workspace(hipStream_t stream, float** workspace, int** counters) {
     SplitWorkspace w{nullptr, nullptr, 0, true};
     TLHIP_CHECK_HIP(hipMalloc((void**)&w.workspace, kSplitWorkspaceFloats * sizeof(float)));
     hipError_t e = hipMalloc((void**)&w.counters, kSplitCounters * sizeof(int));
-    if (e == hipSuccess) e = hipMemset(w.counters, 0, kSplitCounters * sizeof(int));
+    // on the stream that will use them (not capturing: checked above), so the clear is
+    // ordered in front of the first launch whatever the stream's flags are
+    if (e == hipSuccess) e = hipMemsetAsync(w.counters, 0, kSplitCounters * sizeof(int), stream);
     if (e != hipSuccess) {
       (void)hipFree(w.workspace);
       if (w.counters) (void)hipFree(w.counters);
@@ -166,6 +172,7 @@ int problem_scratch(const Problem& p, hipStream_t stream, float** workspace, int
 }
 
 int device_cu_count() { return g_init ? g_props.multiProcessorCount : 0; }
+int device_index() { return g_init ? g_device : -1; }
 
 void count_gemv_dispatch() { g_gemv_dispatches++; }
 void count_gemm_dispatch() { g_gemm_dispatches++; }
@@ -332,6 +339,10 @@ int tlhip_stream_create(tlhip_stream_t* out) {
   {
     std::lock_guard<std::mutex> lock(g_ws_mutex);
     g_live_streams.insert(s);
+    // a handle value can come back after its stream was destroyed: a workspace that live
+    // graphs of the old stream keep is this stream's workspace again
+    auto it = g_workspaces.find(s);
+    if (it != g_workspaces.end()) it->second.stream_alive = true;
   }
   *out = s;
   return TLHIP_OK;
@@ -411,8 +422,8 @@ int tlhip_graph_end_capture(tlhip_stream_t stream, tlhip_graph_t* out) {
   if (e != hipSuccess) return set_error(TLHIP_ERR_DEVICE, "hipGraphInstantiate failed: %s", hipGetErrorString(e));
   {
     std::lock_guard<std::mutex> lock(g_ws_mutex);
-    g_graphs[exec] = s;
     auto it = g_workspaces.find(s);
+    g_graphs[exec] = GraphRecord{s, it != g_workspaces.end()};
     if (it != g_workspaces.end()) it->second.graphs++;
   }
   *out = exec;
@@ -429,7 +440,7 @@ int tlhip_graph_launch(tlhip_graph_t graph, tlhip_stream_t stream) {
     if (it == g_graphs.end()) return set_error(TLHIP_ERR_INVALID, "tlhip_graph_launch: unknown or destroyed graph");
     // the captured kernels use the capture stream's K-slice workspace; on another stream a
     // replay could run next to that stream's own launches on the same tiles and counters
-    if (it->second != s)
+    if (it->second.stream != s)
       return set_error(TLHIP_ERR_INVALID, "tlhip_graph_launch: a graph replays on the stream it was captured on");
   }
   TLHIP_CHECK_HIP(hipGraphLaunch(static_cast<hipGraphExec_t>(graph), s));
@@ -441,11 +452,13 @@ int tlhip_graph_destroy(tlhip_graph_t graph) {
   if (!graph) return TLHIP_OK;
   hipGraphExec_t exec = static_cast<hipGraphExec_t>(graph);
   hipStream_t origin = nullptr;
+  bool held = false;
   {
     std::lock_guard<std::mutex> lock(g_ws_mutex);
     auto it = g_graphs.find(exec);
     if (it == g_graphs.end()) return TLHIP_OK;  // idempotent, like destroy() in the reference
-    origin = it->second;
+    origin = it->second.stream;
+    held = it->second.holds_workspace;
     g_graphs.erase(it);
   }
   // a replay may still be in flight on the capture stream (the library stream is never destroyed
@@ -459,7 +472,7 @@ int tlhip_graph_destroy(tlhip_graph_t graph) {
   TLHIP_CHECK_HIP(hipGraphExecDestroy(exec));
   std::lock_guard<std::mutex> lock(g_ws_mutex);
   auto w = g_workspaces.find(origin);
-  if (w != g_workspaces.end() && w->second.graphs > 0) {
+  if (held && w != g_workspaces.end() && w->second.graphs > 0) {
     w->second.graphs--;
     release_if_unused(origin);
   }
