@@ -134,6 +134,34 @@ def test_tuning_cache_json_round_trip_and_autotune_toggle():
         T.importTuningCache("{}")
 
 
+def test_tuning_cache_import_survives_malformed_text():
+    """Every prefix of a valid cache text, pretty-printed text and junk: an error or a
+    clean import, never a crash, and a failed import leaves the cache as it was."""
+    import json
+    T.clearTuningCache()
+    entries = {"1_4096_4096_int4-grouped_g32_f16_f16": [0, 64, 1, 4, 1, 0, 0, 0],
+               "16_4096_12288_int4-grouped_g32_f16_f16": [1, 8, 4, 4, 2, 0, 1, 0]}
+    text = json.dumps({"version": 1, "entries": entries}, separators=(",", ":"))
+    for cut in range(len(text)):
+        try:
+            T.importTuningCache(text[:cut])
+            # only a text whose entries object is whole is taken (the parser reads no further)
+            assert cut >= len(text) - 1, cut
+            T.clearTuningCache()
+        except L.TlhipError:
+            assert T.exportTuningCache() == '{"version":1,"entries":{}}', cut
+    T.importTuningCache(json.dumps({"version": 1, "entries": entries}, indent=2))   # as json.dump writes it
+    assert json.loads(T.exportTuningCache())["entries"] == entries
+    T.clearTuningCache()
+    for junk in ('{"entries":', '{"entries":{"k":[1,2,3]}}', '{"entries":{"k":"v"}}', '{"entries":{k:[0]}}',
+                 '{"entries":{"a_b":[0,0,0,0,0,0,0,0]}}'):
+        try:
+            T.importTuningCache(junk)
+        except L.TlhipError:
+            pass
+    T.clearTuningCache()
+
+
 def test_format_names_resolve_like_the_reference():
     f = T.resolveWeightFormat("int8-64")
     assert f.elementType == "f16" and f.packing == T.QuantPacking("int8-grouped", 64, "f16")

@@ -1179,7 +1179,7 @@ int tlhip_tune_cache_import(const char* json) {
       v[i] = (int)strtol(p, &end, 10);
       if (end == p) return set_error(TLHIP_ERR_INVALID, "tune_cache_import: expected 8 integers for %s", key.c_str());
       p = end;
-      while (*p == ' ' || *p == ',') ++p;
+      while (*p == ' ' || *p == ',' || *p == '\n' || *p == '\t' || *p == '\r') ++p;
     }
     if (*p != ']') return set_error(TLHIP_ERR_INVALID, "tune_cache_import: expected ] after %s", key.c_str());
     ++p;
