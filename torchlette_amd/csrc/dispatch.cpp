@@ -312,17 +312,11 @@ std::vector<tlhip_kernel_config_t> candidates(const Problem& p) {
   return out;
 }
 
-// The winner of the nearest tuned problem of the same class (autotune.ts:269-300's
-// per-shape-class cache), re-gated on applicability.  "Near" = N and K each within a
-// factor of two and the same number of rows where the kernel family depends on it;
-// farther than that the hand heuristic knows more than a foreign winner does.
-bool class_config(const Problem& p, tlhip_kernel_config_t* out) {
-  std::lock_guard<std::mutex> lock(g_tune_mutex);
-  auto it = g_class_tuned.find(class_key(p));
-  if (it == g_class_tuned.end()) return false;
+// Caller holds g_tune_mutex.
+bool nearest_in_class(const Problem& p, const std::vector<ClassEntry>& list, tlhip_kernel_config_t* out) {
   double best = 1e30;
   bool found = false;
-  for (const auto& e : it->second) {
+  for (const auto& e : list) {
     const double dn = std::fabs(std::log2((double)e.n / (double)p.n));
     const double dk = std::fabs(std::log2((double)e.k / (double)p.k));
     const double dm = std::fabs(std::log2((double)e.m / (double)p.m));
@@ -335,6 +329,24 @@ bool class_config(const Problem& p, tlhip_kernel_config_t* out) {
     }
   }
   return found;
+}
+
+// The winner of the nearest tuned problem of the same class (autotune.ts:269-300's
+// per-shape-class cache), re-gated on applicability.  "Near" = N and K each within a
+// factor of two and the same number of rows where the kernel family depends on it;
+// farther than that the hand heuristic knows more than a foreign winner does.
+// The output type only changes the store at the end of a kernel, so where the class of
+// p's own output type holds nothing near, the class of the other output type is asked.
+bool class_config(const Problem& p, tlhip_kernel_config_t* out) {
+  std::lock_guard<std::mutex> lock(g_tune_mutex);
+  Problem other = p;
+  other.y_dtype = p.y_dtype == TLHIP_F16 ? TLHIP_F32 : TLHIP_F16;
+  for (const Problem* asked : {&p, (const Problem*)&other}) {
+    auto it = g_class_tuned.find(class_key(*asked));
+    if (it == g_class_tuned.end()) continue;
+    if (nearest_in_class(p, it->second, out)) return true;
+  }
+  return false;
 }
 
 tlhip_kernel_config_t select_config(const Problem& p) {
