@@ -186,9 +186,10 @@ def kernel_name_of(cfg) -> str:
             4: "gemv_xreg_kernel (16x16x32 f16, activations in registers)"}[cfg.variant]
 
 
-def cpu_step(cases, host_weights, host_x, threads: int) -> float:
+def cpu_step(cases, host_weights, host_x, threads: int, keep=None) -> float:
     """Seconds for one step on the CPU restatement: dequantise as the reference
-    does, then the CPU-backend matmul (f64 accumulate in k order, f32 store)."""
+    does, then the CPU-backend matmul (f64 accumulate in k order, f32 store).
+    `keep`: a list that receives the 15 outputs, in the order of `cases`."""
     from oracle import quant_oracle as O
     t0 = time.perf_counter()
     deq = {}
@@ -196,7 +197,9 @@ def cpu_step(cases, host_weights, host_x, threads: int) -> float:
         packed, scales = host_weights[(n, k)]
         deq[(n, k)] = O.dequant_int4_grouped(packed, scales, n, k, 32)
     for c in cases:
-        O.matmul_nt(host_x[(c["m"], c["k"])].astype(np.float32), deq[(c["n"], c["k"])], threads=threads)
+        y = O.matmul_nt(host_x[(c["m"], c["k"])].astype(np.float32), deq[(c["n"], c["k"])], threads=threads)
+        if keep is not None:
+            keep.append(y)
     return time.perf_counter() - t0
 
 
@@ -877,12 +880,26 @@ def main() -> int:
         from oracle import quant_oracle as O
         sec1 = cpu_step(cases, host_weights, host_x, 1)
         cores = O.max_threads()
-        secn = cpu_step(cases, host_weights, host_x, cores)
+        cpu_out = []
+        secn = cpu_step(cases, host_weights, host_x, cores, keep=cpu_out)
+        # the step that was timed, checked: each of its 15 calls once more on the GPU (same
+        # weights, activations and kernel configuration) against the host's result
+        worst = 0.0
+        for c, want in zip(cases, cpu_out):
+            c["call"]()
+            be.synchronize()
+            got = outs[(c["m"], c["n"])].numpy().astype(np.float64)
+            err = float(np.linalg.norm(got - want) / max(np.linalg.norm(want), 1e-30))
+            worst = max(worst, err)
+        if not worst <= 1e-3:
+            print(f"bench: the timed step's outputs differ from the CPU restatement (rel-L2 {worst:.3g} > 1e-3)", file=sys.stderr)
+            return 1
         result["cpu_baseline"] = {
             "value": round(step_bytes / sec1 / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
             "sample": "one full step (15 calls, dequantisation of the three weights included), C restatement of the "
                       "reference's CPU matmul: f64 accumulate in k order, f32 store",
             "seconds_per_step": round(sec1, 3),
+            "gpu_outputs_checked": {"calls": len(cases), "max_rel_l2": float(f"{worst:.3g}"), "bar": 1e-3},
             "all_cores": {"value": round(step_bytes / secn / 1e9, 4), "cores": cores, "seconds_per_step": round(secn, 3)}}
     if tuning_source == "tuned in this run" and not args.no_details:
         os.makedirs(os.path.dirname(args.tuning_cache), exist_ok=True)
