@@ -64,6 +64,8 @@ def algorithmic_bytes(fmt: str, n: int, k: int, g: int, m: int, x_bytes: int, y_
 
 
 class Bench:
+    only_missing = False  # --autotune-missing: tune() skips problems that have an entry of their own
+
     def __init__(self):
         import torchlette_amd as T
         from torchlette_amd import _lib as L
@@ -170,6 +172,13 @@ class Bench:
         pool, the three fastest once more, and the winner lands in the library's
         per-shape cache.  Returns its time per launch in microseconds."""
         L, be = self.L, self.be
+        if self.only_missing:
+            # --autotune-missing: problems that already have an entry of their own keep it
+            w0 = pool[0]
+            scheme, g = w0.format.packing.scheme, w0.format.packing.groupSize
+            key = f"{m}_{w0.shape[0]}_{w0.shape[1]}_{scheme}_g{0 if scheme == 'int8-row' else g}_{x.dtype}_{out_dtype}"
+            if key in json.loads(self.T.exportTuningCache())["entries"]:
+                return 0.0
         qws = (L.QWeight * len(pool))(*[be._qweight(w, False) for w in pool])
         xd = L.F16 if x.dtype == "f16" else L.F32
         yd = L.F16 if out_dtype == "f16" else L.F32
@@ -388,6 +397,9 @@ def main() -> int:
                     help="time the decode-token sections as stream launches only (no HIP graph capture / replay)")
     ap.add_argument("--autotune", action="store_true",
                     help="re-tune every case (weights rotating through HBM) even if a tuning cache file exists")
+    ap.add_argument("--autotune-missing", action="store_true",
+                    help="import the tuning cache file, tune only the cases it has no entry of their own for, and "
+                         "write the file back")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="for a counter run under rocprofv3 --pmc: 10 launches of each of the step's calls, then "
                          "three device-to-device copies of 256 MiB (the known size the counters are scaled by), and exit")
@@ -410,7 +422,12 @@ def main() -> int:
     # Kernel choices: a committed tuning cache (importTuningCache) when there is one,
     # else a tuning pass; --autotune forces the pass and rewrites the file.
     tuning_source = "heuristic defaults"
-    if not args.no_autotune and not args.autotune and os.path.exists(args.tuning_cache):
+    B.only_missing = False
+    if args.autotune_missing and os.path.exists(args.tuning_cache):
+        T.importTuningCache(open(args.tuning_cache).read())
+        B.only_missing = True
+        tuning_source = "tuned in this run"
+    elif not args.no_autotune and not args.autotune and os.path.exists(args.tuning_cache):
         T.importTuningCache(open(args.tuning_cache).read())
         tuning_source = os.path.relpath(args.tuning_cache, ROOT)
         args.no_autotune = True  # nothing left to tune
@@ -646,7 +663,7 @@ def main() -> int:
         # config 5: LM head 256000 x 2304 int8-row (f32 logits) and the MLP GEMVs
         lm_pool, _ = B.weight_pool("int8-row", 256000, 2304, 0, "f32", pool_bytes=1.25e9)
         lm = []
-        for m in (1, 8):
+        for m in (1, 4, 8, 16):
             x, _ = B.activations(m, 2304)
             out = be._alloc([m, 256000], "f32")
             if not args.no_autotune:
@@ -664,7 +681,7 @@ def main() -> int:
         # int8 with an f16 absmax per group of 64 (quantizeLinearWeight's default)
         g64_pool, _ = B.weight_pool("int8-grouped", 151936, 2048, 64, "f32", pool_bytes=1.0e9)
         lm64 = []
-        for m in (1, 8):
+        for m in (1, 4, 8, 16):
             x, _ = B.activations(m, 2048)
             out = be._alloc([m, 151936], "f32")
             if not args.no_autotune:

@@ -76,6 +76,7 @@ def test_shape_class_level_sits_between_the_tuned_winner_and_the_default(be):
         wide = be.createQuantizedWeight(np.zeros(40960 * 2048 // 8, np.uint32), np.zeros(40960 * 64, np.uint16), 40960, 2048,
                                         T.resolveWeightFormat("int4-32", "f32"))  # same class, N five times larger
         default_near = be.selectedConfig(near, "f16", 8, "f32").as_tuple()
+        default_near16 = be.selectedConfig(near, "f16", 16, "f32").as_tuple()
         default_far = be.selectedConfig(far, "f16", 8, "f32").as_tuple()
         default_wide = be.selectedConfig(wide, "f16", 8, "f32").as_tuple()
         seeded = L.KernelConfig.of(L.VARIANT_GEMV_MFMA, 4, 1, 2, 1)
@@ -87,6 +88,8 @@ def test_shape_class_level_sits_between_the_tuned_winner_and_the_default(be):
         # another class, or the same class but N more than a factor of two away: the heuristic default stays
         assert be.selectedConfig(far, "f16", 8, "f32").as_tuple() == default_far
         assert be.selectedConfig(wide, "f16", 8, "f32").as_tuple() == default_wide
+        # the same rows class but another row count: decode winners do not carry over
+        assert be.selectedConfig(near, "f16", 16, "f32").as_tuple() == default_near16
         # other rows class: untouched
         assert be.selectedConfig(near, "f16", 1, "f32").variant == L.VARIANT_GEMV
         # an exact winner beats the class

@@ -321,6 +321,10 @@ bool nearest_in_class(const Problem& p, const std::vector<ClassEntry>& list, tlh
     const double dk = std::fabs(std::log2((double)e.k / (double)p.k));
     const double dm = std::fabs(std::log2((double)e.m / (double)p.m));
     if (dn > 1.0 || dk > 1.0 || dm > 1.0) continue;
+    // decode kernels are tuned to their row count (the activations a workgroup stages and
+    // the registers a lane holds grow with it): the LM head's M = 8 winner measured 150 us
+    // at M = 16 against 106 us for the heuristic default
+    if (p.m <= 16 && e.m != p.m) continue;
     const double d = dn + 2.0 * dk + dm;  // K decides whether the activations fit LDS: weigh it
     if (d < best && config_applicable(p, e.config, nullptr)) {
       best = d;
@@ -333,7 +337,7 @@ bool nearest_in_class(const Problem& p, const std::vector<ClassEntry>& list, tlh
 
 // The winner of the nearest tuned problem of the same class (autotune.ts:269-300's
 // per-shape-class cache), re-gated on applicability.  "Near" = N and K each within a
-// factor of two and the same number of rows where the kernel family depends on it;
+// factor of two, the same number of rows up to 16 rows and within a factor of two above;
 // farther than that the hand heuristic knows more than a foreign winner does.
 // The output type only changes the store at the end of a kernel, so where the class of
 // p's own output type holds nothing near, the class of the other output type is asked.
