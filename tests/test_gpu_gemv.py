@@ -65,6 +65,29 @@ def test_gemv_matches_oracle(be, fmt, n, k, g, xdt, element, m):
         assert rel_l2(got, want) <= 2e-6  # f32 accumulate of exact products: order noise only
 
 
+@pytest.mark.parametrize("m", [9, 15, 16])
+def test_rows_whose_activations_fit_no_matrix_core_geometry_run_as_two_halves(be, m):
+    """K = 11008 (86 steps of 128): two K slices of 15 or 16 rows do not fit LDS and four do
+    not divide the steps.  The library then launches rows 0..7 and the rest on the matrix
+    cores (two dispatches) instead of the VALU kernel's pass per four rows; M = 9 still
+    fits as it is.  Heuristic defaults (no tuned entry can name such a pair)."""
+    n, k = 768, 11008
+    rng = np.random.default_rng(k + m)
+    packed, scales, deq = make_weight("int4-grouped", n, k, 32, rng)
+    x = make_x(m, k, "f16", rng)
+    saved = T.exportTuningCache()
+    T.clearTuningCache()
+    try:
+        before = T.getQuantGemvDispatchCount()
+        got = run_linear(be, "int4-grouped", packed, scales, n, k, 32, x, "f32")
+        launches = T.getQuantGemvDispatchCount() - before
+    finally:
+        T.importTuningCache(saved)
+    assert launches == (1 if m == 9 else 2), launches
+    want = O.linear(x.astype(np.float32), deq, threads=8)
+    assert rel_l2(got, want) <= 2e-6, rel_l2(got, want)
+
+
 @pytest.mark.parametrize("fmt,n,k,g", [
     ("int4-grouped", 4096, 4096, 32), ("int4-grouped", 12288, 4096, 32), ("int4-grouped", 4096, 12288, 32),
 ])

@@ -208,6 +208,18 @@ tlhip_kernel_config_t default_config(const Problem& p) {
       if ((wgs >= cus || t[0] == 64) && gemm_config_applicable(p, c, nullptr)) return c;
     }
   }
+  // three or four rows of int4 weights with K up to 8192, from 8 MB of weights on: the
+  // VALU kernel's 4x4x4 matrix-core form (tuned winner at 5120..14336 x 4096..8192:
+  // 7.8-12.2 us against 9.9-15.7 us for the skinny kernel below, which is ahead for
+  // longer K and for smaller matrices: 3584 x 3584 took 5.2 against 6.7 us)
+  const double packed_mb = (double)p.n * (double)p.k * (p.format == TLHIP_FMT_INT4_GROUPED ? 0.5 : 1.0) / 1e6;
+  if (p.m >= 3 && p.m <= 4 && p.k <= 8192 && packed_mb >= 8.0) {
+    for (int waves : {8, 4}) {
+      tlhip_kernel_config_t c = gemv_cfg(16, 1, waves, 1, 2);
+      c.p5 = 1;
+      if (gemv_config_applicable(p, c, nullptr)) return c;
+    }
+  }
   // three or more activation rows: the matrix-core kernel, whose time hardly depends on
   // M (measured at the Qwen3-8B shapes: M = 4 takes 5.3 / 10.9 / 11.2 us against 7.5 /
   // 13.4 / 15.1 us for the VALU kernel, whose dot products grow with M; at M = 2 the VALU
@@ -220,11 +232,23 @@ tlhip_kernel_config_t default_config(const Problem& p) {
         c.p5 = 1;
         if (gemv_mfma_config_applicable(p, c, nullptr)) return c;
       }
-    // the fewest K slices across workgroups whose activations fit LDS (measured best)
+    // the fewest K slices across workgroups whose activations fit LDS (measured best);
+    // the preferred split of K over a workgroup's waves first, then whatever closes (the
+    // tiles the waves park in LDS grow with the rounds a workgroup walks: K = 18944 at
+    // M = 16 fits with two K-split waves and not with four)
+    for (int ks = 1; ks <= 16; ks *= 2) {
+      const int preferred = p.n >= 32768 ? 1 : (ks > 1 ? 4 : 8);
+      for (int kw : {preferred, 8, 4, 2, 1})
+        for (int unroll : {2, 1, 4}) {
+          tlhip_kernel_config_t c = mfma_cfg(8, unroll, kw, ks);
+          if (gemv_mfma_config_applicable(p, c, nullptr)) return c;
+        }
+    }
+    // no geometry of the LDS-staged kernel closes: the activations in registers
     for (int ks = 1; ks <= 16; ks *= 2)
-      for (int unroll : {2, 1}) {
-        tlhip_kernel_config_t c = mfma_cfg(8, unroll, p.n >= 32768 ? 1 : (ks > 1 ? 4 : 8), ks);
-        if (gemv_mfma_config_applicable(p, c, nullptr)) return c;
+      for (int waves : {8, 4, 16}) {
+        tlhip_kernel_config_t c = xreg_cfg(waves, 1, 1, ks);
+        if (gemv_xreg_config_applicable(p, c, nullptr)) return c;
       }
   }
   return default_valu_config(p);
@@ -235,16 +259,24 @@ tlhip_kernel_config_t default_config(const Problem& p) {
 tlhip_kernel_config_t default_valu_config(const Problem& p) {
   const int cw = p.format == TLHIP_FMT_INT4_GROUPED ? 32 : 16;
   const int64_t nchunks = p.k / cw;
-  // lanes per row: every lane busy for short rows; all chunks of a row in flight at once
-  int lpr = 64;
-  if (nchunks % 64 != 0) lpr = (nchunks % 32 == 0) ? 32 : 16;
-  if (nchunks < 64) lpr = nchunks >= 32 ? 32 : 16;
-  if (p.n >= 32768) lpr = 16;  // long weight matrices: more rows per wave, walked with a stride
+  if (p.n >= 32768) {
+    // long weight matrices (an LM head): 16 lanes per row, more rows per wave, walked
+    // with a stride, all chunks of a row in flight at once
+    const int per_lane = (int)((nchunks + 15) / 16);
+    const int unroll = per_lane >= 8 ? 8 : (per_lane >= 4 ? 4 : 2);
+    const int r = unroll <= 2 ? 4 : (unroll <= 4 ? 2 : 1);
+    return gemv_cfg(16, r, 8, 1, unroll);
+  }
+  // Lanes per row and chunks in flight, from the tuned winners at 2048..18944 x
+  // 2048..18944 (M = 1): 16 lanes per row up to K = 4096 and 32 beyond, two chunks
+  // in flight per lane (four from twelve chunks per lane on, with eight waves).  More in
+  // flight per lane means fewer rows in flight per CU and measured 5-25 % slower.
+  // (a row need not be a whole number of passes: K = 11008 and 18944 measured 7.8 and
+  // 10.2 us with 32 lanes per row against 10.7 and 15.8 us with 16)
+  const int lpr = nchunks > 128 ? 32 : 16;
   const int per_lane = (int)((nchunks + lpr - 1) / lpr);
-  const int unroll = per_lane >= 8 ? 8 : (per_lane >= 4 ? 4 : 2);
-  int r = 1;
-  if (p.n >= 32768) r = unroll <= 2 ? 4 : (unroll <= 4 ? 2 : 1);
-  return gemv_cfg(lpr, r, p.n >= 32768 ? 8 : 4, 1, unroll);
+  const bool long_rows = per_lane >= 12;
+  return gemv_cfg(lpr, 1, long_rows ? 8 : 4, 1, long_rows ? 4 : 2);
 }
 
 std::vector<tlhip_kernel_config_t> candidates(const Problem& p) {
@@ -449,6 +481,28 @@ int matmul_with(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t st
     if (rc) return rc;
   }
   return TLHIP_OK;
+}
+
+// What the library launches for a problem when the caller names no configuration.
+// 9..16 rows whose activations fit no geometry of the matrix-core kernels (K = 11008 at
+// M = 15 or 16: two K slices of 16 rows take 176 KB of LDS, and four do not divide its
+// 86 steps) would fall to the VALU kernel, which streams the weights once per four rows;
+// two launches of at most 8 rows on the matrix cores stream them twice.
+int run_selected(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t stream) {
+  if (c.variant == VARIANT_GEMV && p.m > 8 && p.m <= 16 && p.pro.kind == TLHIP_PRO_NONE) {
+    Problem lo = p, hi = p;
+    lo.m = 8;
+    hi.m = p.m - 8;
+    const int xb = p.x_dtype == TLHIP_F16 ? 2 : 4, yb = p.y_dtype == TLHIP_F16 ? 2 : 4;
+    hi.x = (const char*)p.x + 8 * p.k * xb;
+    hi.y = (char*)p.y + 8 * p.n * yb;
+    const tlhip_kernel_config_t cl = select_config(lo);
+    if (cl.variant == VARIANT_GEMV_MFMA || cl.variant == VARIANT_GEMV_XREG) {
+      const int rc = run_config(lo, cl, stream);
+      return rc ? rc : matmul_with(hi, select_gemv_config(hi), stream);
+    }
+  }
+  return matmul_with(p, c, stream);
 }
 
 // One-field variations of `base` inside its kernel family, plus the heuristic defaults of
@@ -840,7 +894,7 @@ int tlhip_gemv(const tlhip_qweight_t* w, const void* x, int x_dtype, int64_t m, 
   int rc = make_problem(w, x, x_dtype, m, y, y_dtype, alpha, epilogue, &p, "gemv");
   if (rc) return rc;
   if (m > 16) return set_error(TLHIP_ERR_INVALID, "gemv: M=%lld above 16; use tlhip_gemm_prefill", (long long)m);
-  return run_config(p, select_gemv_config(p), resolve_stream(stream));
+  return run_selected(p, select_gemv_config(p), resolve_stream(stream));
 }
 
 int tlhip_gemv_grouped(const tlhip_gemv_problem_t* problems, int count, int x_dtype, int y_dtype, float alpha,
@@ -893,7 +947,7 @@ int tlhip_gemv_grouped_rows(const tlhip_gemv_problem_t* problems, int count, int
     }
   }
   for (int i = 0; i < count; ++i) {
-    int rc = matmul_with(ps[i], select_gemv_config(ps[i]), s);
+    int rc = run_selected(ps[i], select_gemv_config(ps[i]), s);
     if (rc) return rc;
   }
   return TLHIP_OK;
@@ -1007,7 +1061,7 @@ int tlhip_matmul_quantized(const tlhip_qweight_t* w, const void* x, int x_dtype,
     rc = autotune_problem(p, {}, o, s, nullptr);
     if (rc) return rc;
   }
-  return matmul_with(p, select_config(p), resolve_stream(stream));
+  return run_selected(p, select_config(p), resolve_stream(stream));
 }
 
 int tlhip_matmul_quantized_config(const tlhip_qweight_t* w, const void* x, int x_dtype, int64_t m, void* y,
