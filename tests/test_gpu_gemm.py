@@ -97,14 +97,17 @@ def test_direct_gemm_rejects_what_it_does_not_cover(be):
         be.linear(x8, w8, config=L.KernelConfig.of(3, 256, 256, 128, 2, 4))
 
 
-@pytest.mark.parametrize("m,n,k", [(17, 128, 64), (64, 64, 128), (100, 512, 1024), (1000, 256, 2048), (33, 1000, 4096)])
-def test_default_route_for_m_above_16_is_the_gemm(be, m, n, k):
+@pytest.mark.parametrize("m,n,k,passes", [(17, 128, 64, 0), (64, 64, 128, 0), (100, 512, 1024, 0), (1000, 256, 2048, 0),
+                                          (33, 1000, 4096, 3)])
+def test_default_route_for_m_above_16_is_the_gemm(be, m, n, k, passes):
+    """One tiled launch, except where a few rows on a long K make 16-row passes of the
+    decode kernel cheaper (33 rows, K = 4096: three passes)."""
     rng = np.random.default_rng(m + n + k)
     packed, scales, deq = make_weight("int4-grouped", n, k, 32, rng)
     x = make_x(m, k, "f16", rng, std=0.5)
     g0, v0 = T.getQuantGemmDispatchCount(), T.getQuantGemvDispatchCount()
     got = run(be, "int4-grouped", packed, scales, n, k, 32, x, "f16", fused=False)
-    assert T.getQuantGemmDispatchCount() == g0 + 1 and T.getQuantGemvDispatchCount() == v0
+    assert T.getQuantGemmDispatchCount() == g0 + (0 if passes else 1) and T.getQuantGemvDispatchCount() == v0 + passes
     want = O.linear(x.astype(np.float32), deq, threads=8)
     assert got.dtype == np.float16
     assert rel_l2(got, want) <= REL_L2_TOL, rel_l2(got, want)
@@ -178,6 +181,31 @@ def test_gemm_rejects_f32_activations_and_falls_back_to_gemv_passes(be):
     y = be.linear(xt, w).numpy()
     assert T.getQuantGemvDispatchCount() == v0 + 3      # 16 + 16 + 8 rows
     assert rel_l2(y, O.linear(x, deq)) <= 2e-6
+
+
+@pytest.mark.parametrize("m,passes", [(17, 2), (40, 3), (64, 4)])
+@pytest.mark.parametrize("ydt", ["f16", "f32"])
+def test_a_few_more_rows_than_16_stream_the_weights_once_per_16_rows(be, m, passes, ydt):
+    """17..64 rows on a small matrix: far too few tiles to fill the chip, so the library
+    runs the rows through the decode kernel 16 at a time (one dispatch per pass) instead
+    of one tiled launch.  Heuristic choice: no tuned entry for these problems."""
+    n, k = 1024, 2048
+    rng = np.random.default_rng(m)
+    packed, scales, deq = make_weight("int4-grouped", n, k, 32, rng)
+    x = make_x(m, k, "f16", rng, std=0.5)
+    w = be.createQuantizedWeight(packed, scales, n, k, T.resolveWeightFormat("int4-32", ydt))
+    xt = be.ops.tensorFromArray(x, [m, k], "f16")
+    bias = f16_round(rng.standard_normal(n) * 0.1)
+    bt = be.ops.tensorFromArray(bias, [n], "f16")
+    v0, g0 = T.getQuantGemvDispatchCount(), T.getQuantGemmDispatchCount()
+    y = be.linear(xt, w, bt, "silu", fused=True)
+    got = y.numpy()
+    assert T.getQuantGemvDispatchCount() == v0 + passes and T.getQuantGemmDispatchCount() == g0
+    want = O.linear(x.astype(np.float32), deq, bias.astype(np.float32), "silu", threads=8)
+    assert got.shape == (m, n)
+    assert rel_l2(got, want) <= (REL_L2_TOL if ydt == "f16" else 2e-6), rel_l2(got, want)
+    for t in (y, xt, bt, w):
+        t.destroy()
 
 
 @pytest.mark.parametrize("fmt,g,m,n,k,ydt", [

@@ -193,11 +193,17 @@ tlhip_kernel_config_t default_valu_config(const Problem& p);
 tlhip_kernel_config_t default_config(const Problem& p) {
   if (p.m > 16 && p.x_dtype == TLHIP_F16) {
     const int cus = device_cu_count() > 0 ? device_cu_count() : 256;
-    // int4: the kernel that keeps the weights packed up to the operand registers;
-    // 256 x 256 tiles once they fill the chip twice over, else 256 x 128
+    // int4: the kernel that keeps the weights packed up to the operand registers.
+    // Tiles by how many there are (best of every tile at 2048..28672 x 2048..12288, M =
+    // 32..4096): 256 x 256 once they fill the chip twice over; 128 x 256 with four waves
+    // (two workgroups share a CU) from 160 such tiles on, never more than 7 % behind the
+    // best there; below that 128 x 128, where the 256-row tiles measured 1.4-1.5 times
+    // slower (a launch of few tiles takes the time one workgroup needs to walk K).
     {
       const int64_t t256 = ((p.m + 255) / 256) * ((p.n + 255) / 256);
-      tlhip_kernel_config_t c = t256 >= 2 * cus ? direct_cfg(256, 256, 2, 4) : direct_cfg(256, 128, 2, 4);
+      const int64_t t128x256 = ((p.m + 127) / 128) * ((p.n + 255) / 256);
+      tlhip_kernel_config_t c = t256 >= 2 * cus ? direct_cfg(256, 256, 2, 4)
+                                : (t128x256 >= 160 ? direct_cfg(128, 256, 1, 4) : direct_cfg(128, 128, 2, 2));
       if (gemm_direct_config_applicable(p, c, nullptr)) return c;
     }
     // largest tile that still gives every CU a workgroup
@@ -483,6 +489,11 @@ int matmul_with(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t st
   return TLHIP_OK;
 }
 
+bool has_tuned_entry(const Problem& p) {
+  std::lock_guard<std::mutex> lock(g_tune_mutex);
+  return g_tuned.count(problem_key(p)) != 0;
+}
+
 // What the library launches for a problem when the caller names no configuration.
 // 9..16 rows whose activations fit no geometry of the matrix-core kernels (K = 11008 at
 // M = 15 or 16: two K slices of 16 rows take 176 KB of LDS, and four do not divide its
@@ -500,6 +511,28 @@ int run_selected(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t s
     if (cl.variant == VARIANT_GEMV_MFMA || cl.variant == VARIANT_GEMV_XREG) {
       const int rc = run_config(lo, cl, stream);
       return rc ? rc : matmul_with(hi, select_gemv_config(hi), stream);
+    }
+  }
+  // A few more rows than the decode kernels take, far fewer than fill the chip with
+  // tiles: a tiled launch of at most one round of 128 x 128 tiles takes the time ONE
+  // workgroup needs to walk K (measured 40-45 us per 4096 of K whatever M and N are, up
+  // to 512 resident tiles), the decode kernel streams the weights once per 16 rows (3 us
+  // + 1 us per 3.2 MB of packed weights: 6.3 / 9.9 / 11.9 us at the Qwen3-8B shapes).
+  // Below the break-even the rows go through the decode kernel 16 at a time.
+  // (A tuned entry of the problem itself is a measurement and stands.)
+  if ((c.variant == VARIANT_TILED || c.variant == VARIANT_TILED_DIRECT) && p.m > 16 && p.x_dtype == TLHIP_F16 &&
+      p.pro.kind == TLHIP_PRO_NONE && !has_tuned_entry(p)) {
+    const double packed_mb = (double)p.n * (double)p.k * (p.format == TLHIP_FMT_INT4_GROUPED ? 0.5 : 1.0) / 1e6;
+    const double pass_us = 3.0 + packed_mb / 3.2;
+    const int64_t passes = (p.m + 15) / 16;
+    const int64_t tiles = ((p.m + 127) / 128) * ((p.n + 127) / 128);
+    const double rounds = tiles <= 512 ? 1.0 : (double)tiles / 512.0;
+    const double tiled_us = 42.0 * (double)p.k / 4096.0 * rounds;
+    if ((double)passes * pass_us < 0.8 * tiled_us) {
+      Problem q = p;
+      q.m = 16;
+      const tlhip_kernel_config_t c16 = select_gemv_config(q);
+      if (c16.variant == VARIANT_GEMV_MFMA || c16.variant == VARIANT_GEMV_XREG) return matmul_with(p, c16, stream);
     }
   }
   return matmul_with(p, c, stream);
