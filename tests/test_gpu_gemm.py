@@ -98,10 +98,11 @@ def test_direct_gemm_rejects_what_it_does_not_cover(be):
 
 
 @pytest.mark.parametrize("m,n,k,passes", [(17, 128, 64, 0), (64, 64, 128, 0), (100, 512, 1024, 0), (1000, 256, 2048, 0),
-                                          (33, 1000, 4096, 3)])
+                                          (33, 1000, 4096, 1), (80, 1000, 4096, 2), (130, 1000, 4096, 3)])
 def test_default_route_for_m_above_16_is_the_gemm(be, m, n, k, passes):
-    """One tiled launch, except where a few rows on a long K make 16-row passes of the
-    decode kernel cheaper (33 rows, K = 4096: three passes)."""
+    """One tiled launch, except where a few rows on a long K make the decode kernel
+    cheaper: up to 64 rows per launch of it (33 rows, K = 4096: one; 80 rows: 64 + 16;
+    130 rows: 64 + 64 + 2)."""
     rng = np.random.default_rng(m + n + k)
     packed, scales, deq = make_weight("int4-grouped", n, k, 32, rng)
     x = make_x(m, k, "f16", rng, std=0.5)
@@ -183,13 +184,14 @@ def test_gemm_rejects_f32_activations_and_falls_back_to_gemv_passes(be):
     assert rel_l2(y, O.linear(x, deq)) <= 2e-6
 
 
-@pytest.mark.parametrize("m,passes", [(17, 2), (40, 3), (64, 4)])
+@pytest.mark.parametrize("m,passes", [(17, 1), (40, 1), (64, 1), (72, 2)])
 @pytest.mark.parametrize("ydt", ["f16", "f32"])
-def test_a_few_more_rows_than_16_stream_the_weights_once_per_16_rows(be, m, passes, ydt):
-    """17..64 rows on a small matrix: far too few tiles to fill the chip, so the library
-    runs the rows through the decode kernel 16 at a time (one dispatch per pass) instead
-    of one tiled launch.  Heuristic choice: no tuned entry for these problems."""
-    n, k = 1024, 2048
+def test_a_few_more_rows_than_16_go_through_the_decode_kernel(be, m, passes, ydt):
+    """17..72 rows on a small matrix: far too few tiles to fill the chip, so the library
+    runs the rows through the skinny matrix-core kernel (up to 64 rows per launch, one
+    dispatch per launch) instead of one tiled launch.
+    Heuristic choice: no tuned entry for these problems."""
+    n, k = 1024, 4096
     rng = np.random.default_rng(m)
     packed, scales, deq = make_weight("int4-grouped", n, k, 32, rng)
     x = make_x(m, k, "f16", rng, std=0.5)
@@ -211,7 +213,7 @@ def test_a_few_more_rows_than_16_stream_the_weights_once_per_16_rows(be, m, pass
 @pytest.mark.parametrize("fmt,g,m,n,k,ydt", [
     ("int4-grouped", 32, 64, 256, 512, "f32"),
     ("int4-grouped", 32, 300, 384, 1024, "f32"),       # ragged rows and tiles
-    ("int4-grouped", 128, 2304, 256, 4096, "f32"),     # more rows than one workspace chunk holds (2048 at K = 4096)
+    ("int4-grouped", 128, 4352, 256, 4096, "f32"),     # more rows than one workspace chunk holds (4096 at K = 4096)
     ("int8-grouped", 64, 96, 256, 512, "f32"),
     ("int8-row", 0, 130, 192, 768, "f32"),
 ])
@@ -233,7 +235,7 @@ def test_f32_activations_from_64_rows_take_the_matrix_cores(be, fmt, g, m, n, k,
     y = be.linear(xt, w)
     got = y.numpy()
     assert T.getQuantGemvDispatchCount() == v0
-    assert gemms() == d0 + (2 if m > 2048 else 1)      # one launch per workspace chunk
+    assert gemms() == d0 + (2 if m > 4096 else 1)      # one launch per workspace chunk
     want = O.linear(x, deq, threads=8)
     assert rel_l2(got, want) <= REL_L2_TOL, rel_l2(got, want)
     want16 = O.linear(f16_round(x).astype(np.float32), deq, threads=8)

@@ -65,6 +65,58 @@ def test_gemv_matches_oracle(be, fmt, n, k, g, xdt, element, m):
         assert rel_l2(got, want) <= 2e-6  # f32 accumulate of exact products: order noise only
 
 
+@pytest.mark.parametrize("m", [17, 24, 32, 33, 48, 64])
+@pytest.mark.parametrize("fmt,g,n,k,cfg", [
+    ("int4-grouped", 32, 1000, 2048, (1, 8, 2, 8, 1)),            # K split over the waves of a workgroup
+    ("int4-grouped", 32, 1536, 2048, (1, 8, 2, 4, 2, 0, 1)),      # ... and over two workgroups, whole-line loads
+    ("int4-grouped", 128, 520, 1024, (1, 4, 1, 1, 1)),            # a wave owns its row blocks
+    ("int4-grouped", 32, 2048, 4096, (1, 8, 1, 2, 4)),            # four K slices
+    ("int8-row", 0, 1000, 2304, (1, 8, 2, 1, 2, 0, 1)),
+    ("int8-grouped", 64, 768, 2048, (1, 4, 2, 4, 2)),
+])
+def test_seventeen_to_64_rows_in_one_launch_of_the_matrix_core_gemv(be, fmt, g, n, k, cfg, m):
+    """Two or four tiles of 16 activation rows per weight row block: the weights stream once
+    for all rows.  Against the oracle (f32 out: exact products, order noise only), and
+    bit-identical to the same configuration run on the first 16 rows alone wherever the
+    launch geometry does not enter the arithmetic (every row's sum is formed in the same
+    order whatever the number of tiles)."""
+    rng = np.random.default_rng(zlib.crc32(repr((fmt, n, k, m, cfg)).encode()))
+    packed, scales, deq = make_weight(fmt, n, k, g, rng)
+    x = make_x(m, k, "f16", rng)
+    bias = rng.standard_normal(n).astype(np.float32)
+    c = L.KernelConfig.of(*cfg)
+    before = T.getQuantGemvDispatchCount()
+    try:
+        got = run_linear(be, fmt, packed, scales, n, k, g, x, "f32", bias=bias, act="silu", fused=True, config=c)
+    except L.TlhipError as e:
+        if "do not fit LDS" in str(e) and m > 32:
+            pytest.skip("four tiles of rows: this geometry's activations and parked tiles exceed LDS")
+        raise
+    assert T.getQuantGemvDispatchCount() == before + 1
+    want = O.linear(x.astype(np.float32), deq, bias, "silu", threads=8)
+    assert got.shape == (m, n)
+    assert rel_l2(got, want) <= 2e-6, rel_l2(got, want)
+    first = run_linear(be, fmt, packed, scales, n, k, g, x[:16].copy(), "f32", bias=bias, act="silu", fused=True, config=c)
+    assert np.array_equal(got[:16], first)
+    got16 = run_linear(be, fmt, packed, scales, n, k, g, x, "f16", config=c)
+    assert got16.dtype == np.float16
+    assert rel_l2(got16, O.linear(x.astype(np.float32), deq, threads=8)) <= REL_L2_TOL
+
+
+def test_more_than_16_rows_reject_what_the_matrix_core_gemv_does_not_cover(be):
+    rng = np.random.default_rng(5)
+    packed, scales, _ = make_weight("int4-grouped", 256, 1024, 32, rng)
+    w = be.createQuantizedWeight(packed, scales, 256, 1024, T.resolveWeightFormat("int4-32", "f32"))
+    x = be.ops.tensorFromArray(make_x(40, 1024, "f16", rng), [40, 1024], "f16")
+    with pytest.raises(L.TlhipError, match="at most 8 waves"):
+        be.linear(x, w, config=L.KernelConfig.of(1, 16, 1, 16, 1))
+    with pytest.raises(L.TlhipError, match="1 or 2 above 32 rows"):
+        be.linear(x, w, config=L.KernelConfig.of(1, 8, 4, 8, 1))
+    x65 = be.ops.tensorFromArray(make_x(65, 1024, "f16", rng), [65, 1024], "f16")
+    with pytest.raises(L.TlhipError, match="M must be"):
+        be.linear(x65, w, config=L.KernelConfig.of(1, 8, 1, 8, 1))
+
+
 @pytest.mark.parametrize("m", [9, 15, 16])
 def test_rows_whose_activations_fit_no_matrix_core_geometry_run_as_two_halves(be, m):
     """K = 11008 (86 steps of 128): two K slices of 15 or 16 rows do not fit LDS and four do

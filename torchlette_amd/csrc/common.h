@@ -109,7 +109,7 @@ int launch_gemm_direct(const Problem& p, const tlhip_kernel_config_t& c, hipStre
 // zero whenever no launch is in flight.  One per stream, so launches on different
 // streams never share it; created on the stream's first use, which must not
 // happen while the stream is being captured.
-constexpr size_t kSplitWorkspaceFloats = 4u << 20;  // 16 MiB
+constexpr size_t kSplitWorkspaceFloats = 8u << 20;  // 32 MiB
 constexpr int kSplitCounters = 1 << 16;
 int split_workspace(hipStream_t stream, float** workspace, int** counters);
 // The scratch a launch of `p` combines its K slices through: the caller's, or the

@@ -75,6 +75,29 @@ __device__ __forceinline__ float apply_epilogue(const DevEpilogue& ep, float v, 
   return v;
 }
 
+// The same on COUNT values of one output column: the ops are the outer loop, unrolled
+// over the fixed capacity with constant indices, so that the epilogue's fields stay in
+// scalar registers however many values the caller holds (a run-time index into the
+// kernel arguments makes the compiler copy them to scratch memory).
+template <int COUNT>
+__device__ __forceinline__ void apply_epilogue_all(const DevEpilogue& ep, float (&v)[COUNT], int64_t col) {
+#pragma unroll
+  for (int i = 0; i < TLHIP_MAX_EPILOGUE_OPS; ++i) {
+    if (i < ep.n_ops) {
+      if (ep.kind[i] == TLHIP_EPI_BIAS) {
+        float b;
+        if (ep.input_dtype[i] == TLHIP_F16) b = (float)((const _Float16*)ep.input[i])[col];
+        else b = ((const float*)ep.input[i])[col];
+#pragma unroll
+        for (int j = 0; j < COUNT; ++j) v[j] += b;
+      } else if (ep.kind[i] == TLHIP_EPI_UNARY) {
+#pragma unroll
+        for (int j = 0; j < COUNT; ++j) v[j] = apply_unary(ep.unary[i], v[j]);
+      }
+    }
+  }
+}
+
 __device__ __forceinline__ void store_out(void* y, int y_dtype, int64_t idx, float v) {
   if (y_dtype == TLHIP_F16) ((_Float16*)y)[idx] = (_Float16)v;
   else ((float*)y)[idx] = v;

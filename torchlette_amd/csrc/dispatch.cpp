@@ -309,11 +309,11 @@ std::vector<tlhip_kernel_config_t> candidates(const Problem& p) {
           if (gemv_config_applicable(p, c, nullptr)) out.push_back(c);
         }
   }
-  if (p.m <= 16) {
+  if (p.m <= 64) {  // above 16 rows: two or four tiles of rows per weight row block
     for (int waves : {4, 8, 16})
       for (int unroll : {1, 2, 4})
         for (int kw : {1, 2, 4, 8, 16})
-          for (int ks : {1, 2, 4, 8}) {
+          for (int ks : {1, 2, 4, 8, 16}) {
             if (kw > waves) continue;
             tlhip_kernel_config_t c = mfma_cfg(waves, unroll, kw, ks);
             if (gemv_mfma_config_applicable(p, c, nullptr)) out.push_back(c);
@@ -359,10 +359,12 @@ bool nearest_in_class(const Problem& p, const std::vector<ClassEntry>& list, tlh
     const double dk = std::fabs(std::log2((double)e.k / (double)p.k));
     const double dm = std::fabs(std::log2((double)e.m / (double)p.m));
     if (dn > 1.0 || dk > 1.0 || dm > 1.0) continue;
-    // decode kernels are tuned to their row count (the activations a workgroup stages and
-    // the registers a lane holds grow with it): the LM head's M = 8 winner measured 150 us
-    // at M = 16 against 106 us for the heuristic default
-    if (p.m <= 16 && e.m != p.m) continue;
+    // Winners do not carry over to another row count.  Decode kernels are tuned to theirs
+    // (the activations a workgroup stages and the registers a lane holds grow with it: the
+    // LM head's M = 8 winner measured 150 us at M = 16 against 106 us for the heuristic default
+    // at M = 16; a prefill winner is fitted to its number of tiles: the 256 x 128 tile
+    // that wins M = 512 at 12288 x 4096 took 71 us at M = 256 against 54 us for the default)
+    if (e.m != p.m) continue;
     const double d = dn + 2.0 * dk + dm;  // K decides whether the activations fit LDS: weigh it
     if (d < best && config_applicable(p, e.config, nullptr)) {
       best = d;
@@ -375,7 +377,7 @@ bool nearest_in_class(const Problem& p, const std::vector<ClassEntry>& list, tlh
 
 // The winner of the nearest tuned problem of the same class (autotune.ts:269-300's
 // per-shape-class cache), re-gated on applicability.  "Near" = N and K each within a
-// factor of two, the same number of rows up to 16 rows and within a factor of two above;
+// factor of two and the same number of rows;
 // farther than that the hand heuristic knows more than a foreign winner does.
 // The output type only changes the store at the end of a kernel, so where the class of
 // p's own output type holds nothing near, the class of the other output type is asked.
@@ -473,6 +475,8 @@ bool f32_rows_through_tiled(const Problem& p, hipStream_t stream, int* rc) {
 int matmul_with(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t stream) {
   if (c.variant == VARIANT_TILED || c.variant == VARIANT_TILED_DIRECT) return run_config(p, c, stream);
   if (p.m <= 16) return run_config(p, c, stream);
+  // 17..64 rows in one launch of the skinny matrix-core kernel (two or four tiles of 16 rows)
+  if (p.m <= 64 && c.variant == VARIANT_GEMV_MFMA && gemv_mfma_config_applicable(p, c, nullptr)) return run_config(p, c, stream);
   int rc = TLHIP_OK;
   if (f32_rows_through_tiled(p, stream, &rc)) return rc;
   // f32 activations below kF32TiledFromRows rows (or a shape the tiled kernels reject):
@@ -487,6 +491,29 @@ int matmul_with(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t st
     if (rc) return rc;
   }
   return TLHIP_OK;
+}
+
+// 17..64 rows in ONE launch of the skinny matrix-core kernel: eight waves, two iterations
+// in flight, the fewest K slices across workgroups whose activations fit LDS, and the
+// fewest K-split waves per row block that still give every CU a workgroup (measured best
+// or within 5 % of it at 4096..28672 x 4096..12288, M = 24..64).
+bool rows_in_one_launch_config(const Problem& p, tlhip_kernel_config_t* out) {
+  if (p.m <= 16 || p.m > 64 || p.x_dtype != TLHIP_F16) return false;
+  const int cus = device_cu_count() > 0 ? device_cu_count() : 256;
+  const int64_t nblocks = (p.n + 15) / 16;
+  for (int ks = 1; ks <= 16; ks *= 2) {
+    int fill = 1;  // K-split waves per row block: 8 / fill row blocks per workgroup
+    while (fill < 8 && (nblocks * fill / 8) * ks < cus) fill *= 2;
+    for (int kw : {fill, 8, 4, 2, 1})
+      for (int unroll : {2, 1}) {
+        const tlhip_kernel_config_t c = mfma_cfg(8, unroll, kw, ks);
+        if (gemv_mfma_config_applicable(p, c, nullptr)) {
+          *out = c;
+          return true;
+        }
+      }
+  }
+  return false;
 }
 
 bool has_tuned_entry(const Problem& p) {
@@ -518,7 +545,8 @@ int run_selected(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t s
   // workgroup needs to walk K (measured 40-45 us per 4096 of K whatever M and N are, up
   // to 512 resident tiles), the decode kernel streams the weights once per 16 rows (3 us
   // + 1 us per 3.2 MB of packed weights: 6.3 / 9.9 / 11.9 us at the Qwen3-8B shapes).
-  // Below the break-even the rows go through the decode kernel 16 at a time.
+  // Below the break-even the rows go through the decode kernel: up to 64 per launch, or
+  // 16 at a time where the activations of more rows fit no geometry.
   // (A tuned entry of the problem itself is a measurement and stands.)
   if ((c.variant == VARIANT_TILED || c.variant == VARIANT_TILED_DIRECT) && p.m > 16 && p.x_dtype == TLHIP_F16 &&
       p.pro.kind == TLHIP_PRO_NONE && !has_tuned_entry(p)) {
@@ -528,6 +556,38 @@ int run_selected(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t s
     const int64_t tiles = ((p.m + 127) / 128) * ((p.n + 127) / 128);
     const double rounds = tiles <= 512 ? 1.0 : (double)tiles / 512.0;
     const double tiled_us = 42.0 * (double)p.k / 4096.0 * rounds;
+    // Up to 64 rows per launch of the decode kernel: 1.2-1.6 times a 16-row pass for two
+    // tiles of rows, 2.3-3.2 times for four (the activations a workgroup stages grow with
+    // the rows, and their K slices are combined across workgroups).  More rows go 64 at a
+    // time while that beats the tiles (128 rows at 4096 x 4096: 2 x 16 us against 49 us).
+    auto chunk_us = [&](int64_t rows) { return pass_us * (rows <= 16 ? 1.0 : (rows <= 32 ? 1.5 : 2.7)); };
+    const int64_t full = p.m / 64, rest = p.m % 64;
+    const double rows_us = (double)full * chunk_us(64) + (rest ? chunk_us(rest) : 0.0);
+    if (rows_us < 0.9 * tiled_us) {
+      const int xb = 2, yb = p.y_dtype == TLHIP_F16 ? 2 : 4;
+      bool ok = true;
+      tlhip_kernel_config_t cfg64, cfg_rest;
+      Problem q64 = p, qr = p;
+      q64.m = 64;
+      qr.m = rest;
+      if (full) ok = rows_in_one_launch_config(q64, &cfg64);
+      if (ok && rest > 16) ok = rows_in_one_launch_config(qr, &cfg_rest);
+      if (ok && rest > 0 && rest <= 16) {
+        cfg_rest = select_gemv_config(qr);
+        ok = cfg_rest.variant == VARIANT_GEMV_MFMA || cfg_rest.variant == VARIANT_GEMV_XREG || rest <= 4;
+      }
+      if (ok) {
+        for (int64_t m0 = 0; m0 < p.m; m0 += 64) {
+          Problem q = p;
+          q.m = std::min<int64_t>(64, p.m - m0);
+          q.x = (const char*)p.x + m0 * p.k * xb;
+          q.y = (char*)p.y + m0 * p.n * yb;
+          const int rc = run_config(q, q.m == 64 ? cfg64 : cfg_rest, stream);
+          if (rc) return rc;
+        }
+        return TLHIP_OK;
+      }
+    }
     if ((double)passes * pass_us < 0.8 * tiled_us) {
       Problem q = p;
       q.m = 16;

@@ -15,6 +15,9 @@ struct MfmaGeometry {
   size_t lds_bytes;
   size_t patch_offset;  // bytes of activations and parked tiles in front of the patches
 };
+// Tiles of 16 activation rows per weight row block: 1, 2 or 4 (M <= 16 / 32 / 64).
+static int row_tiles(int64_t m) { return m <= 16 ? 1 : (m <= 32 ? 2 : 4); }
+
 static bool mfma_geometry(int64_t nblocks, int64_t k, int64_t m, int waves, int kw, int ks, size_t patch_bytes, MfmaGeometry* out) {
   const int threads = waves * 64;
   const int blocks_per_wg = waves / kw;
@@ -31,7 +34,7 @@ static bool mfma_geometry(int64_t nblocks, int64_t k, int64_t m, int waves, int 
     if (sets > nwgblocks) sets = nwgblocks;
     if (sets < 1) sets = 1;
     const int64_t rounds = (nwgblocks + sets - 1) / sets;
-    const size_t parked = kw > 1 ? (size_t)rounds * waves * 1024 : 0;
+    const size_t parked = kw > 1 ? (size_t)rounds * waves * 1024 * row_tiles(m) : 0;
     const size_t lds = x_bytes + parked + patch_bytes;
     if (lds * per_cu <= kXLdsBudget) {
       out->grid = (int)(sets * ks);
@@ -54,10 +57,10 @@ static bool mfma_applicable(const Problem& p, int64_t nblocks, const tlhip_kerne
       "not the gemv_mfma variant",
       "waves per workgroup must be 4, 8 or 16 (16: at most two iterations in flight)",
       "activations must be f16",
-      "M must be 1..16",
+      "M must be 1..16 (17..64 for one problem with at most 8 waves per workgroup)",
       "K must be a multiple of 128 (int4) or 64 (int8)",
       "group size must be a multiple of 32 (int4) or 64 (int8)",
-      "iterations in flight must be 1, 2 or 4",
+      "iterations in flight must be 1, 2 or 4 (1 or 2 above 32 rows)",
       "K-split waves must be a power of two that divides the waves per workgroup",
       "activations (M x K/slices f16) plus one parked tile per round and wave do not fit LDS",
       "K slices must be a power of two (1..16) that divides K/128 (int4) or K/64 (int8)",
@@ -74,7 +77,9 @@ static bool mfma_applicable(const Problem& p, int64_t nblocks, const tlhip_kerne
   if (c.p0 != 4 && c.p0 != 8 && c.p0 != 16) return fail(1);
   if (c.p0 == 16 && c.p1 > 2) return fail(1);
   if (p.x_dtype != TLHIP_F16) return fail(2);
-  if (p.m < 1 || p.m > 16) return fail(3);
+  if (p.m < 1 || p.m > 64) return fail(3);
+  if (p.m > 16 && c.p0 > 8) return fail(3);
+  if (p.m > 32 && c.p1 > 2) return fail(6);  // four tiles of rows and four iterations in flight: more registers than a lane has
   const int kper = p.format == TLHIP_FMT_INT4_GROUPED ? 128 : 64;
   if (p.k % kper != 0) return fail(4);
   if (p.format == TLHIP_FMT_INT4_GROUPED && p.group_size % 32 != 0) return fail(5);
@@ -94,7 +99,8 @@ static bool mfma_applicable(const Problem& p, int64_t nblocks, const tlhip_kerne
   MfmaGeometry geo;
   if (!mfma_geometry(nblocks, p.k, p.m, c.p0, kw, ks, line_patch_bytes(c), &geo)) return fail(8);
   if ((iters / ks) % c.p1 != 0) return fail(11);
-  if (ks > 1 && (nblocks > scratch_counters(p) || (size_t)nblocks * ks * 256 > scratch_tile_floats(p))) return fail(10);
+  if (ks > 1 && (nblocks > scratch_counters(p) || (size_t)nblocks * ks * 256 * row_tiles(p.m) > scratch_tile_floats(p)))
+    return fail(10);
   return true;
 }
 
@@ -111,7 +117,7 @@ bool gemv_mfma_group_applicable(const Problem* ps, int count, const tlhip_kernel
   }
   int64_t nblocks = 0;
   for (int i = 0; i < count; ++i) {
-    if (ps[i].x != ps[0].x || ps[i].m != ps[0].m || ps[i].format != ps[0].format || ps[i].group_size != ps[0].group_size ||
+    if ((count > 1 && ps[i].m > 16) || ps[i].x != ps[0].x || ps[i].m != ps[0].m || ps[i].format != ps[0].format || ps[i].group_size != ps[0].group_size ||
         ps[i].k != ps[0].k || ps[i].x_dtype != ps[0].x_dtype || ps[i].y_dtype != ps[0].y_dtype || ps[i].alpha != ps[0].alpha) {
       if (why) *why = "the problems of a group share activations, rows, format, group size, K, output type and alpha";
       return false;
@@ -179,8 +185,10 @@ int launch_gemv_mfma_group(const Problem* ps, int count, const tlhip_kernel_conf
   const int grid = geo.grid;
   // the single-problem instances keep the problem's fields in scalar registers without a
   // table lookup per batch (measured 0.7-1.4 us per launch at the 9-28 MB decode shapes)
-  const int rc = a.count == 1 ? launch_mfma_single(p.format, p.group_size, p.k, unroll, c.p5, a, grid, threads, lds_bytes, stream)
-                              : launch_mfma_grouped(p.format, p.group_size, p.k, unroll, c.p5, a, grid, threads, lds_bytes, stream);
+  int rc;
+  if (p.m > 16) rc = launch_mfma_rows(row_tiles(p.m), p.format, p.group_size, p.k, unroll, c.p5, a, grid, threads, lds_bytes, stream);
+  else if (a.count == 1) rc = launch_mfma_single(p.format, p.group_size, p.k, unroll, c.p5, a, grid, threads, lds_bytes, stream);
+  else rc = launch_mfma_grouped(p.format, p.group_size, p.k, unroll, c.p5, a, grid, threads, lds_bytes, stream);
   if (rc) return rc;
   TLHIP_CHECK_HIP(hipGetLastError());
   for (int i = 0; i < a.count; ++i) count_gemv_dispatch();
@@ -202,8 +210,9 @@ int launch_mfma_single(int format, int group_size, int64_t k, int unroll, int li
 int prepare_mfma_single() { return prepare_mfma_instances<false>(); }
 
 int prepare_gemv_mfma_kernels() {
-  const int rc = prepare_mfma_single();
-  return rc ? rc : prepare_mfma_grouped();
+  int rc = prepare_mfma_single();
+  if (!rc) rc = prepare_mfma_grouped();
+  return rc ? rc : prepare_mfma_rows();
 }
 
 }  // namespace tlhip

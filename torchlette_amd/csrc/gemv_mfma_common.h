@@ -31,11 +31,11 @@ __device__ __forceinline__ void transpose4(uint32_t& r0, uint32_t& r1, uint32_t&
 }
 
 // The last arriver's sum over the ks (a power of two >= 2) published tiles of a row
-// block, in slice order.  `tiles` + sl*256 + at + 16*q (q = 0..3) are this lane's four
+// block, in slice order.  `tiles` + sl*stride + at + 16*q (q = 0..3) are this lane's four
 // values of slice sl.  The loads of four slices are issued together: one load per
 // loop iteration (the sum needs it at once) made every slice a round trip to L2 of
 // its own, about 1 us each.
-__device__ __forceinline__ float4_t sum_slices(const float* tiles, int ks, int at) {
+__device__ __forceinline__ float4_t sum_slices(const float* tiles, int ks, int at, int stride = 256) {
   float4_t sum = {0.f, 0.f, 0.f, 0.f};
   for (int sl0 = 0; sl0 < ks; sl0 += 4) {
     float v[4][4];
@@ -44,7 +44,7 @@ __device__ __forceinline__ float4_t sum_slices(const float* tiles, int ks, int a
       const int sl = min(sl0 + j, ks - 1);  // ks = 2: the second slice again, not added below
 #pragma unroll
       for (int q = 0; q < 4; ++q)
-        v[j][q] = __hip_atomic_load(tiles + sl * 256 + at + 16 * q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        v[j][q] = __hip_atomic_load(tiles + sl * stride + at + 16 * q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 #pragma unroll
     for (int j = 0; j < 4; ++j) {

@@ -1,5 +1,6 @@
-// Skinny GEMM (2 <= M <= 16 activation rows) over packed weights on the matrix
-// cores: the weights are streamed from HBM exactly once whatever M is.
+// Skinny GEMM (2 <= M <= 16 activation rows, and 17..64 rows as MT = 2 or 4 tiles of 16
+// rows per weight row block) over packed weights on the matrix cores: the weights are
+// streamed from HBM exactly once whatever M is.
 //
 // Weight rows are processed in blocks of 16.  A wave feeds v_mfma_f32_16x16x32_f16 with
 //   A = activations  (lane l supplies x[m = l%16][8 k-values of sub-block l/16])
@@ -110,7 +111,11 @@ __device__ __forceinline__ int x_unit(int t, int g, int m, int row_units) {
 // consumed exactly as before.  A read-only kernel streams the LM head's 590 MB in
 // 84-86 us with the first load shape and in 94-95 us (plain) or 102-106 us (hint) with
 // the second.
-template <int FMT, int U, bool WIDE, int MAXT, bool LINE, bool GROUP>
+//
+// MT (1, 2, 4): tiles of 16 activation rows per weight row block.  A dequantised weight
+// operand feeds MT MFMAs, one per tile, and everything that holds a 16 x 16 result
+// (accumulators, parked tiles, K-slice tiles in the workspace) holds MT of them.
+template <int FMT, int U, bool WIDE, int MAXT, bool LINE, bool GROUP, int MT = 1>
 __global__ __launch_bounds__(MAXT) void gemv_mfma_kernel(const MfmaArgs a) {
   static_assert(!LINE || U % 2 == 0, "whole-line loads: an even number of iterations in flight");
   using Tr = MfmaTraits<FMT>;
@@ -126,7 +131,9 @@ __global__ __launch_bounds__(MAXT) void gemv_mfma_kernel(const MfmaArgs a) {
   const int nl = lane & 15;   // weight row inside the block / activation row for the A operand
   const int g = lane >> 4;    // k sub-block
   const int mrows = a.m;
-  const int ml = nl < mrows ? nl : mrows - 1;  // rows beyond M alias the last row; never stored
+  int ml[MT];  // this lane's activation row in each tile; rows beyond M alias the last row, never stored
+#pragma unroll
+  for (int t = 0; t < MT; ++t) ml[t] = min(16 * t + nl, mrows - 1);
 
   // A workgroup keeps ONE K slice (all of K when ks == 1) of the activations in
   // LDS and walks row-block groups with a grid stride; the ks workgroups of
@@ -257,12 +264,17 @@ __global__ __launch_bounds__(MAXT) void gemv_mfma_kernel(const MfmaArgs a) {
     }
   };
 
-  float4_t acc = {0.f, 0.f, 0.f, 0.f};
+  float4_t acc[MT];
   // one scale per row (no per-group f32 step between the MFMAs): two accumulators take
   // the MFMA steps in turn, so that consecutive MFMAs of a wave do not depend on each other
-  float4_t acc_odd = {0.f, 0.f, 0.f, 0.f};
+  float4_t acc_odd[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    acc[t] = (float4_t){0.f, 0.f, 0.f, 0.f};
+    acc_odd[t] = (float4_t){0.f, 0.f, 0.f, 0.f};
+  }
 
-  auto compute_batch = [&](const Batch& b, int step) {
+  auto compute_batch = [&](const Batch& b, int step) __attribute__((always_inline)) {
     const int bidx = kw_idx + step * a.kw;
     const bool valid = bidx < nbatches;  // wave-uniform
     const int tlb = min(bidx, nbatches - 1) * U * STEPS;
@@ -314,30 +326,30 @@ __global__ __launch_bounds__(MAXT) void gemv_mfma_kernel(const MfmaArgs a) {
         if (valid) {
 #pragma unroll
           for (int s = 0; s < STEPS; ++s) {
-            const u32x4 xa = lds[x_unit<FMT>(tl + s, g, ml, row_units)];
-            if (s & 1) acc_odd = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, xa), bw[s], acc_odd, 0, 0, 0);
-            else acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, xa), bw[s], acc, 0, 0, 0);
+#pragma unroll
+            for (int t = 0; t < MT; ++t) {
+              const u32x4 xa = lds[x_unit<FMT>(tl + s, g, ml[t], row_units)];
+              if (s & 1) acc_odd[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, xa), bw[s], acc_odd[t], 0, 0, 0);
+              else acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, xa), bw[s], acc[t], 0, 0, 0);
+            }
           }
         }
       } else if (FMT == TLHIP_FMT_INT8_GROUPED) {
         // both steps of an iteration lie in one scale group
-        const u32x4 xa0 = lds[x_unit<FMT>(tl, g, ml, row_units)];
-        const u32x4 xa1 = lds[x_unit<FMT>(tl + 1, g, ml, row_units)];
-        float4_t d = {0.f, 0.f, 0.f, 0.f};
-        d = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, xa0), bw[0], d, 0, 0, 0);
-        d = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, xa1), bw[1], d, 0, 0, 0);
         const uint16_t sbits = WIDE ? (uint16_t)((u & 1) ? (b.sv[u >> 1] >> 16) : (b.sv[u >> 1] & 0xffffu)) : b.s[u][0];
         const float sc = valid ? half_bits_to_float(sbits) : 0.f;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) acc[r] = fmaf(sc, d[r], acc[r]);
-      } else {
-        float4_t d[STEPS];
+        for (int t = 0; t < MT; ++t) {
+          const u32x4 xa0 = lds[x_unit<FMT>(tl, g, ml[t], row_units)];
+          const u32x4 xa1 = lds[x_unit<FMT>(tl + 1, g, ml[t], row_units)];
+          float4_t d = {0.f, 0.f, 0.f, 0.f};
+          d = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, xa0), bw[0], d, 0, 0, 0);
+          d = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, xa1), bw[1], d, 0, 0, 0);
 #pragma unroll
-        for (int s = 0; s < STEPS; ++s) {
-          const u32x4 xa = lds[x_unit<FMT>(tl + s, g, ml, row_units)];
-          const float4_t zero = {0.f, 0.f, 0.f, 0.f};
-          d[s] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, xa), bw[s], zero, 0, 0, 0);
+          for (int r = 0; r < 4; ++r) acc[t][r] = fmaf(sc, d[r], acc[t][r]);
         }
+      } else {
+        float sc[STEPS];
 #pragma unroll
         for (int s = 0; s < STEPS; ++s) {
           uint16_t bits;
@@ -347,20 +359,34 @@ __global__ __launch_bounds__(MAXT) void gemv_mfma_kernel(const MfmaArgs a) {
           } else {
             bits = b.s[u][s];
           }
-          const float sc = valid ? half_bits_to_float(bits) : 0.f;
+          sc[s] = valid ? half_bits_to_float(bits) : 0.f;
+        }
 #pragma unroll
-          for (int r = 0; r < 4; ++r) acc[r] = fmaf(sc, d[s][r], acc[r]);
+        for (int t = 0; t < MT; ++t) {
+          float4_t d[STEPS];
+#pragma unroll
+          for (int s = 0; s < STEPS; ++s) {
+            const u32x4 xa = lds[x_unit<FMT>(tl + s, g, ml[t], row_units)];
+            const float4_t zero = {0.f, 0.f, 0.f, 0.f};
+            d[s] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, xa), bw[s], zero, 0, 0, 0);
+          }
+#pragma unroll
+          for (int s = 0; s < STEPS; ++s) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) acc[t][r] = fmaf(sc[s], d[s][r], acc[t][r]);
+          }
         }
       }
     }
   };
 
-  // One finished 16 x 16 tile (all of this workgroup's K): combine with the other
-  // workgroups' K slices when ks > 1, apply the epilogue, store.
-  auto emit = [&](int rb, float4_t t) {
+  // The finished 16 x 16 tiles of one row block (all of this workgroup's K), one per tile
+  // of activation rows: combine with the other workgroups' K slices when ks > 1, apply the
+  // epilogue, store.
+  auto emit = [&](int rb, float4_t (&tile)[MT]) __attribute__((always_inline)) {
     bool owner = true;  // wave-uniform
     if (a.ks > 1) {
-      // Publish this slice's tile; the workgroup that arrives last for the row
+      // Publish this slice's tiles; the workgroup that arrives last for the row
       // block adds the ks tiles in slice order (so the sum does not depend on
       // who is last), resets the counter for the next launch and stores.
       // Tiles and counters move with device-scope atomic accesses only: those
@@ -368,10 +394,14 @@ __global__ __launch_bounds__(MAXT) void gemv_mfma_kernel(const MfmaArgs a) {
       // device-scope fence (a write-back and invalidate of a whole L2 per row
       // block) measured 3x slower for the whole kernel.  Order: tile stores,
       // wait until the memory system has acknowledged them, then the counter.
-      float* mine = a.workspace + ((size_t)rb * a.ks + slice) * 256;
+      // Every access to tiles and counters here and in sum_slices must stay a
+      // device-scope atomic: a plain load could be served from this XCD's L2.
+      float* mine = a.workspace + ((size_t)rb * a.ks + slice) * (MT * 256);
 #pragma unroll
-      for (int r = 0; r < 4; ++r)
-        __hip_atomic_store(mine + (4 * g + r) * 16 + nl, t[r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      for (int t = 0; t < MT; ++t)
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          __hip_atomic_store(mine + t * 256 + (4 * g + r) * 16 + nl, tile[t][r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
       __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): every store of this wave is acknowledged
       int old = 0;
@@ -380,8 +410,9 @@ __global__ __launch_bounds__(MAXT) void gemv_mfma_kernel(const MfmaArgs a) {
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
       owner = old == a.ks - 1;
       if (owner) {
-        const float* tiles = a.workspace + (size_t)rb * a.ks * 256;
-        t = sum_slices(tiles, a.ks, (4 * g) * 16 + nl);
+        const float* tiles = a.workspace + (size_t)rb * a.ks * (MT * 256);
+#pragma unroll
+        for (int t = 0; t < MT; ++t) tile[t] = sum_slices(tiles + t * 256, a.ks, (4 * g) * 16 + nl, MT * 256);
         if (lane == 0) __hip_atomic_store(a.counters + rb, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
     }
@@ -391,13 +422,29 @@ __global__ __launch_bounds__(MAXT) void gemv_mfma_kernel(const MfmaArgs a) {
       if (orow < P.n) {
         float rs = a.scale_mul * a.alpha;
         if (!GROUPED) rs *= ((const float*)P.scales)[orow];
+        if constexpr (MT == 1) {
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const int m = 4 * g + r;
-          if (m < mrows) {
-            const float v = apply_epilogue(P.epi, t[r] * rs, orow);
-            store_out(P.y, a.y_dtype, (int64_t)m * P.n + orow, v);
+          for (int r = 0; r < 4; ++r) {
+            const int m = 4 * g + r;
+            if (m < mrows) {
+              const float v = apply_epilogue(P.epi, tile[0][r] * rs, orow);
+              store_out(P.y, a.y_dtype, (int64_t)m * P.n + orow, v);
+            }
           }
+        } else {
+          float v[MT * 4];
+#pragma unroll
+          for (int t = 0; t < MT; ++t)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) v[4 * t + r] = tile[t][r] * rs;
+          apply_epilogue_all(P.epi, v, orow);
+#pragma unroll
+          for (int t = 0; t < MT; ++t)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              const int m = 16 * t + 4 * g + r;
+              if (m < mrows) store_out(P.y, a.y_dtype, (int64_t)m * P.n + orow, v[4 * t + r]);
+            }
         }
       }
     }
@@ -410,21 +457,27 @@ __global__ __launch_bounds__(MAXT) void gemv_mfma_kernel(const MfmaArgs a) {
   // wave's memory latency, and with K slices one drain of the load pipeline, per
   // block: 3 us of a 12 us kernel, 6 us with four K slices.)
   int round = 0;
-  auto finish = [&](int wb) {
+  auto finish = [&](int wb) __attribute__((always_inline)) {
     if (!GROUPED) {
-      acc += acc_odd;
-      acc_odd = (float4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int t = 0; t < MT; ++t) {
+        acc[t] += acc_odd[t];
+        acc_odd[t] = (float4_t){0.f, 0.f, 0.f, 0.f};
+      }
     }
     if (a.kw == 1) {
       const int rb = wb * a.blocks_per_wg + bw_idx;
       if (rb < a.nblocks) emit(rb, acc);
     } else {
-      float* tile = partial + (size_t)(round * (int)(blockDim.x >> 6) + wave) * 256;
+      float* tile = partial + (size_t)(round * (int)(blockDim.x >> 6) + wave) * (MT * 256);
 #pragma unroll
-      for (int r = 0; r < 4; ++r) tile[(4 * g + r) * 16 + nl] = acc[r];
+      for (int t = 0; t < MT; ++t)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) tile[t * 256 + (4 * g + r) * 16 + nl] = acc[t][r];
     }
     ++round;
-    acc = (float4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int t = 0; t < MT; ++t) acc[t] = (float4_t){0.f, 0.f, 0.f, 0.f};
   };
 
   // Activations first (they return first), then the first weight batch, then
@@ -514,7 +567,7 @@ __global__ __launch_bounds__(MAXT) void gemv_mfma_kernel(const MfmaArgs a) {
       b += wg_stride;
     }
   };
-  auto consume = [&](const Batch& b, int wb, int st) {
+  auto consume = [&](const Batch& b, int wb, int st) __attribute__((always_inline)) {
     compute_batch(b, st);
     if (st == a.nsteps - 1) finish(wb);
   };
@@ -552,11 +605,15 @@ __global__ __launch_bounds__(MAXT) void gemv_mfma_kernel(const MfmaArgs a) {
       const int r = t >> bshift, b = t & (a.blocks_per_wg - 1);
       const int rb = (wgb0 + r * wg_stride) * a.blocks_per_wg + b;
       if (rb >= a.nblocks) continue;  // wave-uniform
-      const float* tiles = partial + (size_t)(r * waves + b * a.kw) * 256;
-      float4_t sum = {0.f, 0.f, 0.f, 0.f};
+      const float* tiles = partial + (size_t)(r * waves + b * a.kw) * (MT * 256);
+      float4_t sum[MT];
+#pragma unroll
+      for (int t = 0; t < MT; ++t) sum[t] = (float4_t){0.f, 0.f, 0.f, 0.f};
       for (int w = 0; w < a.kw; ++w) {
 #pragma unroll
-        for (int q = 0; q < 4; ++q) sum[q] += tiles[w * 256 + (4 * g + q) * 16 + nl];
+        for (int t = 0; t < MT; ++t)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) sum[t][q] += tiles[(w * MT + t) * 256 + (4 * g + q) * 16 + nl];
       }
       emit(rb, sum);
     }
@@ -564,18 +621,23 @@ __global__ __launch_bounds__(MAXT) void gemv_mfma_kernel(const MfmaArgs a) {
 }
 
 
-template <int FMT, bool WIDE, bool GROUP>
+template <int FMT, bool WIDE, bool GROUP, int MT>
 int launch_mfma_u(int unroll, const MfmaArgs& a, int grid, int threads, size_t lds_bytes, hipStream_t stream) {
   // 16 waves leave 128 registers per lane: enough for one or two iterations in flight
+  // (and for one tile of activation rows: more tiles come with at most 8 waves)
   const void* fn;
   if (threads > 512) {
-    fn = unroll == 1 ? (const void*)gemv_mfma_kernel<FMT, 1, WIDE, 1024, false, GROUP>
-                     : (const void*)gemv_mfma_kernel<FMT, 2, WIDE, 1024, false, GROUP>;
+    if constexpr (MT > 1) {
+      return set_error(TLHIP_ERR_INVALID, "gemv_mfma: more than 16 activation rows take at most 8 waves per workgroup");
+    } else {
+      fn = unroll == 1 ? (const void*)gemv_mfma_kernel<FMT, 1, WIDE, 1024, false, GROUP>
+                       : (const void*)gemv_mfma_kernel<FMT, 2, WIDE, 1024, false, GROUP>;
+    }
   } else {
     switch (unroll) {
-      case 1: fn = (const void*)gemv_mfma_kernel<FMT, 1, WIDE, 512, false, GROUP>; break;
-      case 2: fn = (const void*)gemv_mfma_kernel<FMT, 2, WIDE, 512, false, GROUP>; break;
-      default: fn = (const void*)gemv_mfma_kernel<FMT, 4, WIDE, 512, false, GROUP>; break;
+      case 1: fn = (const void*)gemv_mfma_kernel<FMT, 1, WIDE, 512, false, GROUP, MT>; break;
+      case 2: fn = (const void*)gemv_mfma_kernel<FMT, 2, WIDE, 512, false, GROUP, MT>; break;
+      default: fn = (const void*)gemv_mfma_kernel<FMT, 4, WIDE, 512, false, GROUP, MT>; break;
     }
   }
   void* args[] = {(void*)&a};
@@ -583,57 +645,65 @@ int launch_mfma_u(int unroll, const MfmaArgs& a, int grid, int threads, size_t l
 }
 
 // The form with whole-line weight loads (2 or 4 iterations in flight).
-template <int FMT, bool WIDE, bool GROUP>
+template <int FMT, bool WIDE, bool GROUP, int MT>
 int launch_mfma_line(int unroll, const MfmaArgs& a, int grid, int threads, size_t lds_bytes, hipStream_t stream) {
   const void* fn;
-  if (threads > 512) fn = (const void*)gemv_mfma_kernel<FMT, 2, WIDE, 1024, true, GROUP>;
-  else if (unroll == 2) fn = (const void*)gemv_mfma_kernel<FMT, 2, WIDE, 512, true, GROUP>;
-  else fn = (const void*)gemv_mfma_kernel<FMT, 4, WIDE, 512, true, GROUP>;
+  if (threads > 512) {
+    if constexpr (MT > 1) {
+      return set_error(TLHIP_ERR_INVALID, "gemv_mfma: more than 16 activation rows take at most 8 waves per workgroup");
+    } else {
+      fn = (const void*)gemv_mfma_kernel<FMT, 2, WIDE, 1024, true, GROUP>;
+    }
+  } else if (unroll == 2) {
+    fn = (const void*)gemv_mfma_kernel<FMT, 2, WIDE, 512, true, GROUP, MT>;
+  } else {
+    fn = (const void*)gemv_mfma_kernel<FMT, 4, WIDE, 512, true, GROUP, MT>;
+  }
   void* args[] = {(void*)&a};
   return launch_kernel(fn, dim3(grid), dim3(threads), args, lds_bytes, stream);
 }
 
 // Kernel instance for (format, group size, K, configuration): the scale loads are wide
 // wherever a batch's scales are contiguous and aligned.
-template <bool GROUP>
+template <bool GROUP, int MT = 1>
 int launch_mfma_instance(int format, int group_size, int64_t k, int unroll, int line, const MfmaArgs& a, int grid,
                          int threads, size_t lds_bytes, hipStream_t stream) {
   switch (format) {
     case TLHIP_FMT_INT4_GROUPED:
       // one scale per 16-byte chunk and 16-byte aligned scale vectors: wide scale loads
       if (line == 1)  // group size 32 and K % 256 == 0: the wide scale loads as well
-        return launch_mfma_line<TLHIP_FMT_INT4_GROUPED, true, GROUP>(unroll, a, grid, threads, lds_bytes, stream);
+        return launch_mfma_line<TLHIP_FMT_INT4_GROUPED, true, GROUP, MT>(unroll, a, grid, threads, lds_bytes, stream);
       if (group_size == 32 && (unroll == 1 || k % 256 == 0))
-        return launch_mfma_u<TLHIP_FMT_INT4_GROUPED, true, GROUP>(unroll, a, grid, threads, lds_bytes, stream);
-      return launch_mfma_u<TLHIP_FMT_INT4_GROUPED, false, GROUP>(unroll, a, grid, threads, lds_bytes, stream);
+        return launch_mfma_u<TLHIP_FMT_INT4_GROUPED, true, GROUP, MT>(unroll, a, grid, threads, lds_bytes, stream);
+      return launch_mfma_u<TLHIP_FMT_INT4_GROUPED, false, GROUP, MT>(unroll, a, grid, threads, lds_bytes, stream);
     case TLHIP_FMT_INT8_GROUPED:
       if (line == 1 && group_size == 64)  // one scale per iteration: the wide scale loads as well
-        return launch_mfma_line<TLHIP_FMT_INT8_GROUPED, true, GROUP>(unroll, a, grid, threads, lds_bytes, stream);
-      if (line == 1) return launch_mfma_line<TLHIP_FMT_INT8_GROUPED, false, GROUP>(unroll, a, grid, threads, lds_bytes, stream);
-      return launch_mfma_u<TLHIP_FMT_INT8_GROUPED, false, GROUP>(unroll, a, grid, threads, lds_bytes, stream);
+        return launch_mfma_line<TLHIP_FMT_INT8_GROUPED, true, GROUP, MT>(unroll, a, grid, threads, lds_bytes, stream);
+      if (line == 1) return launch_mfma_line<TLHIP_FMT_INT8_GROUPED, false, GROUP, MT>(unroll, a, grid, threads, lds_bytes, stream);
+      return launch_mfma_u<TLHIP_FMT_INT8_GROUPED, false, GROUP, MT>(unroll, a, grid, threads, lds_bytes, stream);
     default:
-      if (line == 1) return launch_mfma_line<TLHIP_FMT_INT8_ROW, false, GROUP>(unroll, a, grid, threads, lds_bytes, stream);
-      return launch_mfma_u<TLHIP_FMT_INT8_ROW, false, GROUP>(unroll, a, grid, threads, lds_bytes, stream);
+      if (line == 1) return launch_mfma_line<TLHIP_FMT_INT8_ROW, false, GROUP, MT>(unroll, a, grid, threads, lds_bytes, stream);
+      return launch_mfma_u<TLHIP_FMT_INT8_ROW, false, GROUP, MT>(unroll, a, grid, threads, lds_bytes, stream);
   }
 }
 
 // Every instance launch_mfma_instance can reach, in prepare mode (see launch_kernel).
-template <bool GROUP>
+template <bool GROUP, int MT = 1>
 int prepare_mfma_instances() {
   MfmaArgs a;
   memset(&a, 0, sizeof a);
   for (int threads : {512, 1024})
     for (int unroll : {1, 2, 4}) {
-      if (threads == 1024 && unroll == 4) continue;
-      int rc = launch_mfma_instance<GROUP>(TLHIP_FMT_INT4_GROUPED, 32, 256, unroll, 0, a, 1, threads, 0, nullptr);
-      if (!rc) rc = launch_mfma_instance<GROUP>(TLHIP_FMT_INT4_GROUPED, 64, 256, unroll, 0, a, 1, threads, 0, nullptr);
-      if (!rc) rc = launch_mfma_instance<GROUP>(TLHIP_FMT_INT8_GROUPED, 128, 256, unroll, 0, a, 1, threads, 0, nullptr);
-      if (!rc) rc = launch_mfma_instance<GROUP>(TLHIP_FMT_INT8_ROW, 0, 256, unroll, 0, a, 1, threads, 0, nullptr);
+      if (threads == 1024 && (unroll == 4 || MT > 1)) continue;
+      int rc = launch_mfma_instance<GROUP, MT>(TLHIP_FMT_INT4_GROUPED, 32, 256, unroll, 0, a, 1, threads, 0, nullptr);
+      if (!rc) rc = launch_mfma_instance<GROUP, MT>(TLHIP_FMT_INT4_GROUPED, 64, 256, unroll, 0, a, 1, threads, 0, nullptr);
+      if (!rc) rc = launch_mfma_instance<GROUP, MT>(TLHIP_FMT_INT8_GROUPED, 128, 256, unroll, 0, a, 1, threads, 0, nullptr);
+      if (!rc) rc = launch_mfma_instance<GROUP, MT>(TLHIP_FMT_INT8_ROW, 0, 256, unroll, 0, a, 1, threads, 0, nullptr);
       if (unroll != 1) {
-        if (!rc) rc = launch_mfma_instance<GROUP>(TLHIP_FMT_INT4_GROUPED, 32, 256, unroll, 1, a, 1, threads, 0, nullptr);
-        if (!rc) rc = launch_mfma_instance<GROUP>(TLHIP_FMT_INT8_GROUPED, 64, 256, unroll, 1, a, 1, threads, 0, nullptr);
-        if (!rc) rc = launch_mfma_instance<GROUP>(TLHIP_FMT_INT8_GROUPED, 128, 256, unroll, 1, a, 1, threads, 0, nullptr);
-        if (!rc) rc = launch_mfma_instance<GROUP>(TLHIP_FMT_INT8_ROW, 0, 256, unroll, 1, a, 1, threads, 0, nullptr);
+        if (!rc) rc = launch_mfma_instance<GROUP, MT>(TLHIP_FMT_INT4_GROUPED, 32, 256, unroll, 1, a, 1, threads, 0, nullptr);
+        if (!rc) rc = launch_mfma_instance<GROUP, MT>(TLHIP_FMT_INT8_GROUPED, 64, 256, unroll, 1, a, 1, threads, 0, nullptr);
+        if (!rc) rc = launch_mfma_instance<GROUP, MT>(TLHIP_FMT_INT8_GROUPED, 128, 256, unroll, 1, a, 1, threads, 0, nullptr);
+        if (!rc) rc = launch_mfma_instance<GROUP, MT>(TLHIP_FMT_INT8_ROW, 0, 256, unroll, 1, a, 1, threads, 0, nullptr);
       }
       if (rc) return rc;
     }
@@ -650,5 +720,10 @@ int launch_mfma_grouped(int format, int group_size, int64_t k, int unroll, int l
                         size_t lds_bytes, hipStream_t stream);
 int prepare_mfma_single();
 int prepare_mfma_grouped();
+// The instances for 17..64 activation rows (`tiles` = 2 or 4 tiles of 16 rows), single
+// problem, at most 8 waves per workgroup: gemv_mfma_rows.hip.
+int launch_mfma_rows(int tiles, int format, int group_size, int64_t k, int unroll, int line, const MfmaArgs& a, int grid,
+                     int threads, size_t lds_bytes, hipStream_t stream);
+int prepare_mfma_rows();
 
 }  // namespace tlhip
