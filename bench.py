@@ -660,6 +660,38 @@ def main() -> int:
                 w._base.destroy()
                 w.scales.destroy()
 
+        # batched decode beyond 16 rows (batch 32 / 64 / 128 of a serving loop) at the same three
+        # shapes: what the library selects (up to 64 rows per launch of the skinny matrix-core
+        # kernel while that beats the tiles) beside ONE tiled launch (128 x 128 tiles)
+        rows_section = []
+        fnc = L.load().tlhip_matmul_quantized_config
+        tile128 = L.KernelConfig.of(3, 128, 128, 128, 2, 2)
+        for (n, k) in shapes:
+            qws = [be._qweight(w, False) for w in pools[(n, k)]]
+            for m in (32, 64, 128):
+                x, _ = B.activations(m, k, std=0.5)
+                out = be._alloc([m, n], "f16")
+                if not args.no_autotune and m <= 64:
+                    B.tune(pools[(n, k)], x, m, out)
+                us = B.median_time(B.make_call(pools[(n, k)], x, m, out), 30)
+                st = {"i": 0}
+
+                def tiled_call():
+                    qw = qws[st["i"] % len(qws)]
+                    st["i"] += 1
+                    rc = fnc(C.byref(qw), x.ptr, L.F16, m, out.ptr, L.F16, 1.0, None, C.byref(tile128), None)
+                    if rc:
+                        L.check(rc)
+                us_tiled = B.median_time(tiled_call, 20)
+                by = algorithmic_bytes("int4", n, k, 32, m, 2, 2)
+                rows_section.append({"m": m, "n": n, "k": k, "us": round(us, 2), "gbps": round(by / us / 1e3, 1),
+                                     "frac_of_peak": round(by / us / 1e3 / HBM_PEAK_GBPS, 4),
+                                     "us_one_tiled_launch_128x128": round(us_tiled, 2),
+                                     "config": list(be.selectedConfig(pools[(n, k)][0], "f16", m, "f16").as_tuple())})
+                out.destroy()
+                x.destroy()
+        details["qwen3_8b_batched_decode_32_to_128_rows"] = rows_section
+
         # config 5: LM head 256000 x 2304 int8-row (f32 logits) and the MLP GEMVs
         lm_pool, _ = B.weight_pool("int8-row", 256000, 2304, 0, "f32", pool_bytes=1.25e9)
         lm = []

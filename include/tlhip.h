@@ -263,7 +263,11 @@ int tlhip_gemm_prefill(const tlhip_qweight_t* w, const void* x, int x_dtype, int
 
 /* The matmul seam for a packed B operand: matmulQuantizedB
  * (matmul-ops.ts:113-182).  Routes small m to the GEMV kernels and larger m to
- * the prefill GEMM.  f32 activations: up to 63 rows run as GEMV passes of <= 16
+ * the prefill GEMM.  A few more rows than 16 on a matrix that gives far fewer
+ * tiles than the chip has CUs (batched decode at batch 32..128) go through the
+ * skinny matrix-core GEMV, up to 64 rows per launch, while the library's cost
+ * model puts that below one tiled launch; a tuned entry of the problem itself
+ * overrides the model.  f32 activations: up to 63 rows run as GEMV passes of <= 16
  * rows in f32 arithmetic; from 64 rows on they are rounded to f16 (the operand
  * type of the matrix cores; |x| above 65504 becomes inf) by a cast launch into
  * the stream's workspace and take the prefill GEMM of the f16 problem, which is
@@ -387,7 +391,9 @@ int tlhip_candidate_get(const tlhip_qweight_t* w, int x_dtype, int64_t m, int y_
 /* The configuration tlhip_matmul_quantized would use now: the tuned winner of this
  * exact problem if cached, else the winner of the nearest tuned problem of the same
  * shape class (autotune.ts:269-300), else the heuristic default — selectMatmulChoice,
- * dispatch.ts:171-192.  Every level is re-gated on applicability. */
+ * dispatch.ts:171-192.  Every level is re-gated on applicability.  Where the rows
+ * go in several launches (see tlhip_matmul_quantized) it is the configuration of
+ * the first launch. */
 int tlhip_selected_config(const tlhip_qweight_t* w, int x_dtype, int64_t m, int y_dtype,
                           tlhip_kernel_config_t* host_out);
 

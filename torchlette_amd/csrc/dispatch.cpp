@@ -521,35 +521,40 @@ bool has_tuned_entry(const Problem& p) {
   return g_tuned.count(problem_key(p)) != 0;
 }
 
-// What the library launches for a problem when the caller names no configuration.
+// What the library launches for a problem when the caller names no configuration: the
+// selected configuration on all rows, or the rows in chunks.
+struct Route {
+  int64_t chunk;                // rows per launch; 0: one launch (or matmul_with's own passes) of `first` on all rows
+  tlhip_kernel_config_t first;  // configuration of the whole chunks (of everything when chunk == 0)
+  tlhip_kernel_config_t last;   // configuration of the remaining rows, if any
+};
+
 // 9..16 rows whose activations fit no geometry of the matrix-core kernels (K = 11008 at
 // M = 15 or 16: two K slices of 16 rows take 176 KB of LDS, and four do not divide its
 // 86 steps) would fall to the VALU kernel, which streams the weights once per four rows;
 // two launches of at most 8 rows on the matrix cores stream them twice.
-int run_selected(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t stream) {
-  if (c.variant == VARIANT_GEMV && p.m > 8 && p.m <= 16 && p.pro.kind == TLHIP_PRO_NONE) {
+//
+// A few more rows than the decode kernels take, far fewer than fill the chip with
+// tiles: a tiled launch of at most one round of 128 x 128 tiles takes the time ONE
+// workgroup needs to walk K (measured 40-45 us per 4096 of K whatever M and N are, up
+// to 512 resident tiles), the decode kernel streams the weights once per 16 rows (3 us
+// + 1 us per 3.2 MB of packed weights: 6.3 / 9.9 / 11.9 us at the Qwen3-8B shapes).
+// Below the break-even the rows go through the decode kernel: up to 64 per launch, or
+// 16 at a time where the activations of more rows fit no geometry.
+// (A tuned entry of the problem itself is a measurement and stands.)
+Route plan_route(const Problem& p, const tlhip_kernel_config_t& c) {
+  Route r{0, c, c};
+  if (p.pro.kind != TLHIP_PRO_NONE) return r;
+  if (c.variant == VARIANT_GEMV && p.m > 8 && p.m <= 16) {
     Problem lo = p, hi = p;
     lo.m = 8;
     hi.m = p.m - 8;
-    const int xb = p.x_dtype == TLHIP_F16 ? 2 : 4, yb = p.y_dtype == TLHIP_F16 ? 2 : 4;
-    hi.x = (const char*)p.x + 8 * p.k * xb;
-    hi.y = (char*)p.y + 8 * p.n * yb;
     const tlhip_kernel_config_t cl = select_config(lo);
-    if (cl.variant == VARIANT_GEMV_MFMA || cl.variant == VARIANT_GEMV_XREG) {
-      const int rc = run_config(lo, cl, stream);
-      return rc ? rc : matmul_with(hi, select_gemv_config(hi), stream);
-    }
+    if (cl.variant == VARIANT_GEMV_MFMA || cl.variant == VARIANT_GEMV_XREG) return Route{8, cl, select_gemv_config(hi)};
+    return r;
   }
-  // A few more rows than the decode kernels take, far fewer than fill the chip with
-  // tiles: a tiled launch of at most one round of 128 x 128 tiles takes the time ONE
-  // workgroup needs to walk K (measured 40-45 us per 4096 of K whatever M and N are, up
-  // to 512 resident tiles), the decode kernel streams the weights once per 16 rows (3 us
-  // + 1 us per 3.2 MB of packed weights: 6.3 / 9.9 / 11.9 us at the Qwen3-8B shapes).
-  // Below the break-even the rows go through the decode kernel: up to 64 per launch, or
-  // 16 at a time where the activations of more rows fit no geometry.
-  // (A tuned entry of the problem itself is a measurement and stands.)
   if ((c.variant == VARIANT_TILED || c.variant == VARIANT_TILED_DIRECT) && p.m > 16 && p.x_dtype == TLHIP_F16 &&
-      p.pro.kind == TLHIP_PRO_NONE && !has_tuned_entry(p)) {
+      !has_tuned_entry(p)) {
     const double packed_mb = (double)p.n * (double)p.k * (p.format == TLHIP_FMT_INT4_GROUPED ? 0.5 : 1.0) / 1e6;
     const double pass_us = 3.0 + packed_mb / 3.2;
     const int64_t passes = (p.m + 15) / 16;
@@ -564,38 +569,43 @@ int run_selected(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t s
     const int64_t full = p.m / 64, rest = p.m % 64;
     const double rows_us = (double)full * chunk_us(64) + (rest ? chunk_us(rest) : 0.0);
     if (rows_us < 0.9 * tiled_us) {
-      const int xb = 2, yb = p.y_dtype == TLHIP_F16 ? 2 : 4;
       bool ok = true;
-      tlhip_kernel_config_t cfg64, cfg_rest;
+      Route q{64, c, c};
       Problem q64 = p, qr = p;
       q64.m = 64;
       qr.m = rest;
-      if (full) ok = rows_in_one_launch_config(q64, &cfg64);
-      if (ok && rest > 16) ok = rows_in_one_launch_config(qr, &cfg_rest);
+      if (full) ok = rows_in_one_launch_config(q64, &q.first);
+      if (ok && rest > 16) ok = rows_in_one_launch_config(qr, &q.last);
       if (ok && rest > 0 && rest <= 16) {
-        cfg_rest = select_gemv_config(qr);
-        ok = cfg_rest.variant == VARIANT_GEMV_MFMA || cfg_rest.variant == VARIANT_GEMV_XREG || rest <= 4;
+        q.last = select_gemv_config(qr);
+        ok = q.last.variant == VARIANT_GEMV_MFMA || q.last.variant == VARIANT_GEMV_XREG || rest <= 4;
       }
-      if (ok) {
-        for (int64_t m0 = 0; m0 < p.m; m0 += 64) {
-          Problem q = p;
-          q.m = std::min<int64_t>(64, p.m - m0);
-          q.x = (const char*)p.x + m0 * p.k * xb;
-          q.y = (char*)p.y + m0 * p.n * yb;
-          const int rc = run_config(q, q.m == 64 ? cfg64 : cfg_rest, stream);
-          if (rc) return rc;
-        }
-        return TLHIP_OK;
-      }
+      if (!full) q.first = q.last;
+      if (ok) return q;
     }
     if ((double)passes * pass_us < 0.8 * tiled_us) {
       Problem q = p;
       q.m = 16;
       const tlhip_kernel_config_t c16 = select_gemv_config(q);
-      if (c16.variant == VARIANT_GEMV_MFMA || c16.variant == VARIANT_GEMV_XREG) return matmul_with(p, c16, stream);
+      if (c16.variant == VARIANT_GEMV_MFMA || c16.variant == VARIANT_GEMV_XREG) return Route{0, c16, c16};  // matmul_with's passes
     }
   }
-  return matmul_with(p, c, stream);
+  return r;
+}
+
+int run_selected(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t stream) {
+  const Route r = plan_route(p, c);
+  if (r.chunk == 0) return matmul_with(p, r.first, stream);
+  const int xb = p.x_dtype == TLHIP_F16 ? 2 : 4, yb = p.y_dtype == TLHIP_F16 ? 2 : 4;
+  for (int64_t m0 = 0; m0 < p.m; m0 += r.chunk) {
+    Problem q = p;
+    q.m = std::min<int64_t>(r.chunk, p.m - m0);
+    q.x = (const char*)p.x + m0 * p.k * xb;
+    q.y = (char*)p.y + m0 * p.n * yb;
+    const int rc = matmul_with(q, q.m == r.chunk ? r.first : r.last, stream);
+    if (rc) return rc;
+  }
+  return TLHIP_OK;
 }
 
 // One-field variations of `base` inside its kernel family, plus the heuristic defaults of
@@ -1214,7 +1224,7 @@ int tlhip_selected_config(const tlhip_qweight_t* w, int x_dtype, int64_t m, int 
   int rc = shape_problem(w, x_dtype, m, y_dtype, &p);
   if (rc) return rc;
   if (!out) return set_error(TLHIP_ERR_INVALID, "selected_config: null output");
-  *out = select_config(p);
+  *out = plan_route(p, select_config(p)).first;  // of the first launch, where the rows go in chunks
   if (p.x_dtype == TLHIP_F32 && p.m >= kF32TiledFromRows) {
     // what tlhip_matmul_quantized launches for these rows: the f16 problem's tiled kernel
     const tlhip_kernel_config_t c = select_config(as_f16_activations(p));
