@@ -350,11 +350,15 @@ int tlhip_topk(const float* logits, int64_t offset, int64_t length, int k, float
  * dispatch.ts:60-207, 405-578) ---- */
 
 /* A launch configuration.  variant 0 = "gemv" (VALU dot), 1 = "gemv_mfma"
- * (skinny MFMA), 2 = "tiled" (prefill MFMA GEMM, both operands through LDS),
+ * (skinny MFMA: up to 16 rows, and 17..64 rows for one problem with at most 8
+ * waves per workgroup and, above 32 rows, at most 2 iterations in flight),
+ * 2 = "tiled" (prefill MFMA GEMM, both operands through LDS),
  * 3 = "tiled_direct" (prefill MFMA GEMM for int4, weights dequantised in
  * registers; fields as "tiled" with tile K 128; tiles (M, N, waves M, waves N):
  * 256x256 2x4, 256x128 2x4, 128x256 2x4, 256x128 4x2, 128x128 2x2, 256x256 2x2,
- * 128x256 1x4, 128x192 2x2),
+ * 128x256 1x4, 128x192 2x2; p5 = 2, 4, 8 or 16: that many workgroups share a
+ * tile, each walking a slice of K, and the last to arrive adds their partial
+ * tiles in slice order - for launches of far fewer tiles than the chip has CUs),
  * 4 = "gemv_mfma_xreg" (skinny MFMA for int4 g32 with the activations held in
  * registers: p0 waves per workgroup, p1 iterations in flight, p2 workgroups per
  * CU, p3 K slices across workgroups, p4 = 1: every weight load of a wave issued
@@ -370,7 +374,8 @@ typedef struct {
   int32_t p4; /* gemv: chunks in flight (2/4/8)    tiled: waves N */
   int32_t p5; /* gemv: 1 = dot products on the 4x4x4 matrix-core instruction (int4, f16 x, m <= 4, p0 = 16, p1 = 1)
                * gemv_mfma: 1 = whole-line weight loads through a wave-private LDS patch (int8 with
-               * K % 128 == 0 or int4-g32 with K % 256 == 0; p1 = 2 or 4) */
+               * K % 128 == 0 or int4-g32 with K % 256 == 0; p1 = 2 or 4)
+               * tiled_direct: K slices across workgroups (0/1 = none) */
   int32_t p6;
 } tlhip_kernel_config_t;
 

@@ -184,6 +184,45 @@ def test_gemm_rejects_f32_activations_and_falls_back_to_gemv_passes(be):
     assert rel_l2(y, O.linear(x, deq)) <= 2e-6
 
 
+@pytest.mark.parametrize("m,n,k,cfg", [
+    (100, 384, 1024, (3, 128, 128, 128, 2, 2, 2)),
+    (256, 512, 2048, (3, 128, 128, 128, 2, 2, 8)),
+    (130, 300, 1024, (3, 256, 128, 128, 2, 4, 2)),     # ragged rows and columns
+    (64, 256, 4096, (3, 128, 256, 128, 1, 4, 16)),
+    (300, 520, 1536, (3, 128, 192, 128, 2, 2, 4)),     # three-tile-wide waves
+])
+@pytest.mark.parametrize("ydt", ["f16", "f32"])
+def test_direct_gemm_with_k_slices_across_workgroups(be, m, n, k, cfg, ydt):
+    """p5 workgroups share a tile, each walking a slice of K; the last to arrive adds the
+    partial tiles in slice order and runs the epilogue.  Against the oracle, bit-stable
+    from launch to launch (the order of the sum does not depend on who arrives last), and
+    as close to the oracle as the unsplit kernel."""
+    rng = np.random.default_rng(m + n + k)
+    packed, scales, deq = make_weight("int4-grouped", n, k, 32, rng)
+    x = make_x(m, k, "f16", rng, std=0.5)
+    bias = f16_round(rng.standard_normal(n) * 0.1)
+    want = O.linear(x.astype(np.float32), deq, bias.astype(np.float32), "gelu", threads=8)
+    got = run(be, "int4-grouped", packed, scales, n, k, 32, x, ydt, bias=bias, act="gelu", config=L.KernelConfig.of(*cfg))
+    assert got.shape == (m, n)
+    err = rel_l2(got, want)
+    assert err <= REL_L2_TOL, err
+    for _ in range(3):
+        again = run(be, "int4-grouped", packed, scales, n, k, 32, x, ydt, bias=bias, act="gelu", config=L.KernelConfig.of(*cfg))
+        assert np.array_equal(again, got)
+    unsplit = run(be, "int4-grouped", packed, scales, n, k, 32, x, ydt, bias=bias, act="gelu", config=L.KernelConfig.of(*cfg[:6]))
+    assert abs(rel_l2(unsplit, want) - err) <= 2e-5
+
+
+def test_direct_gemm_k_slices_reject_what_they_do_not_cover(be):
+    rng = np.random.default_rng(3)
+    packed, scales, _ = make_weight("int4-grouped", 256, 1024, 32, rng)
+    w = be.createQuantizedWeight(packed, scales, 256, 1024, T.resolveWeightFormat("int4-32", "f32"))
+    xt = be.ops.tensorFromArray(make_x(64, 1024, "f16", rng), [64, 1024], "f16")
+    for ks in (3, 16, 32):   # not a power of two / does not divide K / 128 = 8 / too many
+        with pytest.raises(L.TlhipError, match="K split across workgroups"):
+            be.linear(xt, w, config=L.KernelConfig.of(3, 128, 128, 128, 2, 2, ks))
+
+
 @pytest.mark.parametrize("m,passes", [(17, 1), (40, 1), (64, 1), (72, 2)])
 @pytest.mark.parametrize("ydt", ["f16", "f32"])
 def test_a_few_more_rows_than_16_go_through_the_decode_kernel(be, m, passes, ydt):

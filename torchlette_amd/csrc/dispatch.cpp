@@ -189,6 +189,27 @@ bool config_applicable(const Problem& p, const tlhip_kernel_config_t& c, const c
 
 tlhip_kernel_config_t default_valu_config(const Problem& p);
 
+// Time of one round of 128 x 128 tiles of the direct GEMM with `ks` K slices across
+// workgroups, in microseconds: a workgroup walks 4096 of K in 42 us, and the slices cost 12
+// us plus 1.6 us each to combine (fitted at 4096..12288 x 4096..12288, M = 64..512).
+double direct_round_us(int64_t k, int ks) {
+  const double walk = 42.0 * (double)k / 4096.0 / ks;
+  return ks > 1 ? walk + 12.0 + 1.6 * ks : walk;
+}
+
+// K slices across workgroups for a launch of 128 x 128 tiles of the direct GEMM: of 1, 2,
+// 4, 8 the cheapest by direct_round_us that keeps tiles x slices within the CUs, divides
+// the 128-k steps and leaves every slice at least four of them.
+int direct_k_split(const Problem& p) {
+  const int cus = device_cu_count() > 0 ? device_cu_count() : 256;
+  const int64_t tiles = ((p.m + 127) / 128) * ((p.n + 127) / 128);
+  const int64_t steps = p.k / 128;
+  int best = 1;
+  for (int ks = 2; ks <= 8; ks *= 2)
+    if (tiles * ks <= cus && steps % ks == 0 && steps / ks >= 4 && direct_round_us(p.k, ks) < direct_round_us(p.k, best)) best = ks;
+  return best;
+}
+
 // Heuristic default, used when nothing is tuned.
 tlhip_kernel_config_t default_config(const Problem& p) {
   if (p.m > 16 && p.x_dtype == TLHIP_F16) {
@@ -204,6 +225,16 @@ tlhip_kernel_config_t default_config(const Problem& p) {
       const int64_t t128x256 = ((p.m + 127) / 128) * ((p.n + 255) / 256);
       tlhip_kernel_config_t c = t256 >= 2 * cus ? direct_cfg(256, 256, 2, 4)
                                 : (t128x256 >= 160 ? direct_cfg(128, 256, 1, 4) : direct_cfg(128, 128, 2, 2));
+      if (c.p0 == 128 && c.p1 == 128) {
+        // fewer 128 x 128 tiles than CUs: 2, 4 or 8 workgroups share a tile, each walking a
+        // slice of K of at least four steps (4096 x 12288 at M = 256: 53 us against 141 us)
+        const int ks = direct_k_split(p);
+        if (ks > 1) {
+          tlhip_kernel_config_t split = c;
+          split.p5 = ks;
+          if (gemm_direct_config_applicable(p, split, nullptr)) return split;
+        }
+      }
       if (gemm_direct_config_applicable(p, c, nullptr)) return c;
     }
     // largest tile that still gives every CU a workgroup
@@ -346,6 +377,13 @@ std::vector<tlhip_kernel_config_t> candidates(const Problem& p) {
       tlhip_kernel_config_t c = direct_cfg(t[0], t[1], t[2], t[3]);
       if (gemm_direct_config_applicable(p, c, nullptr)) out.push_back(c);
     }
+    // K slices across workgroups where the 128 x 128 tiles are fewer than the CUs
+    if (((p.m + 127) / 128) * ((p.n + 127) / 128) < (device_cu_count() > 0 ? device_cu_count() : 256))
+      for (int ks : {2, 4, 8}) {
+        tlhip_kernel_config_t c = direct_cfg(128, 128, 2, 2);
+        c.p5 = ks;
+        if (gemm_direct_config_applicable(p, c, nullptr)) out.push_back(c);
+      }
   }
   return out;
 }
@@ -449,8 +487,9 @@ Problem as_f16_activations(const Problem& p) {
 bool f32_rows_through_tiled(const Problem& p, hipStream_t stream, int* rc) {
   if (p.x_dtype != TLHIP_F32 || p.m < kF32TiledFromRows || p.pro.kind != TLHIP_PRO_NONE) return false;
   Problem q = as_f16_activations(p);
-  const tlhip_kernel_config_t c = select_config(q);
+  tlhip_kernel_config_t c = select_config(q);
   if (c.variant != VARIANT_TILED && c.variant != VARIANT_TILED_DIRECT) return false;
+  if (c.variant == VARIANT_TILED_DIRECT) c.p5 = 0;  // no K split across workgroups: its partial tiles live in the workspace too
   const int64_t capacity = (int64_t)(kSplitWorkspaceFloats * sizeof(float) / sizeof(_Float16));
   int64_t rows = capacity / std::max<int64_t>(p.k, 1);
   if (rows >= 256) rows -= rows % 256;  // whole tiles per chunk
@@ -560,7 +599,7 @@ Route plan_route(const Problem& p, const tlhip_kernel_config_t& c) {
     const int64_t passes = (p.m + 15) / 16;
     const int64_t tiles = ((p.m + 127) / 128) * ((p.n + 127) / 128);
     const double rounds = tiles <= 512 ? 1.0 : (double)tiles / 512.0;
-    const double tiled_us = 42.0 * (double)p.k / 4096.0 * rounds;
+    const double tiled_us = direct_round_us(p.k, c.variant == VARIANT_TILED_DIRECT && c.p5 > 1 ? c.p5 : 1) * rounds;
     // Up to 64 rows per launch of the decode kernel: 1.2-1.6 times a 16-row pass for two
     // tiles of rows, 2.3-3.2 times for four (the activations a workgroup stages grow with
     // the rows, and their K slices are combined across workgroups).  More rows go 64 at a
@@ -1227,7 +1266,8 @@ int tlhip_selected_config(const tlhip_qweight_t* w, int x_dtype, int64_t m, int 
   *out = plan_route(p, select_config(p)).first;  // of the first launch, where the rows go in chunks
   if (p.x_dtype == TLHIP_F32 && p.m >= kF32TiledFromRows) {
     // what tlhip_matmul_quantized launches for these rows: the f16 problem's tiled kernel
-    const tlhip_kernel_config_t c = select_config(as_f16_activations(p));
+    tlhip_kernel_config_t c = select_config(as_f16_activations(p));
+    if (c.variant == VARIANT_TILED_DIRECT) c.p5 = 0;  // as f32_rows_through_tiled launches it
     if (c.variant == VARIANT_TILED || c.variant == VARIANT_TILED_DIRECT) *out = c;
   }
   return TLHIP_OK;

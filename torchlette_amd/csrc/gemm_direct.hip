@@ -57,6 +57,9 @@ struct DirectArgs {
   int cpg_shift;          // log2(16-byte chunks per scale group)
   int groups_per_row;
   int ksteps;             // K / 128
+  int ksplit;             // workgroups that share a tile, each walking ksteps / ksplit steps of K (1 = none)
+  float* workspace;       // ksplit > 1: partial tiles, [tile][slice][wave][MFMA tile][register][lane]
+  int* counters;          // ksplit > 1: arrival counters, one per tile; zero between launches
   TileMap map;
   OutArgs out;
 };
@@ -88,15 +91,22 @@ __global__ __launch_bounds__(WM * WN * 64, (TM * TN >= 16 ? 1 : 2)) void gemm_di
   const int wm = wave / WN, wn = wave % WN;
   const int lrow = lane & 31, lk = lane >> 5;
 
+  // K split across workgroups: the ksplit workgroups of consecutive ids take the slices of
+  // one tile.  A launch of a few tiles (M of a few hundred rows on a decode-sized matrix)
+  // would leave most CUs idle while each workgroup walks all of K on its own.
+  const int slice = a.ksplit > 1 ? (int)(blockIdx.x % (unsigned)a.ksplit) : 0;
+  const int tile_id = a.ksplit > 1 ? (int)(blockIdx.x / (unsigned)a.ksplit) : (int)blockIdx.x;
+  const int nsteps = a.ksteps / a.ksplit;  // steps of this workgroup
+  const int step0 = slice * nsteps;        // its first step of K
   int tm_idx, tn_idx;
-  if (!tile_of(a.map, blockIdx.x, tm_idx, tn_idx)) return;  // padding of the tile map (whole workgroup)
+  if (!tile_of(a.map, tile_id, tm_idx, tn_idx)) return;  // padding of the tile map (whole workgroup)
   const int m0 = tm_idx * BM, n0 = tn_idx * BN;
 
   // ---- W: global -> registers -> LDS, packed --------------------------------
   // chunk q = tid + i*THREADS of the tile: row q/4, chunk q%4 of the step's 64 bytes
   u32x4 wr[W_LOADS];
   auto load_w = [&](int step) {
-    const int st = min(step, a.ksteps - 1);  // past the end: a harmless reload of the last step
+    const int st = step0 + min(step, nsteps - 1);  // past the end: a harmless reload of the last step
 #pragma unroll
     for (int i = 0; i < W_LOADS; ++i) {
       const int q = tid + i * THREADS;
@@ -124,7 +134,7 @@ __global__ __launch_bounds__(WM * WN * 64, (TM * TN >= 16 ? 1 : 2)) void gemm_di
     uint32_t s[TN][2];  // G32: s[j][0] holds both scales; else one 16-bit scale each
   };
   auto load_s = [&](int step, Scales& sc) {
-    const int st = min(step, a.ksteps - 1);
+    const int st = step0 + min(step, nsteps - 1);
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
       if (G32) {
@@ -144,7 +154,7 @@ __global__ __launch_bounds__(WM * WN * 64, (TM * TN >= 16 ? 1 : 2)) void gemm_di
   constexpr int XH = X_LOADS / 4;
   u32x4 xr[XH];
   auto load_x = [&](int step, int half, int part) {
-    const int k0 = min(step, a.ksteps - 1) * DK;
+    const int k0 = (step0 + min(step, nsteps - 1)) * DK;
 #pragma unroll
     for (int i = 0; i < XH; ++i) {
       const int u = tid + (part * XH + i) * THREADS;
@@ -308,12 +318,70 @@ __global__ __launch_bounds__(WM * WN * 64, (TM * TN >= 16 ? 1 : 2)) void gemm_di
   // counters at the loop head pessimistic.
   step(0, s0, std::false_type{});
   int s = 1;
-  for (; s + 1 < a.ksteps; s += 2) {
+  for (; s + 1 < nsteps; s += 2) {
     step(s, s1, std::true_type{});
     step(s + 1, s0, std::true_type{});
   }
-  if (s < a.ksteps) step(s, s1, std::true_type{});
+  if (s < nsteps) step(s, s1, std::true_type{});
   if constexpr (CARRY) group(bfB, -1);  // group 7 of the last step
+
+  if (a.ksplit > 1) {
+    // Publish this slice's partial tile; the workgroup that arrives last for the tile adds
+    // the ksplit partials in slice order (so the sum does not depend on who is last),
+    // resets the counter for the next launch and goes on to the epilogue.  Tiles and
+    // counters move with device-scope atomic accesses only (coherent between the L2
+    // caches of the chip by themselves; a plain access could be served from this XCD's
+    // L2).  Order: every wave's stores acknowledged (vmcnt(0)), workgroup barrier, counter.
+    constexpr int WAVE_FLOATS = TM * TN * 16 * 64;
+    const int tile_linear = tm_idx * a.map.tiles_n + tn_idx;
+    float* tile_base = a.workspace + (size_t)tile_linear * a.ksplit * (BM * BN);
+    float* mine = tile_base + (size_t)slice * (BM * BN) + wave * WAVE_FLOATS + lane;
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          __hip_atomic_store(mine + ((i * TN + j) * 16 + r) * 64, acc[i][j][r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): every store of this wave is acknowledged
+    __syncthreads();
+    int* flag = (int*)lds;  // the staging buffers are free behind the last barrier of the main loop
+    if (tid == 0) *flag = __hip_atomic_fetch_add(a.counters + tile_linear, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    const bool owner = *flag == a.ksplit - 1;  // workgroup-uniform
+    __syncthreads();                           // everyone has read the flag before LDS is reused
+    if (!owner) return;
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    const float* theirs = tile_base + wave * WAVE_FLOATS + lane;
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+        // the loads of four slices are issued together: one slice per round trip made the
+        // combine a chain of 4 * ksplit trips to memory (19 us of a 29 us launch)
+        for (int sl0 = 0; sl0 < a.ksplit; sl0 += 4) {
+          float v[4][16];
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const int sl = min(sl0 + q, a.ksplit - 1);  // ksplit = 2: the second slice again, not added below
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+              v[q][r] = __hip_atomic_load(theirs + (size_t)sl * (BM * BN) + ((i * TN + j) * 16 + r) * 64, __ATOMIC_RELAXED,
+                                          __HIP_MEMORY_SCOPE_AGENT);
+          }
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const bool keep = sl0 + q < a.ksplit;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] += keep ? v[q][r] : 0.f;
+          }
+        }
+      }
+    if (tid == 0) __hip_atomic_store(a.counters + tile_linear, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
 
   // Epilogue: one 32-row block of the wave at a time through a private LDS patch
   // (the staging buffers are free after the last barrier).
@@ -335,7 +403,7 @@ int launch_direct_tile(const DirectArgs& a, bool g32, hipStream_t stream) {
   int grid = 0;
   b.map = make_tile_map((a.m + BM - 1) / BM, (a.n + BN - 1) / BN, &grid);
   void* args[] = {(void*)&b};
-  return launch_kernel(fn, dim3(grid), dim3(WM * WN * 64), args, lds_bytes, stream);
+  return launch_kernel(fn, dim3(grid * (a.ksplit > 1 ? a.ksplit : 1)), dim3(WM * WN * 64), args, lds_bytes, stream);
 }
 
 struct DirectTile {
@@ -362,6 +430,8 @@ bool gemm_direct_config_applicable(const Problem& p, const tlhip_kernel_config_t
       "activations must be f16",
       "K must be a multiple of 128",
       "group size must be a multiple of 32",
+      "K split across workgroups (p5) must be 0, 1 or a power of two up to 16 that divides K / 128, with the partial "
+      "tiles (tiles x p5 x tile size, f32) and one counter per tile inside the library's workspace",
       "tile (M, N, waves M, waves N) must be one of 256x256 2x4, 256x128 2x4, 128x256 2x4, 256x128 4x2, 128x128 2x2, 256x256 2x2, 128x256 1x4, 128x192 2x2 with tile K 128",
   };
   auto fail = [&](int i) {
@@ -373,10 +443,18 @@ bool gemm_direct_config_applicable(const Problem& p, const tlhip_kernel_config_t
   if (p.x_dtype != TLHIP_F16) return fail(2);
   if (p.k % DK != 0 || p.k == 0) return fail(3);
   if (p.group_size % 32 != 0) return fail(4);
-  if (c.p2 != DK) return fail(5);
+  if (c.p2 != DK) return fail(6);
   for (const auto& t : kDirectTiles)
-    if (t.bm == c.p0 && t.bn == c.p1 && t.wm == c.p3 && t.wn == c.p4) return true;
-  return fail(5);
+    if (t.bm == c.p0 && t.bn == c.p1 && t.wm == c.p3 && t.wn == c.p4) {
+      const int ks = c.p5 < 1 ? 1 : c.p5;
+      if (ks > 1) {
+        if (ks > 16 || (ks & (ks - 1)) != 0 || (p.k / DK) % ks != 0) return fail(5);
+        const int64_t tiles = ((p.m + t.bm - 1) / t.bm) * ((p.n + t.bn - 1) / t.bn);
+        if (tiles > kSplitCounters || (size_t)tiles * ks * t.bm * t.bn > kSplitWorkspaceFloats) return fail(5);
+      }
+      return true;
+    }
+  return fail(6);
 }
 
 int launch_gemm_direct(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t stream) {
@@ -395,6 +473,13 @@ int launch_gemm_direct(const Problem& p, const tlhip_kernel_config_t& c, hipStre
   a.cpg_shift = __builtin_ctz((unsigned)(p.group_size / 32));
   a.groups_per_row = (int)(p.k / p.group_size);
   a.ksteps = (int)(p.k / DK);
+  a.ksplit = c.p5 < 1 ? 1 : c.p5;
+  a.workspace = nullptr;
+  a.counters = nullptr;
+  if (a.ksplit > 1) {
+    const int rc = split_workspace(stream, &a.workspace, &a.counters);
+    if (rc) return rc;
+  }
   a.out.y = p.y;
   a.out.y_dtype = p.y_dtype;
   a.out.vec_ok = (p.n % 8 == 0) && ((uintptr_t)p.y % 16 == 0);
@@ -423,6 +508,7 @@ int prepare_gemm_direct_kernels() {
   DirectArgs a;
   memset(&a, 0, sizeof a);
   a.m = a.n = 1;
+  a.ksplit = 1;
   for (bool g32 : {true, false}) {
     int rc = launch_direct_tile<2, 2, 4, 4>(a, g32, nullptr);
     if (!rc) rc = launch_direct_tile<2, 4, 4, 2>(a, g32, nullptr);
