@@ -190,23 +190,26 @@ bool config_applicable(const Problem& p, const tlhip_kernel_config_t& c, const c
 tlhip_kernel_config_t default_valu_config(const Problem& p);
 
 // Time of one round of 128 x 128 tiles of the direct GEMM with `ks` K slices across
-// workgroups, in microseconds: a workgroup walks 4096 of K in 42 us, and the slices cost 12
-// us plus 1.6 us each to combine (fitted at 4096..12288 x 4096..12288, M = 64..512).
-double direct_round_us(int64_t k, int ks) {
-  const double walk = 42.0 * (double)k / 4096.0 / ks;
-  return ks > 1 ? walk + 12.0 + 1.6 * ks : walk;
+// workgroups, in microseconds: a workgroup walks 4096 of K in 42 us; the slices' partial
+// sums (ks planes of M x N f32) are written and read back by a second launch, 6 us plus
+// 0.6 us per MB of planes (fitted at 4096..12288 x 4096..12288, M = 64..512).
+double direct_round_us(const Problem& p, int ks) {
+  const double walk = 42.0 * (double)p.k / 4096.0 / ks;
+  if (ks <= 1) return walk;
+  return walk + 6.0 + 0.6 * (double)ks * (double)p.m * (double)p.n * 4.0 / 1e6;
 }
 
 // K slices across workgroups for a launch of 128 x 128 tiles of the direct GEMM: of 1, 2,
-// 4, 8 the cheapest by direct_round_us that keeps tiles x slices within the CUs, divides
-// the 128-k steps and leaves every slice at least four of them.
+// 4, 8 the cheapest by direct_round_us that keeps tiles x slices within twice the CUs (two
+// workgroups of this tile share a CU), divides the 128-k steps and leaves every slice at
+// least four of them.
 int direct_k_split(const Problem& p) {
   const int cus = device_cu_count() > 0 ? device_cu_count() : 256;
   const int64_t tiles = ((p.m + 127) / 128) * ((p.n + 127) / 128);
   const int64_t steps = p.k / 128;
   int best = 1;
   for (int ks = 2; ks <= 8; ks *= 2)
-    if (tiles * ks <= cus && steps % ks == 0 && steps / ks >= 4 && direct_round_us(p.k, ks) < direct_round_us(p.k, best)) best = ks;
+    if (tiles * ks <= 2 * cus && steps % ks == 0 && steps / ks >= 4 && direct_round_us(p, ks) < direct_round_us(p, best)) best = ks;
   return best;
 }
 
@@ -226,8 +229,8 @@ tlhip_kernel_config_t default_config(const Problem& p) {
       tlhip_kernel_config_t c = t256 >= 2 * cus ? direct_cfg(256, 256, 2, 4)
                                 : (t128x256 >= 160 ? direct_cfg(128, 256, 1, 4) : direct_cfg(128, 128, 2, 2));
       if (c.p0 == 128 && c.p1 == 128) {
-        // fewer 128 x 128 tiles than CUs: 2, 4 or 8 workgroups share a tile, each walking a
-        // slice of K of at least four steps (4096 x 12288 at M = 256: 53 us against 141 us)
+        // few 128 x 128 tiles: 2, 4 or 8 workgroups share a tile, each walking a slice of K
+        // of at least four steps (4096 x 12288 at M = 256: 48 us against 141 us)
         const int ks = direct_k_split(p);
         if (ks > 1) {
           tlhip_kernel_config_t split = c;
@@ -379,11 +382,12 @@ std::vector<tlhip_kernel_config_t> candidates(const Problem& p) {
     }
     // K slices across workgroups where the 128 x 128 tiles are fewer than the CUs
     if (((p.m + 127) / 128) * ((p.n + 127) / 128) < (device_cu_count() > 0 ? device_cu_count() : 256))
-      for (int ks : {2, 4, 8}) {
-        tlhip_kernel_config_t c = direct_cfg(128, 128, 2, 2);
-        c.p5 = ks;
-        if (gemm_direct_config_applicable(p, c, nullptr)) out.push_back(c);
-      }
+      for (int ks : {2, 4, 8})
+        for (auto& t : {std::array<int, 4>{128, 128, 2, 2}, std::array<int, 4>{128, 256, 1, 4}}) {
+          tlhip_kernel_config_t c = direct_cfg(t[0], t[1], t[2], t[3]);
+          c.p5 = ks;
+          if (gemm_direct_config_applicable(p, c, nullptr)) out.push_back(c);
+        }
   }
   return out;
 }
@@ -599,7 +603,7 @@ Route plan_route(const Problem& p, const tlhip_kernel_config_t& c) {
     const int64_t passes = (p.m + 15) / 16;
     const int64_t tiles = ((p.m + 127) / 128) * ((p.n + 127) / 128);
     const double rounds = tiles <= 512 ? 1.0 : (double)tiles / 512.0;
-    const double tiled_us = direct_round_us(p.k, c.variant == VARIANT_TILED_DIRECT && c.p5 > 1 ? c.p5 : 1) * rounds;
+    const double tiled_us = direct_round_us(p, c.variant == VARIANT_TILED_DIRECT && c.p5 > 1 ? c.p5 : 1) * rounds;
     // Up to 64 rows per launch of the decode kernel: 1.2-1.6 times a 16-row pass for two
     // tiles of rows, 2.3-3.2 times for four (the activations a workgroup stages grow with
     // the rows, and their K slices are combined across workgroups).  More rows go 64 at a

@@ -58,8 +58,7 @@ struct DirectArgs {
   int groups_per_row;
   int ksteps;             // K / 128
   int ksplit;             // workgroups that share a tile, each walking ksteps / ksplit steps of K (1 = none)
-  float* workspace;       // ksplit > 1: partial tiles, [tile][slice][wave][MFMA tile][register][lane]
-  int* counters;          // ksplit > 1: arrival counters, one per tile; zero between launches
+  float* workspace;       // ksplit > 1: the slices' partial sums, [slice][M][N] f32
   TileMap map;
   OutArgs out;
 };
@@ -92,8 +91,9 @@ __global__ __launch_bounds__(WM * WN * 64, (TM * TN >= 16 ? 1 : 2)) void gemm_di
   const int lrow = lane & 31, lk = lane >> 5;
 
   // K split across workgroups: the ksplit workgroups of consecutive ids take the slices of
-  // one tile.  A launch of a few tiles (M of a few hundred rows on a decode-sized matrix)
-  // would leave most CUs idle while each workgroup walks all of K on its own.
+  // one tile and leave their partial sums in the workspace (a second launch adds them).  A
+  // launch of a few tiles (M of a few hundred rows on a decode-sized matrix) would leave
+  // most CUs idle while each workgroup walks all of K on its own.
   const int slice = a.ksplit > 1 ? (int)(blockIdx.x % (unsigned)a.ksplit) : 0;
   const int tile_id = a.ksplit > 1 ? (int)(blockIdx.x / (unsigned)a.ksplit) : (int)blockIdx.x;
   const int nsteps = a.ksteps / a.ksplit;  // steps of this workgroup
@@ -325,70 +325,73 @@ __global__ __launch_bounds__(WM * WN * 64, (TM * TN >= 16 ? 1 : 2)) void gemm_di
   if (s < nsteps) step(s, s1, std::true_type{});
   if constexpr (CARRY) group(bfB, -1);  // group 7 of the last step
 
-  if (a.ksplit > 1) {
-    // Publish this slice's partial tile; the workgroup that arrives last for the tile adds
-    // the ksplit partials in slice order (so the sum does not depend on who is last),
-    // resets the counter for the next launch and goes on to the epilogue.  Tiles and
-    // counters move with device-scope atomic accesses only (coherent between the L2
-    // caches of the chip by themselves; a plain access could be served from this XCD's
-    // L2).  Order: every wave's stores acknowledged (vmcnt(0)), workgroup barrier, counter.
-    constexpr int WAVE_FLOATS = TM * TN * 16 * 64;
-    const int tile_linear = tm_idx * a.map.tiles_n + tn_idx;
-    float* tile_base = a.workspace + (size_t)tile_linear * a.ksplit * (BM * BN);
-    float* mine = tile_base + (size_t)slice * (BM * BN) + wave * WAVE_FLOATS + lane;
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-      for (int j = 0; j < TN; ++j)
-#pragma unroll
-        for (int r = 0; r < 16; ++r)
-          __hip_atomic_store(mine + ((i * TN + j) * 16 + r) * 64, acc[i][j][r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): every store of this wave is acknowledged
-    __syncthreads();
-    int* flag = (int*)lds;  // the staging buffers are free behind the last barrier of the main loop
-    if (tid == 0) *flag = __hip_atomic_fetch_add(a.counters + tile_linear, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __syncthreads();
-    const bool owner = *flag == a.ksplit - 1;  // workgroup-uniform
-    __syncthreads();                           // everyone has read the flag before LDS is reused
-    if (!owner) return;
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-    const float* theirs = tile_base + wave * WAVE_FLOATS + lane;
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-      for (int j = 0; j < TN; ++j) {
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-        // the loads of four slices are issued together: one slice per round trip made the
-        // combine a chain of 4 * ksplit trips to memory (19 us of a 29 us launch)
-        for (int sl0 = 0; sl0 < a.ksplit; sl0 += 4) {
-          float v[4][16];
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            const int sl = min(sl0 + q, a.ksplit - 1);  // ksplit = 2: the second slice again, not added below
-#pragma unroll
-            for (int r = 0; r < 16; ++r)
-              v[q][r] = __hip_atomic_load(theirs + (size_t)sl * (BM * BN) + ((i * TN + j) * 16 + r) * 64, __ATOMIC_RELAXED,
-                                          __HIP_MEMORY_SCOPE_AGENT);
-          }
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            const bool keep = sl0 + q < a.ksplit;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] += keep ? v[q][r] : 0.f;
-          }
-        }
-      }
-    if (tid == 0) __hip_atomic_store(a.counters + tile_linear, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  }
-
   // Epilogue: one 32-row block of the wave at a time through a private LDS patch
   // (the staging buffers are free after the last barrier).
   float* patch = (float*)lds + wave * (32 * (TN * 32 + 4));
+  if (a.ksplit > 1) {
+    // a K slice: the bare partial sums, f32, row-major, into this slice's M x N plane of the
+    // workspace; direct_reduce_kernel adds the planes in slice order and runs the epilogue
+    OutArgs po;
+    po.y = a.workspace + (size_t)slice * a.m * a.n;
+    po.y_dtype = TLHIP_F32;
+    po.vec_ok = a.n % 8 == 0;
+    po.m = a.m;
+    po.n = a.n;
+    po.alpha = 1.f;
+    po.epi.n_ops = 0;
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+      wave_epilogue<TN>(patch, acc[i], lane, m0 + (wm * TM + i) * 32, n0 + wn * TN * 32, po);
+    return;
+  }
 #pragma unroll
   for (int i = 0; i < TM; ++i)
     wave_epilogue<TN>(patch, acc[i], lane, m0 + (wm * TM + i) * 32, n0 + wn * TN * 32, a.out);
+}
+
+// Second launch of a K-sliced GEMM: y = epilogue(alpha * sum over the slices' planes, in
+// slice order).  A reduction by the last workgroup to arrive for a tile (one launch) was
+// built first and cost 12 us + 1.6 us per slice: one CU reading up to 512 KB of partial
+// tiles with device-scope loads.  Here every CU takes its share, the kernel boundary orders
+// the planes' stores before these loads, and the sum is the same from launch to launch.
+// VEC: 8 consecutive columns per thread (N % 8 == 0, y 16-byte aligned), else one element.
+template <bool VEC>
+__global__ __launch_bounds__(256) void direct_reduce_kernel(const float* __restrict__ planes, int ks, const OutArgs o) {
+  const int64_t plane = (int64_t)o.m * o.n;
+  const int64_t idx = ((int64_t)blockIdx.x * 256 + threadIdx.x) * (VEC ? 8 : 1);
+  if (idx >= plane) return;
+  constexpr int W = VEC ? 8 : 1;
+  float v[W];
+#pragma unroll
+  for (int e = 0; e < W; ++e) v[e] = 0.f;
+  for (int sl = 0; sl < ks; ++sl) {
+    const float* src = planes + sl * plane + idx;
+    if (VEC) {
+      const float4_t a0 = __builtin_nontemporal_load((const float4_t*)src);
+      const float4_t a1 = __builtin_nontemporal_load((const float4_t*)(src + 4));
+      v[0] += a0[0]; v[1] += a0[1]; v[2] += a0[2]; v[3] += a0[3];
+      if (W == 8) { v[W - 4] += a1[0]; v[W - 3] += a1[1]; v[W - 2] += a1[2]; v[W - 1] += a1[3]; }
+    } else {
+      v[0] += __builtin_nontemporal_load(src);
+    }
+  }
+  const int64_t col = idx % o.n;
+#pragma unroll
+  for (int e = 0; e < W; ++e) v[e] = apply_epilogue(o.epi, v[e] * o.alpha, col + e);
+  if (VEC) {
+    if (o.y_dtype == TLHIP_F16) {
+      half8_t h;
+#pragma unroll
+      for (int e = 0; e < W; ++e) h[e] = (_Float16)v[e];
+      *(half8_t*)((_Float16*)o.y + idx) = h;
+    } else {
+      float* dst = (float*)o.y + idx;
+      *(float4_t*)dst = (float4_t){v[0], v[1], v[2], v[3]};
+      if (W == 8) *(float4_t*)(dst + 4) = (float4_t){v[W - 4], v[W - 3], v[W - 2], v[W - 1]};
+    }
+  } else {
+    store_out(o.y, o.y_dtype, idx, v[0]);
+  }
 }
 
 template <int WM, int WN, int TM, int TN>
@@ -430,8 +433,8 @@ bool gemm_direct_config_applicable(const Problem& p, const tlhip_kernel_config_t
       "activations must be f16",
       "K must be a multiple of 128",
       "group size must be a multiple of 32",
-      "K split across workgroups (p5) must be 0, 1 or a power of two up to 16 that divides K / 128, with the partial "
-      "tiles (tiles x p5 x tile size, f32) and one counter per tile inside the library's workspace",
+      "K split across workgroups (p5) must be 0, 1 or a power of two up to 16 that divides K / 128, with the slices' "
+      "partial sums (p5 x M x N, f32) inside the library's workspace",
       "tile (M, N, waves M, waves N) must be one of 256x256 2x4, 256x128 2x4, 128x256 2x4, 256x128 4x2, 128x128 2x2, 256x256 2x2, 128x256 1x4, 128x192 2x2 with tile K 128",
   };
   auto fail = [&](int i) {
@@ -449,8 +452,7 @@ bool gemm_direct_config_applicable(const Problem& p, const tlhip_kernel_config_t
       const int ks = c.p5 < 1 ? 1 : c.p5;
       if (ks > 1) {
         if (ks > 16 || (ks & (ks - 1)) != 0 || (p.k / DK) % ks != 0) return fail(5);
-        const int64_t tiles = ((p.m + t.bm - 1) / t.bm) * ((p.n + t.bn - 1) / t.bn);
-        if (tiles > kSplitCounters || (size_t)tiles * ks * t.bm * t.bn > kSplitWorkspaceFloats) return fail(5);
+        if ((size_t)p.m * (size_t)p.n * ks > kSplitWorkspaceFloats) return fail(5);
       }
       return true;
     }
@@ -475,9 +477,9 @@ int launch_gemm_direct(const Problem& p, const tlhip_kernel_config_t& c, hipStre
   a.ksteps = (int)(p.k / DK);
   a.ksplit = c.p5 < 1 ? 1 : c.p5;
   a.workspace = nullptr;
-  a.counters = nullptr;
   if (a.ksplit > 1) {
-    const int rc = split_workspace(stream, &a.workspace, &a.counters);
+    int* counters = nullptr;  // this kernel combines its slices in a second launch, not by arrival
+    const int rc = split_workspace(stream, &a.workspace, &counters);
     if (rc) return rc;
   }
   a.out.y = p.y;
@@ -499,6 +501,14 @@ int launch_gemm_direct(const Problem& p, const tlhip_kernel_config_t& c, hipStre
   else rc = launch_direct_tile<4, 2, 2, 2>(a, g32, stream);
   if (rc) return rc;
   TLHIP_CHECK_HIP(hipGetLastError());
+  if (a.ksplit > 1) {
+    const bool vec = a.out.vec_ok;
+    const int64_t threads = ((int64_t)a.m * a.n + (vec ? 7 : 0)) / (vec ? 8 : 1);
+    const unsigned grid = (unsigned)((threads + 255) / 256);
+    if (vec) hipLaunchKernelGGL(direct_reduce_kernel<true>, dim3(grid), dim3(256), 0, stream, a.workspace, a.ksplit, a.out);
+    else hipLaunchKernelGGL(direct_reduce_kernel<false>, dim3(grid), dim3(256), 0, stream, a.workspace, a.ksplit, a.out);
+    TLHIP_CHECK_HIP(hipGetLastError());
+  }
   count_gemm_dispatch();
   return TLHIP_OK;
 }
