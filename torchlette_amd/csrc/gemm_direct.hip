@@ -349,36 +349,65 @@ __global__ __launch_bounds__(WM * WN * 64, (TM * TN >= 16 ? 1 : 2)) void gemm_di
     wave_epilogue<TN>(patch, acc[i], lane, m0 + (wm * TM + i) * 32, n0 + wn * TN * 32, a.out);
 }
 
+// v[e] = ops(alpha * v[e]) for the W consecutive columns from `col` on.
+template <int W>
+__device__ __forceinline__ void apply_epilogue_scaled(const OutArgs& o, float (&v)[W], int64_t col) {
+#pragma unroll
+  for (int e = 0; e < W; ++e) v[e] *= o.alpha;
+#pragma unroll
+  for (int i = 0; i < TLHIP_MAX_EPILOGUE_OPS; ++i) {
+    if (i < o.epi.n_ops) {
+      if (o.epi.kind[i] == TLHIP_EPI_BIAS) {
+#pragma unroll
+        for (int e = 0; e < W; ++e) {
+          if (o.epi.input_dtype[i] == TLHIP_F16) v[e] += (float)((const _Float16*)o.epi.input[i])[col + e];
+          else v[e] += ((const float*)o.epi.input[i])[col + e];
+        }
+      } else if (o.epi.kind[i] == TLHIP_EPI_UNARY) {
+#pragma unroll
+        for (int e = 0; e < W; ++e) v[e] = apply_unary(o.epi.unary[i], v[e]);
+      }
+    }
+  }
+}
+
 // Second launch of a K-sliced GEMM: y = epilogue(alpha * sum over the slices' planes, in
 // slice order).  A reduction by the last workgroup to arrive for a tile (one launch) was
 // built first and cost 12 us + 1.6 us per slice: one CU reading up to 512 KB of partial
 // tiles with device-scope loads.  Here every CU takes its share, the kernel boundary orders
 // the planes' stores before these loads, and the sum is the same from launch to launch.
 // VEC: 8 consecutive columns per thread (N % 8 == 0, y 16-byte aligned), else one element.
-template <bool VEC>
-__global__ __launch_bounds__(256) void direct_reduce_kernel(const float* __restrict__ planes, int ks, const OutArgs o) {
+template <bool VEC, int KS>
+__global__ __launch_bounds__(256) void direct_reduce_kernel(const float* __restrict__ planes, const OutArgs o) {
   const int64_t plane = (int64_t)o.m * o.n;
   const int64_t idx = ((int64_t)blockIdx.x * 256 + threadIdx.x) * (VEC ? 8 : 1);
   if (idx >= plane) return;
   constexpr int W = VEC ? 8 : 1;
-  float v[W];
+  // every plane's loads issued before the first is added (a loop over a run-time slice
+  // count made each plane a round trip to memory of its own)
+  float part[KS][W];
 #pragma unroll
-  for (int e = 0; e < W; ++e) v[e] = 0.f;
-  for (int sl = 0; sl < ks; ++sl) {
+  for (int sl = 0; sl < KS; ++sl) {
     const float* src = planes + sl * plane + idx;
-    if (VEC) {
+    if constexpr (VEC) {
       const float4_t a0 = __builtin_nontemporal_load((const float4_t*)src);
       const float4_t a1 = __builtin_nontemporal_load((const float4_t*)(src + 4));
-      v[0] += a0[0]; v[1] += a0[1]; v[2] += a0[2]; v[3] += a0[3];
-      if (W == 8) { v[W - 4] += a1[0]; v[W - 3] += a1[1]; v[W - 2] += a1[2]; v[W - 1] += a1[3]; }
+      part[sl][0] = a0[0]; part[sl][1] = a0[1]; part[sl][2] = a0[2]; part[sl][3] = a0[3];
+      part[sl][W - 4] = a1[0]; part[sl][W - 3] = a1[1]; part[sl][W - 2] = a1[2]; part[sl][W - 1] = a1[3];
     } else {
-      v[0] += __builtin_nontemporal_load(src);
+      part[sl][0] = __builtin_nontemporal_load(src);
     }
   }
-  const int64_t col = idx % o.n;
+  float v[W];
 #pragma unroll
-  for (int e = 0; e < W; ++e) v[e] = apply_epilogue(o.epi, v[e] * o.alpha, col + e);
-  if (VEC) {
+  for (int e = 0; e < W; ++e) {
+    v[e] = 0.f;
+#pragma unroll
+    for (int sl = 0; sl < KS; ++sl) v[e] += part[sl][e];  // slice order
+  }
+  const int64_t col = idx % o.n;
+  apply_epilogue_scaled(o, v, col);
+  if constexpr (VEC) {
     if (o.y_dtype == TLHIP_F16) {
       half8_t h;
 #pragma unroll
@@ -387,11 +416,22 @@ __global__ __launch_bounds__(256) void direct_reduce_kernel(const float* __restr
     } else {
       float* dst = (float*)o.y + idx;
       *(float4_t*)dst = (float4_t){v[0], v[1], v[2], v[3]};
-      if (W == 8) *(float4_t*)(dst + 4) = (float4_t){v[W - 4], v[W - 3], v[W - 2], v[W - 1]};
+      *(float4_t*)(dst + 4) = (float4_t){v[W - 4], v[W - 3], v[W - 2], v[W - 1]};
     }
   } else {
     store_out(o.y, o.y_dtype, idx, v[0]);
   }
+}
+
+template <bool VEC>
+int launch_direct_reduce(int ks, unsigned grid, const float* planes, const OutArgs& o, hipStream_t stream) {
+  switch (ks) {
+    case 2: hipLaunchKernelGGL((direct_reduce_kernel<VEC, 2>), dim3(grid), dim3(256), 0, stream, planes, o); break;
+    case 4: hipLaunchKernelGGL((direct_reduce_kernel<VEC, 4>), dim3(grid), dim3(256), 0, stream, planes, o); break;
+    case 8: hipLaunchKernelGGL((direct_reduce_kernel<VEC, 8>), dim3(grid), dim3(256), 0, stream, planes, o); break;
+    default: hipLaunchKernelGGL((direct_reduce_kernel<VEC, 16>), dim3(grid), dim3(256), 0, stream, planes, o); break;
+  }
+  return TLHIP_OK;
 }
 
 template <int WM, int WN, int TM, int TN>
@@ -505,8 +545,8 @@ int launch_gemm_direct(const Problem& p, const tlhip_kernel_config_t& c, hipStre
     const bool vec = a.out.vec_ok;
     const int64_t threads = ((int64_t)a.m * a.n + (vec ? 7 : 0)) / (vec ? 8 : 1);
     const unsigned grid = (unsigned)((threads + 255) / 256);
-    if (vec) hipLaunchKernelGGL(direct_reduce_kernel<true>, dim3(grid), dim3(256), 0, stream, a.workspace, a.ksplit, a.out);
-    else hipLaunchKernelGGL(direct_reduce_kernel<false>, dim3(grid), dim3(256), 0, stream, a.workspace, a.ksplit, a.out);
+    if (vec) launch_direct_reduce<true>(a.ksplit, grid, a.workspace, a.out, stream);
+    else launch_direct_reduce<false>(a.ksplit, grid, a.workspace, a.out, stream);
     TLHIP_CHECK_HIP(hipGetLastError());
   }
   count_gemm_dispatch();
