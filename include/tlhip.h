@@ -375,7 +375,8 @@ typedef struct {
   int32_t p5; /* gemv: 1 = dot products on the 4x4x4 matrix-core instruction (int4, f16 x, m <= 4, p0 = 16, p1 = 1)
                * gemv_mfma: 1 = whole-line weight loads through a wave-private LDS patch (int8 with
                * K % 128 == 0 or int4-g32 with K % 256 == 0; p1 = 2 or 4)
-               * tiled_direct: K slices across workgroups (0/1 = none) */
+               * tiled, tiled_direct: K slices across workgroups (0/1 = none; 2..16: that many
+               * workgroups share a tile and a second launch adds their partial sums) */
   int32_t p6;
 } tlhip_kernel_config_t;
 

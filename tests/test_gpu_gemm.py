@@ -217,6 +217,30 @@ def test_direct_gemm_with_k_slices_across_workgroups(be, m, n, k, cfg, ydt):
     assert abs(rel_l2(unsplit, want) - err) <= 2e-5
 
 
+@pytest.mark.parametrize("fmt,g,m,n,k,cfg", [
+    ("int8-grouped", 64, 100, 384, 1024, (2, 128, 128, 64, 2, 2, 2)),
+    ("int8-row", 0, 130, 300, 2048, (2, 64, 128, 64, 2, 2, 8)),      # ragged rows and columns
+    ("int8-grouped", 128, 256, 512, 4096, (2, 128, 128, 64, 2, 2, 16)),
+    ("int4-grouped", 128, 70, 256, 2048, (2, 64, 128, 64, 2, 2, 4)),
+])
+@pytest.mark.parametrize("ydt", ["f16", "f32"])
+def test_staged_gemm_with_k_slices_across_workgroups(be, fmt, g, m, n, k, cfg, ydt):
+    """The LDS-staged GEMM (every format) with p5 workgroups per tile: against the oracle,
+    bit-stable from launch to launch, as close to the oracle as the unsplit kernel."""
+    rng = np.random.default_rng(m + n + k)
+    packed, scales, deq = make_weight(fmt, n, k, g, rng)
+    x = make_x(m, k, "f16", rng, std=0.5)
+    bias = f16_round(rng.standard_normal(n) * 0.1)
+    want = O.linear(x.astype(np.float32), deq, bias.astype(np.float32), "silu", threads=8)
+    got = run(be, fmt, packed, scales, n, k, g, x, ydt, bias=bias, act="silu", config=L.KernelConfig.of(*cfg))
+    err = rel_l2(got, want)
+    assert got.shape == (m, n) and err <= REL_L2_TOL, err
+    again = run(be, fmt, packed, scales, n, k, g, x, ydt, bias=bias, act="silu", config=L.KernelConfig.of(*cfg))
+    assert np.array_equal(again, got)
+    unsplit = run(be, fmt, packed, scales, n, k, g, x, ydt, bias=bias, act="silu", config=L.KernelConfig.of(*cfg[:6]))
+    assert abs(rel_l2(unsplit, want) - err) <= 2e-5
+
+
 def test_direct_gemm_k_slices_reject_what_they_do_not_cover(be):
     rng = np.random.default_rng(3)
     packed, scales, _ = make_weight("int4-grouped", 256, 1024, 32, rng)

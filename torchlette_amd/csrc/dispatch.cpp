@@ -193,8 +193,8 @@ tlhip_kernel_config_t default_valu_config(const Problem& p);
 // workgroups, in microseconds: a workgroup walks 4096 of K in 42 us; the slices' partial
 // sums (ks planes of M x N f32) are written and read back by a second launch, 6 us plus
 // 0.6 us per MB of planes (fitted at 4096..12288 x 4096..12288, M = 64..512).
-double direct_round_us(const Problem& p, int ks) {
-  const double walk = 42.0 * (double)p.k / 4096.0 / ks;
+double direct_round_us(const Problem& p, int ks, double walk_4096_us = 42.0) {
+  const double walk = walk_4096_us * (double)p.k / 4096.0 / ks;
   if (ks <= 1) return walk;
   return walk + 6.0 + 0.6 * (double)ks * (double)p.m * (double)p.n * 4.0 / 1e6;
 }
@@ -245,7 +245,20 @@ tlhip_kernel_config_t default_config(const Problem& p) {
     for (auto& t : tiles) {
       const int64_t wgs = ((p.m + t[0] - 1) / t[0]) * ((p.n + t[1] - 1) / t[1]);
       tlhip_kernel_config_t c = tiled_cfg(t[0], t[1], 64, 2, 2);
-      if ((wgs >= cus || t[0] == 64) && gemm_config_applicable(p, c, nullptr)) return c;
+      if (!(wgs >= cus || t[0] == 64) || !gemm_config_applicable(p, c, nullptr)) continue;
+      if (wgs < cus && t[1] == 128 && t[0] <= 128) {
+        // far fewer tiles than CUs: K slices across workgroups, the cheapest by the model
+        // (this kernel walks 4096 of K in 52 us), every slice at least 512 of K
+        int best = 1;
+        for (int ks = 2; ks <= 8; ks *= 2)
+          if (wgs * ks <= 2 * cus && (p.k / 64) % ks == 0 && p.k / ks >= 512 &&
+              direct_round_us(p, ks, 52.0) < direct_round_us(p, best, 52.0))
+            best = ks;
+        tlhip_kernel_config_t split = c;
+        split.p5 = best;
+        if (best > 1 && gemm_config_applicable(p, split, nullptr)) return split;
+      }
+      return c;
     }
   }
   // three or four rows of int4 weights with K up to 8192, from 8 MB of weights on: the
@@ -389,6 +402,13 @@ std::vector<tlhip_kernel_config_t> candidates(const Problem& p) {
     for (auto& t : tiles) {
       tlhip_kernel_config_t c = tiled_cfg(t[0], t[1], t[2], t[3], t[4]);
       if (gemm_config_applicable(p, c, nullptr)) out.push_back(c);
+      // K slices across workgroups where the tiles are fewer than the CUs
+      if (t[0] <= 128 && t[1] == 128 &&
+          ((p.m + t[0] - 1) / t[0]) * ((p.n + t[1] - 1) / t[1]) < (device_cu_count() > 0 ? device_cu_count() : 256))
+        for (int ks : {2, 4, 8}) {
+          c.p5 = ks;
+          if (gemm_config_applicable(p, c, nullptr)) out.push_back(c);
+        }
     }
     static const int direct[][4] = {{256, 256, 2, 4}, {256, 128, 2, 4}, {128, 256, 2, 4}, {256, 128, 4, 2}, {128, 128, 2, 2}, {256, 256, 2, 2}, {128, 256, 1, 4}, {128, 192, 2, 2}};
     for (auto& t : direct) {
@@ -508,7 +528,7 @@ bool f32_rows_through_tiled(const Problem& p, hipStream_t stream, int* rc) {
   Problem q = as_f16_activations(p);
   tlhip_kernel_config_t c = select_config(q);
   if (c.variant != VARIANT_TILED && c.variant != VARIANT_TILED_DIRECT) return false;
-  if (c.variant == VARIANT_TILED_DIRECT) c.p5 = 0;  // no K split across workgroups: its partial tiles live in the workspace too
+  c.p5 = 0;  // no K split across workgroups: its partial sums live in the workspace too
   const int64_t capacity = (int64_t)(kSplitWorkspaceFloats * sizeof(float) / sizeof(_Float16));
   int64_t rows = capacity / std::max<int64_t>(p.k, 1);
   if (rows >= 256) rows -= rows % 256;  // whole tiles per chunk
@@ -618,7 +638,7 @@ Route plan_route(const Problem& p, const tlhip_kernel_config_t& c) {
     const int64_t passes = (p.m + 15) / 16;
     const int64_t tiles = ((p.m + 127) / 128) * ((p.n + 127) / 128);
     const double rounds = tiles <= 512 ? 1.0 : (double)tiles / 512.0;
-    const double tiled_us = direct_round_us(p, c.variant == VARIANT_TILED_DIRECT && c.p5 > 1 ? c.p5 : 1) * rounds;
+    const double tiled_us = direct_round_us(p, c.p5 > 1 ? c.p5 : 1, c.variant == VARIANT_TILED_DIRECT ? 42.0 : 52.0) * rounds;
     // Up to 64 rows per launch of the decode kernel: 1.2-1.6 times a 16-row pass for two
     // tiles of rows, 2.3-3.2 times for four (the activations a workgroup stages grow with
     // the rows, and their K slices are combined across workgroups).  More rows go 64 at a
@@ -1286,7 +1306,7 @@ int tlhip_selected_config(const tlhip_qweight_t* w, int x_dtype, int64_t m, int 
   if (p.x_dtype == TLHIP_F32 && p.m >= kF32TiledFromRows) {
     // what tlhip_matmul_quantized launches for these rows: the f16 problem's tiled kernel
     tlhip_kernel_config_t c = select_config(as_f16_activations(p));
-    if (c.variant == VARIANT_TILED_DIRECT) c.p5 = 0;  // as f32_rows_through_tiled launches it
+    c.p5 = 0;  // as f32_rows_through_tiled launches it
     if (c.variant == VARIANT_TILED || c.variant == VARIANT_TILED_DIRECT) *out = c;
   }
   return TLHIP_OK;

@@ -59,6 +59,9 @@ struct OutArgs {
   DevEpilogue epi;
 };
 
+// Defined in gemm_direct.hip: the second launch of a K-sliced tiled GEMM.
+int launch_k_slice_reduce(int ks, const float* planes, const OutArgs& o, hipStream_t stream);
+
 // Epilogue of one 32-row block of a wave: TN accumulator tiles of
 // v_mfma_f32_32x32x16 side by side (32 x 32*TN outputs).  The accumulator layout
 // (lane l: column l%32, rows 8*(r/4) + 4*(l/32) + r%4) would give 64-byte row
@@ -67,9 +70,20 @@ struct OutArgs {
 // (bias indexed by n, unary) -> cast, stored as one 16-byte (f16) or two 16-byte
 // (f32) pieces, whole 128-byte lines per row for f16 and TN = 2.
 // `patch` holds 32 * (32*TN + 4) floats and belongs to this wave alone.
-template <int TN>
+// `plane` != null (a K slice of a K-sliced launch): the bare sums go to that M x N f32
+// plane instead, no alpha, no ops; `o` then only gives the shape.  (A modified copy of
+// `o` would do the same, but a copy of the kernel arguments whose op arrays are indexed
+// at run time lands in scratch memory.)
+// PLANE = false: instances that never take K slices compile without the choice.
+template <int TN, bool PLANE = false>
 __device__ __forceinline__ void wave_epilogue(float* patch, const float16_t (&acc)[TN], int lane, int row0,
-                                              int col0, const OutArgs& o) {
+                                              int col0, const OutArgs& o, float* plane = nullptr) {
+  const bool bare = PLANE && plane != nullptr;  // uniform
+  // read where they are used (with PLANE = false exactly the kernel-argument reads of before:
+  // hoisted copies cost scalar registers, and the largest instances have none to spare)
+  auto out_base = [&]() -> void* { return bare ? (void*)plane : o.y; };
+  auto out_dtype = [&]() -> int { return bare ? (int)TLHIP_F32 : o.y_dtype; };
+  auto out_alpha = [&]() -> float { return bare ? 1.f : o.alpha; };
   constexpr int PW = TN * 32 + 4;
   constexpr int LPR = TN * 4;     // lanes per row, 8 columns each
   constexpr int RPP = 64 / LPR;   // rows per pass (TN = 3: 5 rows on 60 lanes, four lanes idle)
@@ -83,11 +97,11 @@ __device__ __forceinline__ void wave_epilogue(float* patch, const float16_t (&ac
   const int rr0 = lane / LPR, cc = (lane % LPR) * 8;
   const bool lane_used = rr0 < RPP;
   const int col = col0 + cc;
-  const bool vec = o.vec_ok && col + 8 <= o.n;
+  const bool vec = (bare ? o.n % 8 == 0 : o.vec_ok != 0) && col + 8 <= o.n;
   // The common chain, [bias] then [unary], keeps the lane's 8 bias values in
   // registers across the passes (the column does not change) and runs no loop
   // over the ops per element.
-  const int n_ops = o.epi.n_ops;
+  const int n_ops = bare ? 0 : o.epi.n_ops;
   const bool has_bias = n_ops >= 1 && o.epi.kind[0] == TLHIP_EPI_BIAS;
   const int un_at = has_bias ? 1 : 0;
   const bool simple = n_ops <= un_at + 1 && (n_ops == un_at || o.epi.kind[un_at] == TLHIP_EPI_UNARY);
@@ -111,27 +125,27 @@ __device__ __forceinline__ void wave_epilogue(float* patch, const float16_t (&ac
     if (row < o.m && lane_used && p * RPP + rr0 < 32) {
       if (simple) {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) v[e] = apply_unary(unary, v[e] * o.alpha + bias[e]);
+        for (int e = 0; e < 8; ++e) v[e] = apply_unary(unary, v[e] * out_alpha() + bias[e]);
       } else {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) v[e] = apply_epilogue(o.epi, v[e] * o.alpha, min(col + e, o.n - 1));
+        for (int e = 0; e < 8; ++e) v[e] = apply_epilogue(o.epi, v[e] * out_alpha(), min(col + e, o.n - 1));
       }
       if (vec) {
         const int64_t idx = (int64_t)row * o.n + col;
-        if (o.y_dtype == TLHIP_F16) {
+        if (out_dtype() == TLHIP_F16) {
           half8_t h;
 #pragma unroll
           for (int e = 0; e < 8; ++e) h[e] = (_Float16)v[e];
-          __builtin_nontemporal_store(h, (half8_t*)((_Float16*)o.y + idx));  // written once, not read back: 0.5-1.5 % faster
+          __builtin_nontemporal_store(h, (half8_t*)((_Float16*)out_base() + idx));  // written once, not read back: 0.5-1.5 % faster
         } else {
-          float* dst = (float*)o.y + idx;
+          float* dst = (float*)out_base() + idx;
           __builtin_nontemporal_store((float4_t){v[0], v[1], v[2], v[3]}, (float4_t*)dst);
           __builtin_nontemporal_store((float4_t){v[4], v[5], v[6], v[7]}, (float4_t*)(dst + 4));
         }
       } else {
 #pragma unroll
         for (int e = 0; e < 8; ++e)
-          if (col + e < o.n) store_out(o.y, o.y_dtype, (int64_t)row * o.n + col + e, v[e]);
+          if (col + e < o.n) store_out(out_base(), out_dtype(), (int64_t)row * o.n + col + e, v[e]);
       }
     }
   }

@@ -328,25 +328,12 @@ __global__ __launch_bounds__(WM * WN * 64, (TM * TN >= 16 ? 1 : 2)) void gemm_di
   // Epilogue: one 32-row block of the wave at a time through a private LDS patch
   // (the staging buffers are free after the last barrier).
   float* patch = (float*)lds + wave * (32 * (TN * 32 + 4));
-  if (a.ksplit > 1) {
-    // a K slice: the bare partial sums, f32, row-major, into this slice's M x N plane of the
-    // workspace; direct_reduce_kernel adds the planes in slice order and runs the epilogue
-    OutArgs po;
-    po.y = a.workspace + (size_t)slice * a.m * a.n;
-    po.y_dtype = TLHIP_F32;
-    po.vec_ok = a.n % 8 == 0;
-    po.m = a.m;
-    po.n = a.n;
-    po.alpha = 1.f;
-    po.epi.n_ops = 0;
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-      wave_epilogue<TN>(patch, acc[i], lane, m0 + (wm * TM + i) * 32, n0 + wn * TN * 32, po);
-    return;
-  }
+  // a K slice leaves its bare partial sums, f32, row-major, in this slice's M x N plane of
+  // the workspace; the reduce launch adds the planes in slice order and runs the epilogue
+  float* const plane = a.ksplit > 1 ? a.workspace + (size_t)slice * a.m * a.n : nullptr;
 #pragma unroll
   for (int i = 0; i < TM; ++i)
-    wave_epilogue<TN>(patch, acc[i], lane, m0 + (wm * TM + i) * 32, n0 + wn * TN * 32, a.out);
+    wave_epilogue<TN, true>(patch, acc[i], lane, m0 + (wm * TM + i) * 32, n0 + wn * TN * 32, a.out, plane);
 }
 
 // v[e] = ops(alpha * v[e]) for the W consecutive columns from `col` on.
@@ -466,6 +453,18 @@ constexpr DirectTile kDirectTiles[] = {
 
 }  // namespace
 
+// y = epilogue(alpha * sum of the `ks` planes of o.m x o.n f32 partial sums at `planes`),
+// enqueued behind the launch that wrote them: the second launch of a K-sliced tiled GEMM.
+int launch_k_slice_reduce(int ks, const float* planes, const OutArgs& o, hipStream_t stream) {
+  const bool vec = o.vec_ok;
+  const int64_t threads = ((int64_t)o.m * o.n + (vec ? 7 : 0)) / (vec ? 8 : 1);
+  const unsigned grid = (unsigned)((threads + 255) / 256);
+  if (vec) launch_direct_reduce<true>(ks, grid, planes, o, stream);
+  else launch_direct_reduce<false>(ks, grid, planes, o, stream);
+  TLHIP_CHECK_HIP(hipGetLastError());
+  return TLHIP_OK;
+}
+
 bool gemm_direct_config_applicable(const Problem& p, const tlhip_kernel_config_t& c, const char** why) {
   static const char* reasons[] = {
       "not the tiled_direct variant",
@@ -542,12 +541,8 @@ int launch_gemm_direct(const Problem& p, const tlhip_kernel_config_t& c, hipStre
   if (rc) return rc;
   TLHIP_CHECK_HIP(hipGetLastError());
   if (a.ksplit > 1) {
-    const bool vec = a.out.vec_ok;
-    const int64_t threads = ((int64_t)a.m * a.n + (vec ? 7 : 0)) / (vec ? 8 : 1);
-    const unsigned grid = (unsigned)((threads + 255) / 256);
-    if (vec) launch_direct_reduce<true>(a.ksplit, grid, a.workspace, a.out, stream);
-    else launch_direct_reduce<false>(a.ksplit, grid, a.workspace, a.out, stream);
-    TLHIP_CHECK_HIP(hipGetLastError());
+    const int rr = launch_k_slice_reduce(a.ksplit, a.workspace, a.out, stream);
+    if (rr) return rr;
   }
   count_gemm_dispatch();
   return TLHIP_OK;

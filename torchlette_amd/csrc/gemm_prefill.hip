@@ -45,6 +45,8 @@ struct GemmArgs {
   float scale_mul;
   TileMap map;
   OutArgs out;
+  int ksplit;             // workgroups that share a tile, each walking ksteps / ksplit steps of K (1 = none)
+  float* workspace;       // ksplit > 1: the slices' partial sums, [slice][M][N] f32
 };
 
 // Unpack one 16-byte chunk to f16 values already multiplied by the scale.
@@ -104,7 +106,9 @@ struct WChunk<TLHIP_FMT_INT8_GROUPED> : WChunkInt8<TLHIP_FMT_INT8_GROUPED> {};
 template <>
 struct WChunk<TLHIP_FMT_INT8_ROW> : WChunkInt8<TLHIP_FMT_INT8_ROW> {};
 
-template <int FMT, int BM, int BN>
+// SPLIT: the instances that take K slices across workgroups (the 64- and 128-row tiles
+// with 128 columns, the ones a launch of few tiles uses); the others compile as without.
+template <int FMT, int BM, int BN, bool SPLIT>
 __global__ __launch_bounds__(256) void gemm_prefill_kernel(const GemmArgs a) {
   using WC = WChunk<FMT>;
   constexpr bool GROUPED = (FMT != TLHIP_FMT_INT8_ROW);
@@ -119,8 +123,14 @@ __global__ __launch_bounds__(256) void gemm_prefill_kernel(const GemmArgs a) {
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
+  // K split across workgroups, as in gemm_direct.hip: the ksplit workgroups of consecutive
+  // ids take the slices of one tile and leave their partial sums in the workspace.
+  const int slice = SPLIT ? (int)(blockIdx.x % (unsigned)a.ksplit) : 0;
+  const int tile_id = SPLIT ? (int)(blockIdx.x / (unsigned)a.ksplit) : (int)blockIdx.x;
+  const int nsteps = SPLIT ? a.ksteps / a.ksplit : a.ksteps;
+  const int step0 = slice * nsteps;
   int tm_idx, tn_idx;
-  if (!tile_of(a.map, blockIdx.x, tm_idx, tn_idx)) return;  // padding of the tile map (whole workgroup)
+  if (!tile_of(a.map, tile_id, tm_idx, tn_idx)) return;  // padding of the tile map (whole workgroup)
   const int m0 = tm_idx * BM, n0 = tn_idx * BN;
 
   // ---- global -> register staging -------------------------------------
@@ -129,13 +139,15 @@ __global__ __launch_bounds__(256) void gemm_prefill_kernel(const GemmArgs a) {
   // step ks, already in LDS), the tiles of step ks+1 go from registers to the
   // other LDS buffer, and the MFMAs run on step ks: every global load has D-1
   // full steps to arrive.  All loads are unconditional (clamped at the end).
-  constexpr int D = (BM + BN) >= 512 ? 3 : 4;
+  // (the int8 formats hold twice the packed weights per stage: three stages from 384 rows
+  // of tiles on, or the largest instances run out of registers)
+  constexpr int D = ((BM + BN) >= 512 || (FMT != TLHIP_FMT_INT4_GROUPED && (BM + BN) >= 384)) ? 3 : 4;
   u32x4 xr[D][X_LOADS];
   u32x4 wr[D][W_LOADS];
   uint32_t sr[D][W_LOADS];  // raw scale bits (f16) or f32 bits (int8-row)
 
   auto load_tiles = [&](int kstep, u32x4 (&xs)[X_LOADS], u32x4 (&ws)[W_LOADS], uint32_t (&ss)[W_LOADS]) {
-    const int k0 = min(kstep, a.ksteps - 1) * BK;
+    const int k0 = (step0 + min(kstep, nsteps - 1)) * BK;
 #pragma unroll
     for (int i = 0; i < X_LOADS; ++i) {
       const int u = tid + i * 256;
@@ -191,11 +203,11 @@ __global__ __launch_bounds__(256) void gemm_prefill_kernel(const GemmArgs a) {
   lds_barrier();
 
   const int lrow = lane & 31, lk = lane >> 5;
-  for (int ks0 = 0; ks0 < a.ksteps; ks0 += D) {
+  for (int ks0 = 0; ks0 < nsteps; ks0 += D) {
 #pragma unroll
     for (int s = 0; s < D; ++s) {
       const int ks = ks0 + s;
-      if (ks < a.ksteps) {  // uniform
+      if (ks < nsteps) {  // uniform
         const int buf = ks & 1;
         // stage s held step ks (already in LDS): refill it with step ks + D
         load_tiles(ks + D, xr[s], wr[s], sr[s]);
@@ -230,14 +242,22 @@ __global__ __launch_bounds__(256) void gemm_prefill_kernel(const GemmArgs a) {
   // copies of it; the compiler then stops unrolling and the accumulators fall
   // into scratch memory.
   float* patch = (float*)lds + wave * (32 * (TN * 32 + 4));
+  // a K slice leaves its bare partial sums, f32, row-major, in this slice's M x N plane of
+  // the workspace; the reduce launch adds the planes in slice order and runs the epilogue
+  float* const plane = SPLIT ? a.workspace + (size_t)slice * a.m * a.n : nullptr;
 #pragma unroll
   for (int i = 0; i < TM; ++i)
-    wave_epilogue<TN>(patch, acc[i], lane, m0 + wm * (BM / 2) + i * 32, n0 + wn * (BN / 2), a.out);
+    wave_epilogue<TN, SPLIT>(patch, acc[i], lane, m0 + wm * (BM / 2) + i * 32, n0 + wn * (BN / 2), a.out, plane);
 }
 
 template <int FMT, int BM, int BN>
 int launch_tile(const GemmArgs& a, hipStream_t stream) {
-  const void* fn = (const void*)gemm_prefill_kernel<FMT, BM, BN>;
+  const void* fn = (const void*)gemm_prefill_kernel<FMT, BM, BN, false>;
+  if constexpr (BN == 128 && BM <= 128) {
+    if (a.ksplit > 1) fn = (const void*)gemm_prefill_kernel<FMT, BM, BN, true>;
+  } else {
+    if (a.ksplit > 1) return set_error(TLHIP_ERR_INVALID, "gemm: K slices across workgroups take the 64x128 and 128x128 tiles");
+  }
   size_t lds_bytes = (size_t)2 * (BM + BN) * ROW_BYTES;
   const size_t patch_bytes = (size_t)4 * 32 * (BN / 64 * 32 + 4) * sizeof(float);
   if (lds_bytes < patch_bytes) lds_bytes = patch_bytes;
@@ -245,7 +265,7 @@ int launch_tile(const GemmArgs& a, hipStream_t stream) {
   int grid = 0;
   b.map = make_tile_map((a.m + BM - 1) / BM, (a.n + BN - 1) / BN, &grid);
   void* args[] = {(void*)&b};
-  return launch_kernel(fn, dim3(grid), dim3(256), args, lds_bytes, stream);
+  return launch_kernel(fn, dim3(grid * (a.ksplit > 1 ? a.ksplit : 1)), dim3(256), args, lds_bytes, stream);
 }
 
 template <int FMT>
@@ -269,6 +289,8 @@ bool gemm_config_applicable(const Problem& p, const tlhip_kernel_config_t& c, co
       "K must be a multiple of 64",
       "group size must be a multiple of 32 (int4) or 16 (int8)",
       "tile must be one of 256x256 (int4 only), 128x256, 256x128, 128x128, 64x128 with tile K 64 and 2x2 waves",
+      "K split across workgroups (p5) must be 0, 1 or a power of two up to 16 that divides K / 64, on the 64x128 or "
+      "128x128 tile, with the slices' partial sums (p5 x M x N, f32) inside the library's workspace",
   };
   auto fail = [&](int i) {
     if (why) *why = reasons[i];
@@ -285,6 +307,10 @@ bool gemm_config_applicable(const Problem& p, const tlhip_kernel_config_t& c, co
   if (!ok || c.p2 != 64 || c.p3 != 2 || c.p4 != 2) return fail(4);
   // the int8 dequantisation needs more registers: its 256 x 256 instance would spill
   if (bm == 256 && bn == 256 && p.format != TLHIP_FMT_INT4_GROUPED) return fail(4);
+  const int ks = c.p5 < 1 ? 1 : c.p5;
+  if (ks > 1 && (ks > 16 || (ks & (ks - 1)) != 0 || (p.k / BK) % ks != 0 || bn != 128 || bm > 128 ||
+                 (size_t)p.m * (size_t)p.n * ks > kSplitWorkspaceFloats))
+    return fail(5);
   return true;
 }
 
@@ -305,6 +331,13 @@ int launch_gemm(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t st
   a.cpg_shift = p.format == TLHIP_FMT_INT8_ROW ? 0 : __builtin_ctz((unsigned)(p.group_size / cw));
   a.groups_per_row = p.format == TLHIP_FMT_INT8_ROW ? 0 : (int)(p.k / p.group_size);
   a.ksteps = (int)(p.k / BK);
+  a.ksplit = c.p5 < 1 ? 1 : c.p5;
+  a.workspace = nullptr;
+  if (a.ksplit > 1) {
+    int* counters = nullptr;  // the slices are combined by a second launch, not by arrival
+    const int rc = split_workspace(stream, &a.workspace, &counters);
+    if (rc) return rc;
+  }
   a.scale_mul = p.format == TLHIP_FMT_INT8_GROUPED ? (1.0f / 127.0f) : 1.0f;
   a.out.y = p.y;
   a.out.y_dtype = p.y_dtype;
@@ -321,6 +354,10 @@ int launch_gemm(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t st
   }
   if (rc) return rc;
   TLHIP_CHECK_HIP(hipGetLastError());
+  if (a.ksplit > 1) {
+    rc = launch_k_slice_reduce(a.ksplit, a.workspace, a.out, stream);
+    if (rc) return rc;
+  }
   count_gemm_dispatch();
   return TLHIP_OK;
 }
@@ -330,11 +367,19 @@ int prepare_gemm_kernels() {
   GemmArgs a;
   memset(&a, 0, sizeof a);
   a.m = a.n = 1;
+  a.ksplit = 1;
   static const int tiles[][2] = {{256, 256}, {128, 256}, {256, 128}, {128, 128}, {64, 128}};
   for (auto& t : tiles) {
     int rc = launch_fmt<TLHIP_FMT_INT4_GROUPED>(t[0], t[1], a, nullptr);
     if (!rc && t[0] * t[1] != 256 * 256) rc = launch_fmt<TLHIP_FMT_INT8_GROUPED>(t[0], t[1], a, nullptr);
     if (!rc && t[0] * t[1] != 256 * 256) rc = launch_fmt<TLHIP_FMT_INT8_ROW>(t[0], t[1], a, nullptr);
+    if (!rc && t[1] == 128 && t[0] <= 128) {  // the K-sliced instances of these tiles
+      a.ksplit = 2;
+      rc = launch_fmt<TLHIP_FMT_INT4_GROUPED>(t[0], t[1], a, nullptr);
+      if (!rc) rc = launch_fmt<TLHIP_FMT_INT8_GROUPED>(t[0], t[1], a, nullptr);
+      if (!rc) rc = launch_fmt<TLHIP_FMT_INT8_ROW>(t[0], t[1], a, nullptr);
+      a.ksplit = 1;
+    }
     if (rc) return rc;
   }
   return TLHIP_OK;
