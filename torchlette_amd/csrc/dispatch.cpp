@@ -341,7 +341,12 @@ tlhip_kernel_config_t default_valu_config(const Problem& p) {
   // flight per lane means fewer rows in flight per CU and measured 5-25 % slower.
   // (a row need not be a whole number of passes: K = 11008 and 18944 measured 7.8 and
   // 10.2 us with 32 lanes per row against 10.7 and 15.8 us with 16)
-  const int lpr = nchunks > 128 ? 32 : 16;
+  // Fewer rows than give every CU two workgroups of four waves: more lanes per row (a
+  // 1024 x 1024 matrix took 4.4 us with 16 lanes per row and 3.4 us with 64).
+  const int cus = device_cu_count() > 0 ? device_cu_count() : 256;
+  int lpr = nchunks > 128 ? 32 : 16;
+  const bool long_at_base = (nchunks + lpr - 1) / lpr >= 12;  // long rows keep their lanes (K = 18944: 10.2 against 12.6 us)
+  while (!long_at_base && lpr < 64 && p.n * lpr / 256 < 2 * cus) lpr *= 2;
   const int per_lane = (int)((nchunks + lpr - 1) / lpr);
   const bool long_rows = per_lane >= 12;
   return gemv_cfg(lpr, 1, long_rows ? 8 : 4, 1, long_rows ? 4 : 2);
