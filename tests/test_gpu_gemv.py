@@ -117,13 +117,15 @@ def test_more_than_16_rows_reject_what_the_matrix_core_gemv_does_not_cover(be):
         be.linear(x65, w, config=L.KernelConfig.of(1, 8, 1, 8, 1))
 
 
-@pytest.mark.parametrize("m", [9, 15, 16])
-def test_rows_whose_activations_fit_no_matrix_core_geometry_run_as_two_halves(be, m):
-    """K = 11008 (86 steps of 128): two K slices of 15 or 16 rows do not fit LDS and four do
-    not divide the steps.  The library then launches rows 0..7 and the rest on the matrix
-    cores (two dispatches) instead of the VALU kernel's pass per four rows; M = 9 still
-    fits as it is.  Heuristic defaults (no tuned entry can name such a pair)."""
-    n, k = 768, 11008
+@pytest.mark.parametrize("m", [5, 9, 15, 16, 40])
+@pytest.mark.parametrize("k", [11008, 13696])
+def test_k_whose_steps_do_not_divide_over_the_slices(be, m, k):
+    """K = 11008 is 86 steps of 128 and K = 13696 is 107: two equal slices of 16 rows do not
+    fit LDS and four do not divide the steps.  The matrix-core kernel then takes slices of
+    unequal length (22, 22, 21, 21), one launch, instead of falling to the VALU kernel's
+    pass per four rows.  Heuristic defaults; against the oracle, and every explicit
+    configuration with unequal slices gives the same bits from launch to launch."""
+    n = 768
     rng = np.random.default_rng(k + m)
     packed, scales, deq = make_weight("int4-grouped", n, k, 32, rng)
     x = make_x(m, k, "f16", rng)
@@ -135,9 +137,16 @@ def test_rows_whose_activations_fit_no_matrix_core_geometry_run_as_two_halves(be
         launches = T.getQuantGemvDispatchCount() - before
     finally:
         T.importTuningCache(saved)
-    assert launches == (1 if m == 9 else 2), launches
+    assert launches == 1, launches
     want = O.linear(x.astype(np.float32), deq, threads=8)
     assert rel_l2(got, want) <= 2e-6, rel_l2(got, want)
+    if m <= 16:
+        for cfg in ((1, 8, 1, 8, 4), (1, 8, 1, 2, 8), (1, 4, 1, 1, 16)):
+            a = run_linear(be, "int4-grouped", packed, scales, n, k, 32, x, "f32", config=L.KernelConfig.of(*cfg))
+            b = run_linear(be, "int4-grouped", packed, scales, n, k, 32, x, "f32", config=L.KernelConfig.of(*cfg))
+            assert rel_l2(a, want) <= 2e-6 and np.array_equal(a, b), cfg
+        with pytest.raises(L.TlhipError, match="slices of unequal length"):
+            run_linear(be, "int4-grouped", packed, scales, n, k, 32, x, "f32", config=L.KernelConfig.of(1, 8, 2, 8, 4))
 
 
 @pytest.mark.parametrize("fmt,n,k,g", [

@@ -612,10 +612,11 @@ struct Route {
   tlhip_kernel_config_t last;   // configuration of the remaining rows, if any
 };
 
-// 9..16 rows whose activations fit no geometry of the matrix-core kernels (K = 11008 at
-// M = 15 or 16: two K slices of 16 rows take 176 KB of LDS, and four do not divide its
-// 86 steps) would fall to the VALU kernel, which streams the weights once per four rows;
-// two launches of at most 8 rows on the matrix cores stream them twice.
+// 9..16 rows whose activations fit no geometry of the matrix-core kernels (a very long K
+// whose steps no power of two up to 16 slices finely enough) would fall to the VALU kernel,
+// which streams the weights once per four rows; two launches of at most 8 rows on the
+// matrix cores stream them twice.  (K = 11008 and 13696 were such cases until the kernel
+// took K slices of unequal length.)
 //
 // A few more rows than the decode kernels take, far fewer than fill the chip with
 // tiles: a tiled launch of at most one round of 128 x 128 tiles takes the time ONE

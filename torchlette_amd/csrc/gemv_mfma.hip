@@ -18,11 +18,12 @@ struct MfmaGeometry {
 // Tiles of 16 activation rows per weight row block: 1, 2 or 4 (M <= 16 / 32 / 64).
 static int row_tiles(int64_t m) { return m <= 16 ? 1 : (m <= 32 ? 2 : 4); }
 
-static bool mfma_geometry(int64_t nblocks, int64_t k, int64_t m, int waves, int kw, int ks, size_t patch_bytes, MfmaGeometry* out) {
+// `slice_k`: activations of one K slice per row (the longest slice).
+static bool mfma_geometry(int64_t nblocks, int64_t slice_k, int64_t m, int waves, int kw, int ks, size_t patch_bytes, MfmaGeometry* out) {
   const int threads = waves * 64;
   const int blocks_per_wg = waves / kw;
   const int64_t nwgblocks = (nblocks + blocks_per_wg - 1) / blocks_per_wg;
-  const size_t x_bytes = (size_t)m * (k / ks * 2 + 16);
+  const size_t x_bytes = (size_t)m * (slice_k * 2 + 16);
   const int cus = device_cu_count() > 0 ? device_cu_count() : 256;
   for (int per_cu = 2048 / threads; per_cu >= 1; --per_cu) {
     int64_t sets = (int64_t)cus * per_cu / ks;
@@ -63,7 +64,8 @@ static bool mfma_applicable(const Problem& p, int64_t nblocks, const tlhip_kerne
       "iterations in flight must be 1, 2 or 4 (1 or 2 above 32 rows)",
       "K-split waves must be a power of two that divides the waves per workgroup",
       "activations (M x K/slices f16) plus one parked tile per round and wave do not fit LDS",
-      "K slices must be a power of two (1..16) that divides K/128 (int4) or K/64 (int8)",
+      "K slices must be a power of two (1..16) that divides K/128 (int4) or K/64 (int8); slices of unequal length "
+      "(any power of two up to the step count) take one iteration in flight and no whole-line loads",
       "K slices need more partial-tile workspace or counters than the library holds",
       "iterations in flight must divide the 128-weight (int4) or 64-weight (int8) steps of a K slice",
       "whole-line weight loads (p5 = 1) need int8 (K % 128 == 0) or int4 with group size 32 "
@@ -89,16 +91,19 @@ static bool mfma_applicable(const Problem& p, int64_t nblocks, const tlhip_kerne
   if (kw < 1 || (kw & (kw - 1)) != 0 || c.p0 % kw != 0) return fail(7);
   const int ks = c.p3 < 1 ? 1 : c.p3;
   const int64_t iters = p.k / kper;
-  if (ks > 16 || (ks & (ks - 1)) != 0 || iters % ks != 0) return fail(9);
+  if (ks > 16 || (ks & (ks - 1)) != 0 || ks > iters) return fail(9);
+  const bool uneven = iters % ks != 0;
+  if (uneven && (c.p1 != 1 || c.p5 != 0)) return fail(9);
+  const int64_t slice_k = (iters / ks + (uneven ? 1 : 0)) * kper;  // the longest slice
   if (c.p5 != 0) {
     // a pair of iterations = one 128-byte line per row: 128 k of int8, 256 k of int4
     const bool fmt_ok = ((p.format == TLHIP_FMT_INT8_ROW || p.format == TLHIP_FMT_INT8_GROUPED) && p.k % 128 == 0) ||
                         (p.format == TLHIP_FMT_INT4_GROUPED && p.group_size == 32 && p.k % 256 == 0);
-    if (!(c.p5 == 1 && fmt_ok && (c.p1 == 2 || c.p1 == 4) && (iters / ks) % 2 == 0)) return fail(12);
+    if (!(c.p5 == 1 && fmt_ok && (c.p1 == 2 || c.p1 == 4) && !uneven && (iters / ks) % 2 == 0)) return fail(12);
   }
   MfmaGeometry geo;
-  if (!mfma_geometry(nblocks, p.k, p.m, c.p0, kw, ks, line_patch_bytes(c), &geo)) return fail(8);
-  if ((iters / ks) % c.p1 != 0) return fail(11);
+  if (!mfma_geometry(nblocks, slice_k, p.m, c.p0, kw, ks, line_patch_bytes(c), &geo)) return fail(8);
+  if (!uneven && (iters / ks) % c.p1 != 0) return fail(11);
   if (ks > 1 && (nblocks > scratch_counters(p) || (size_t)nblocks * ks * 256 * row_tiles(p.m) > scratch_tile_floats(p)))
     return fail(10);
   return true;
@@ -160,6 +165,7 @@ int launch_gemv_mfma_group(const Problem* ps, int count, const tlhip_kernel_conf
   a.ks = c.p3 < 1 ? 1 : c.p3;
   a.ks_shift = __builtin_ctz((unsigned)a.ks);
   a.slice_iters = a.iters / a.ks;
+  a.slice_rem = a.iters % a.ks;
   a.kw = c.p2 == 0 ? waves : c.p2;
   a.kw_shift = __builtin_ctz((unsigned)a.kw);
   a.blocks_per_wg = waves / a.kw;
@@ -177,7 +183,8 @@ int launch_gemv_mfma_group(const Problem* ps, int count, const tlhip_kernel_conf
   a.scale_mul = p.format == TLHIP_FMT_INT8_GROUPED ? (1.0f / 127.0f) : 1.0f;
   a.y_dtype = p.y_dtype;
   MfmaGeometry geo;
-  if (!mfma_geometry(nblocks, p.k, p.m, waves, a.kw, a.ks, line_patch_bytes(c), &geo))
+  const int kper = int4 ? 128 : 64;
+  if (!mfma_geometry(nblocks, (int64_t)(a.slice_iters + (a.slice_rem ? 1 : 0)) * kper, p.m, waves, a.kw, a.ks, line_patch_bytes(c), &geo))
     return set_error(TLHIP_ERR_INVALID, "gemv_mfma: launch geometry does not close");
   const size_t lds_bytes = geo.lds_bytes;
   a.patch_unit = (int)(geo.patch_offset / 16);

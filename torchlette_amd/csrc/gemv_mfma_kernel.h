@@ -58,7 +58,8 @@ struct MfmaArgs {
   int groups_per_row;
   int ks;             // K slices handled by different workgroups (1 = none, power of two)
   int ks_shift;
-  int slice_iters;    // wave iterations (4 chunks each) per K slice
+  int slice_iters;    // wave iterations (4 chunks each) per K slice (the shorter slices, if they differ)
+  int slice_rem;      // iterations that do not divide over the slices: the first slice_rem slices take one more
   int iters;          // wave iterations over all of K
   int kw;             // waves that split a slice for one 16-row block (power of two)
   int kw_shift;
@@ -141,9 +142,15 @@ __global__ __launch_bounds__(MAXT) void gemv_mfma_kernel(const MfmaArgs a) {
   const int slice = blockIdx.x & (a.ks - 1);
   const int wg_stride = gridDim.x >> a.ks_shift;
   int wgb = blockIdx.x >> a.ks_shift;
-  const int it_begin = slice * a.slice_iters;
+  // K slices of unequal length (K = 11008: 86 iterations over 4 slices = 22, 22, 21, 21)
+  int my_iters = a.slice_iters, it_begin = slice * a.slice_iters, nsteps = a.nsteps;
+  if (a.slice_rem) {
+    my_iters += slice < a.slice_rem ? 1 : 0;
+    it_begin += min(slice, a.slice_rem);
+    nsteps = (my_iters / U + a.kw - 1) >> a.kw_shift;
+  }
   constexpr int UNITS_PER_ITER = FMT == TLHIP_FMT_INT4_GROUPED ? 16 : 8;  // 16-byte x units per iteration
-  const int slice_units = a.slice_iters * UNITS_PER_ITER;  // resident x units per row
+  const int slice_units = my_iters * UNITS_PER_ITER;  // resident x units per row
   const int row_units = slice_units + 1;                    // padded LDS row stride
   const int ku0 = it_begin * UNITS_PER_ITER;                // first resident unit
   const int k_units = a.k >> 3;                             // units per activation row in memory
@@ -161,7 +168,7 @@ __global__ __launch_bounds__(MAXT) void gemv_mfma_kernel(const MfmaArgs a) {
     uint16_t s[U][NS];      // !WIDE
     uint32_t sv[2 * U];     // WIDE: scale 4u+s in half (s & 1) of word 2u + s/2
   };
-  const int nbatches = a.slice_iters / U;  // U divides the iterations of a slice
+  const int nbatches = my_iters / U;  // U divides the iterations of a slice
 
   // row block of the launch -> its problem (wave-uniform).  In the hot loop the problem's
   // fields are SELECTED from the four table entries, each read with a constant index (so
@@ -560,16 +567,16 @@ __global__ __launch_bounds__(MAXT) void gemv_mfma_kernel(const MfmaArgs a) {
   // counters at the join assume it was NOT issued, and the consumer of the other
   // set would then wait for the load just issued.
   const int rounds = (a.nwgblocks - wgb + wg_stride - 1) / wg_stride;
-  const int total = rounds * a.nsteps;
+  const int total = rounds * nsteps;
   auto advance = [&](int& b, int& st) {
-    if (++st == a.nsteps) {
+    if (++st == nsteps) {
       st = 0;
       b += wg_stride;
     }
   };
   auto consume = [&](const Batch& b, int wb, int st) __attribute__((always_inline)) {
     compute_batch(b, st);
-    if (st == a.nsteps - 1) finish(wb);
+    if (st == nsteps - 1) finish(wb);
   };
   Batch other;
   int j = 0;
