@@ -283,6 +283,7 @@ def test_a_few_more_rows_than_16_go_through_the_decode_kernel(be, m, passes, ydt
     ("int4-grouped", 128, 4352, 256, 4096, "f32"),     # more rows than one workspace chunk holds (4096 at K = 4096)
     ("int8-grouped", 64, 96, 256, 512, "f32"),
     ("int8-row", 0, 130, 192, 768, "f32"),
+    ("int4-grouped", 32, 64, 4096, 4096, "f32"),       # the f16 problem's tuned winner is the skinny kernel: the heuristic tile serves
 ])
 def test_f32_activations_from_64_rows_take_the_matrix_cores(be, fmt, g, m, n, k, ydt):
     """f32 activations, 64 rows or more: rounded to f16 once, then the prefill GEMM of

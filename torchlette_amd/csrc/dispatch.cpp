@@ -532,6 +532,9 @@ bool f32_rows_through_tiled(const Problem& p, hipStream_t stream, int* rc) {
   if (p.x_dtype != TLHIP_F32 || p.m < kF32TiledFromRows || p.pro.kind != TLHIP_PRO_NONE) return false;
   Problem q = as_f16_activations(p);
   tlhip_kernel_config_t c = select_config(q);
+  // (a tuned winner of the f16 problem may be the skinny kernel, which keeps its K-slice
+  // tiles where the rounded rows are: the heuristic tile then)
+  if (c.variant != VARIANT_TILED && c.variant != VARIANT_TILED_DIRECT) c = default_config(q);
   if (c.variant != VARIANT_TILED && c.variant != VARIANT_TILED_DIRECT) return false;
   c.p5 = 0;  // no K split across workgroups: its partial sums live in the workspace too
   const int64_t capacity = (int64_t)(kSplitWorkspaceFloats * sizeof(float) / sizeof(_Float16));
@@ -1312,6 +1315,7 @@ int tlhip_selected_config(const tlhip_qweight_t* w, int x_dtype, int64_t m, int 
   if (p.x_dtype == TLHIP_F32 && p.m >= kF32TiledFromRows) {
     // what tlhip_matmul_quantized launches for these rows: the f16 problem's tiled kernel
     tlhip_kernel_config_t c = select_config(as_f16_activations(p));
+    if (c.variant != VARIANT_TILED && c.variant != VARIANT_TILED_DIRECT) c = default_config(as_f16_activations(p));
     c.p5 = 0;  // as f32_rows_through_tiled launches it
     if (c.variant == VARIANT_TILED || c.variant == VARIANT_TILED_DIRECT) *out = c;
   }
