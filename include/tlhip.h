@@ -267,8 +267,8 @@ int tlhip_gemm_prefill(const tlhip_qweight_t* w, const void* x, int x_dtype, int
  * tiles than the chip has CUs (batched decode at batch 32..128) go through the
  * skinny matrix-core GEMV, up to 64 rows per launch, while the library's cost
  * model puts that below one tiled launch; a tuned entry of the problem itself
- * overrides the model.  f32 activations: up to 63 rows run as GEMV passes of <= 16
- * rows in f32 arithmetic; from 64 rows on they are rounded to f16 (the operand
+ * overrides the model.  f32 activations: up to 16 rows run on the VALU kernel in
+ * f32 arithmetic; from 17 rows on they are rounded to f16 (the operand
  * type of the matrix cores; |x| above 65504 becomes inf) by a cast launch into
  * the stream's workspace and take the prefill GEMM of the f16 problem, which is
  * the configuration tlhip_selected_config then reports.  Like a K-sliced GEMV,

@@ -173,7 +173,10 @@ def test_config4_full_size(be, m, act):
     assert rel_l2(y1, pre) <= 5e-4
 
 
-def test_gemm_rejects_f32_activations_and_falls_back_to_gemv_passes(be):
+def test_gemm_rejects_f32_activations_as_an_explicit_configuration(be):
+    """A tiled configuration named by the caller takes f16 activations only; without one,
+    f32 rows above 16 are rounded to f16 and take the tiled kernel (next test), up to 16
+    rows stay on the VALU kernel's f32 arithmetic."""
     rng = np.random.default_rng(41)
     m, n, k = 40, 256, 512
     packed, scales, deq = make_weight("int8-grouped", n, k, 64, rng)
@@ -182,10 +185,15 @@ def test_gemm_rejects_f32_activations_and_falls_back_to_gemv_passes(be):
     xt = be.ops.tensorFromArray(x, [m, k], "f32")
     with pytest.raises(L.TlhipError, match="activations must be f16"):
         be.linear(xt, w, config=tiled(128, 128))
-    v0 = T.getQuantGemvDispatchCount()
+    v0, g0 = T.getQuantGemvDispatchCount(), T.getQuantGemmDispatchCount()
     y = be.linear(xt, w).numpy()
-    assert T.getQuantGemvDispatchCount() == v0 + 3      # 16 + 16 + 8 rows
-    assert rel_l2(y, O.linear(x, deq)) <= 2e-6
+    assert T.getQuantGemvDispatchCount() == v0 and T.getQuantGemmDispatchCount() == g0 + 1
+    assert rel_l2(y, O.linear(x, deq)) <= REL_L2_TOL
+    x16 = be.ops.tensorFromArray(x[:16].copy(), [16, k], "f32")
+    v0 = T.getQuantGemvDispatchCount()
+    y16 = be.linear(x16, w).numpy()
+    assert T.getQuantGemvDispatchCount() == v0 + 1
+    assert rel_l2(y16, O.linear(x[:16], deq)) <= 2e-6
 
 
 @pytest.mark.parametrize("m,n,k,cfg", [
@@ -278,6 +286,7 @@ def test_a_few_more_rows_than_16_go_through_the_decode_kernel(be, m, passes, ydt
 
 
 @pytest.mark.parametrize("fmt,g,m,n,k,ydt", [
+    ("int4-grouped", 32, 17, 256, 512, "f32"),
     ("int4-grouped", 32, 64, 256, 512, "f32"),
     ("int4-grouped", 32, 300, 384, 1024, "f32"),       # ragged rows and tiles
     ("int4-grouped", 128, 4352, 256, 4096, "f32"),     # more rows than one workspace chunk holds (4096 at K = 4096)
@@ -285,8 +294,8 @@ def test_a_few_more_rows_than_16_go_through_the_decode_kernel(be, m, passes, ydt
     ("int8-row", 0, 130, 192, 768, "f32"),
     ("int4-grouped", 32, 64, 4096, 4096, "f32"),       # the f16 problem's tuned winner is the skinny kernel: the heuristic tile serves
 ])
-def test_f32_activations_from_64_rows_take_the_matrix_cores(be, fmt, g, m, n, k, ydt):
-    """f32 activations, 64 rows or more: rounded to f16 once, then the prefill GEMM of
+def test_f32_activations_from_17_rows_take_the_matrix_cores(be, fmt, g, m, n, k, ydt):
+    """f32 activations, 17 rows or more: rounded to f16 once, then the prefill GEMM of
     the f16 problem (no GEMV dispatch).  Checked against the oracle on the ORIGINAL f32
     activations at the stated bar (rel-L2 <= 1e-3: the rounding of x to f16 costs about
     3e-4), and against the oracle on the rounded activations at the prefill kernels' own

@@ -512,9 +512,10 @@ int run_config(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t str
   return launch_gemv(p, c, stream);
 }
 
-// From this many rows on, f32 activations take the matrix-core route below; fewer rows
-// stay on the f32 arithmetic of the GEMV passes (at most four of them).
-constexpr int64_t kF32TiledFromRows = 64;
+// From this many rows on, f32 activations take the matrix-core route below: up to 16 rows
+// (decode) stay on the f32 arithmetic of the VALU kernel; beyond, that kernel would stream
+// the weights once per four rows (63 rows: 16 times).
+constexpr int64_t kF32TiledFromRows = 17;
 
 // The problem an f32-activation prefill runs as: the same one on f16 activations.
 Problem as_f16_activations(const Problem& p) {
