@@ -200,16 +200,16 @@ double direct_round_us(const Problem& p, int ks, double walk_4096_us = 42.0) {
 }
 
 // K slices across workgroups for a launch of 128 x 128 tiles of the direct GEMM: of 1, 2,
-// 4, 8 the cheapest by direct_round_us that keeps tiles x slices within twice the CUs (two
-// workgroups of this tile share a CU), divides the 128-k steps and leaves every slice at
-// least four of them.
+// 4, 8 the cheapest by direct_round_us that keeps tiles x slices within the CUs (beyond,
+// the slices of a tile queue behind each other), divides the 128-k steps and leaves every
+// slice at least four of them.
 int direct_k_split(const Problem& p) {
   const int cus = device_cu_count() > 0 ? device_cu_count() : 256;
   const int64_t tiles = ((p.m + 127) / 128) * ((p.n + 127) / 128);
   const int64_t steps = p.k / 128;
   int best = 1;
   for (int ks = 2; ks <= 8; ks *= 2)
-    if (tiles * ks <= 2 * cus && steps % ks == 0 && steps / ks >= 4 && direct_round_us(p, ks) < direct_round_us(p, best)) best = ks;
+    if (tiles * ks <= cus && steps % ks == 0 && steps / ks >= 4 && direct_round_us(p, ks) < direct_round_us(p, best)) best = ks;
   return best;
 }
 
@@ -240,18 +240,20 @@ tlhip_kernel_config_t default_config(const Problem& p) {
       }
       if (gemm_direct_config_applicable(p, c, nullptr)) return c;
     }
-    // largest tile that still gives every CU a workgroup
-    static const int tiles[][2] = {{256, 256}, {256, 128}, {128, 128}, {64, 128}};
+    // The LDS-staged kernel (the int8 formats): the 128 x 128 tile (best or within 5 % of
+    // the best of every tile at 4096..12288 x 4096..12288, M = 128..8192, with K slices
+    // where the tiles are few; the 256 x 128 tile was up to 42 % slower), else 64 x 128.
+    static const int tiles[][2] = {{128, 128}, {64, 128}};
     for (auto& t : tiles) {
       const int64_t wgs = ((p.m + t[0] - 1) / t[0]) * ((p.n + t[1] - 1) / t[1]);
       tlhip_kernel_config_t c = tiled_cfg(t[0], t[1], 64, 2, 2);
-      if (!(wgs >= cus || t[0] == 64) || !gemm_config_applicable(p, c, nullptr)) continue;
+      if (!gemm_config_applicable(p, c, nullptr)) continue;
       if (wgs < cus && t[1] == 128 && t[0] <= 128) {
         // far fewer tiles than CUs: K slices across workgroups, the cheapest by the model
         // (this kernel walks 4096 of K in 52 us), every slice at least 512 of K
         int best = 1;
         for (int ks = 2; ks <= 8; ks *= 2)
-          if (wgs * ks <= 2 * cus && (p.k / 64) % ks == 0 && p.k / ks >= 512 &&
+          if (wgs * ks <= cus && (p.k / 64) % ks == 0 && p.k / ks >= 512 &&
               direct_round_us(p, ks, 52.0) < direct_round_us(p, best, 52.0))
             best = ks;
         tlhip_kernel_config_t split = c;
