@@ -83,6 +83,58 @@ def test_direct_weight_operand_gemm_every_tile_ragged_shapes(be, g, m, n, k, bm,
     assert rel_l2(got, other) <= 2e-6
 
 
+INT8_DIRECT_TILES = [(128, 128, 2, 2), (128, 256, 2, 4), (256, 128, 2, 4), (256, 256, 2, 4)]
+
+
+@pytest.mark.parametrize("bm,bn,wm,wn", INT8_DIRECT_TILES)
+@pytest.mark.parametrize("g,m,n,k,ks", [(64, 300, 333, 256, 0), (128, 300, 333, 384, 0), (64, 520, 777, 1152, 0),
+                                        (256, 64, 256, 512, 2), (64, 130, 300, 2048, 4), (1024, 200, 136, 1024, 8)])
+@pytest.mark.parametrize("ydt", ["f16", "f32"])
+def test_direct_weight_operand_gemm_on_int8_groups(be, g, m, n, k, ks, bm, bn, wm, wn, ydt):
+    """The same kernel on int8 weights in groups of 64 or more (one f16 scale per group,
+    the format's 1/127 folded into alpha): ragged M and N, odd and even numbers of 128-k
+    steps, one group per step up to one per row, K slices across workgroups, bias +
+    activation fused.  Against the oracle, and as close to it as the LDS-staged kernel."""
+    rng = np.random.default_rng(bm + bn + g + k + ks)
+    packed, scales, deq = make_weight("int8-grouped", n, k, g, rng)
+    x = make_x(m, k, "f16", rng, std=0.5)
+    bias = f16_round(rng.standard_normal(n) * 0.1)
+    cfg = L.KernelConfig.of(3, bm, bn, 128, wm, wn, ks)
+    before = T.getQuantGemmDispatchCount()
+    got = run(be, "int8-grouped", packed, scales, n, k, g, x, ydt, bias=bias, act="silu", config=cfg)
+    assert T.getQuantGemmDispatchCount() == before + 1
+    want = O.linear(x.astype(np.float32), deq, bias.astype(np.float32), "silu", threads=8)
+    assert got.shape == (m, n) and got.dtype == (np.float16 if ydt == "f16" else np.float32)
+    assert rel_l2(got, want) <= REL_L2_TOL, rel_l2(got, want)
+    if ydt == "f32":
+        # the staged kernel rounds q * (scale / 127) to f16, this one q * scale (and divides the
+        # sums by 127): different roundings of a weight, the same distance from the oracle
+        other = run(be, "int8-grouped", packed, scales, n, k, g, x, ydt, bias=bias, act="silu", config=tiled(128, 128))
+        assert abs(rel_l2(other, want) - rel_l2(got, want)) <= 5e-5, (rel_l2(other, want), rel_l2(got, want))
+    again = run(be, "int8-grouped", packed, scales, n, k, g, x, ydt, bias=bias, act="silu", config=cfg)
+    assert np.array_equal(again, got)
+
+
+@pytest.mark.parametrize("m,n", [(1500, 2500), (600, 6500), (1100, 3600)])
+@pytest.mark.parametrize("cfg", [(3, 128, 128, 128, 2, 2), (2, 128, 128, 64, 2, 2), (2, 64, 128, 64, 2, 2)])
+def test_tile_counts_whose_edge_blocks_would_crowd_some_xcds(be, m, n, cfg):
+    """12 x 20, 5 x 51 and 9 x 29 tiles of 128 x 128: with the largest blocks of tiles per
+    XCD the partial blocks on the edges would all fall to the same XCDs, so the workgroup ->
+    tile map takes smaller blocks there.  Every tile must still be computed exactly once."""
+    rng = np.random.default_rng(m + n)
+    k = 256
+    packed, scales, deq = make_weight("int4-grouped", n, k, 32, rng)
+    x = make_x(m, k, "f16", rng, std=0.5)
+    got = run(be, "int4-grouped", packed, scales, n, k, 32, x, "f32", config=L.KernelConfig.of(*cfg))
+    want = O.linear(x.astype(np.float32), deq, threads=8)
+    assert got.shape == (m, n)
+    # per 128 x 128 tile, so that one missing or doubled tile cannot hide in the whole
+    for r0 in range(0, m, 128):
+        for c0 in range(0, n, 128):
+            e = rel_l2(got[r0:r0 + 128, c0:c0 + 128], want[r0:r0 + 128, c0:c0 + 128])
+            assert e <= REL_L2_TOL, (r0, c0, e)
+
+
 def test_direct_gemm_rejects_what_it_does_not_cover(be):
     rng = np.random.default_rng(3)
     x = be.ops.tensorFromArray(make_x(32, 192, "f16", rng), [32, 192], "f16")
@@ -95,6 +147,15 @@ def test_direct_gemm_rejects_what_it_does_not_cover(be):
     x8 = be.ops.tensorFromArray(make_x(32, 256, "f16", rng), [32, 256], "f16")
     with pytest.raises(L.TlhipError, match="int4-grouped"):
         be.linear(x8, w8, config=L.KernelConfig.of(3, 256, 256, 128, 2, 4))
+    # int8 in groups: groups of 64 or more, and only the tiles built for it
+    p32, s32, _ = make_weight("int8-grouped", 64, 256, 32, rng)
+    w32 = be.createQuantizedWeight(p32, s32, 64, 256, T.resolveWeightFormat("int8-32", "f32"))
+    with pytest.raises(L.TlhipError, match="multiple of 64"):
+        be.linear(x8, w32, config=L.KernelConfig.of(3, 128, 128, 128, 2, 2))
+    p64, s64, _ = make_weight("int8-grouped", 64, 256, 64, rng)
+    w64 = be.createQuantizedWeight(p64, s64, 64, 256, T.resolveWeightFormat("int8-64", "f32"))
+    with pytest.raises(L.TlhipError, match="multiple of 64"):
+        be.linear(x8, w64, config=L.KernelConfig.of(3, 128, 256, 128, 1, 4))
 
 
 @pytest.mark.parametrize("m,n,k,route", [(17, 128, 64, "gemm"), (64, 64, 128, "gemm"), (100, 512, 1024, "gemm"),
@@ -205,10 +266,10 @@ def test_gemm_rejects_f32_activations_as_an_explicit_configuration(be):
 ])
 @pytest.mark.parametrize("ydt", ["f16", "f32"])
 def test_direct_gemm_with_k_slices_across_workgroups(be, m, n, k, cfg, ydt):
-    """p5 workgroups share a tile, each walking a slice of K; the last to arrive adds the
-    partial tiles in slice order and runs the epilogue.  Against the oracle, bit-stable
-    from launch to launch (the order of the sum does not depend on who arrives last), and
-    as close to the oracle as the unsplit kernel."""
+    """p5 workgroups share a tile, each walking a slice of K and leaving its partial sums
+    in a plane of the workspace; a second launch adds the planes in slice order and runs
+    the epilogue.  Against the oracle, bit-stable from launch to launch, and as close to
+    the oracle as the unsplit kernel."""
     rng = np.random.default_rng(m + n + k)
     packed, scales, deq = make_weight("int4-grouped", n, k, 32, rng)
     x = make_x(m, k, "f16", rng, std=0.5)

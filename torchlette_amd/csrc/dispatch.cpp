@@ -199,6 +199,23 @@ double direct_round_us(const Problem& p, int ks, double walk_4096_us = 42.0) {
   return walk + 6.0 + 0.6 * (double)ks * (double)p.m * (double)p.n * 4.0 / 1e6;
 }
 
+// Time of a launch of a tiled configuration by the same model, in microseconds: a round of
+// the direct kernel's 128 x 128 tiles walks 4096 of K in 42 us, of the staged kernel's in
+// 52 us, of its 64 x 128 tiles in 42 us; x = tiles x slices / CUs up to 1 is one round,
+// beyond that 0.45 + 0.78 x rounds (workgroups that share a CU slow each other down: the
+// staged kernel measured 1.38 / 1.56 / 1.83 / 2.73 / 5.2 rounds at x = 1.125 / 1.5 / 2 / 3 / 6).
+double tiled_launch_us(const Problem& p, const tlhip_kernel_config_t& c) {
+  const int cus = device_cu_count() > 0 ? device_cu_count() : 256;
+  const int ks = c.p5 > 1 ? c.p5 : 1;
+  const int64_t tiles = ((p.m + c.p0 - 1) / c.p0) * ((p.n + c.p1 - 1) / c.p1);
+  const double walk = c.variant == VARIANT_TILED_DIRECT ? 42.0 : (c.p0 <= 64 ? 42.0 : 52.0);
+  const double fill = (double)(tiles * ks) / (double)cus;
+  const double rounds = fill <= 1.0 ? 1.0 : 0.45 + 0.78 * fill;
+  const double area = (double)c.p0 * c.p1 / (c.p0 <= 64 ? 64.0 * 128.0 : 128.0 * 128.0);  // larger tiles walk longer
+  const double sum_us = ks > 1 ? 6.0 + 0.6 * (double)ks * (double)p.m * (double)p.n * 4.0 / 1e6 : 0.0;
+  return rounds * walk * area * (double)p.k / 4096.0 / ks + sum_us;
+}
+
 // K slices across workgroups for a launch of 128 x 128 tiles of the direct GEMM: of 1, 2,
 // 4, 8 the cheapest by direct_round_us that keeps tiles x slices within the CUs (beyond,
 // the slices of a tile queue behind each other), divides the 128-k steps and leaves every
@@ -223,7 +240,7 @@ tlhip_kernel_config_t default_config(const Problem& p) {
     // (two workgroups share a CU) from 160 such tiles on, never more than 7 % behind the
     // best there; below that 128 x 128, where the 256-row tiles measured 1.4-1.5 times
     // slower (a launch of few tiles takes the time one workgroup needs to walk K).
-    {
+    if (p.format == TLHIP_FMT_INT4_GROUPED) {
       const int64_t t256 = ((p.m + 255) / 256) * ((p.n + 255) / 256);
       const int64_t t128x256 = ((p.m + 127) / 128) * ((p.n + 255) / 256);
       tlhip_kernel_config_t c = t256 >= 2 * cus ? direct_cfg(256, 256, 2, 4)
@@ -240,27 +257,58 @@ tlhip_kernel_config_t default_config(const Problem& p) {
       }
       if (gemm_direct_config_applicable(p, c, nullptr)) return c;
     }
-    // The LDS-staged kernel (the int8 formats): the 128 x 128 tile (best or within 5 % of
-    // the best of every tile at 4096..12288 x 4096..12288, M = 128..8192, with K slices
-    // where the tiles are few; the 256 x 128 tile was up to 42 % slower), else 64 x 128.
-    static const int tiles[][2] = {{128, 128}, {64, 128}};
-    for (auto& t : tiles) {
-      const int64_t wgs = ((p.m + t[0] - 1) / t[0]) * ((p.n + t[1] - 1) / t[1]);
-      tlhip_kernel_config_t c = tiled_cfg(t[0], t[1], 64, 2, 2);
-      if (!gemm_config_applicable(p, c, nullptr)) continue;
-      if (wgs < cus && t[1] == 128 && t[0] <= 128) {
-        // far fewer tiles than CUs: K slices across workgroups, the cheapest by the model
-        // (this kernel walks 4096 of K in 52 us), every slice at least 512 of K
-        int best = 1;
-        for (int ks = 2; ks <= 8; ks *= 2)
-          if (wgs * ks <= cus && (p.k / 64) % ks == 0 && p.k / ks >= 512 &&
-              direct_round_us(p, ks, 52.0) < direct_round_us(p, best, 52.0))
-            best = ks;
-        tlhip_kernel_config_t split = c;
-        split.p5 = best;
-        if (best > 1 && gemm_config_applicable(p, split, nullptr)) return split;
+    // int8 in groups of 64 or more: the same kernel once its 256-row tiles fill the chip
+    // (2048..28672 x 2048..14336, M = 32..8192, groups of 64 and 128: the 256 x 256 tile
+    // was the best of every tile of both kernels from 144 tiles on, 4-23 % ahead of the
+    // staged kernel; 256 x 128 from 192 tiles on, 3-9 % ahead); with fewer tiles the
+    // staged kernel below is ahead by 3-40 %.
+    // Not where the rows fill less than 70 % of their 256-row tiles (128 rows on 28672
+    // columns: 78 us against 52 us).
+    if (p.format == TLHIP_FMT_INT8_GROUPED && p.m * 10 >= ((p.m + 255) / 256) * 256 * 7) {
+      const int64_t t256 = ((p.m + 255) / 256) * ((p.n + 255) / 256);
+      const int64_t t256x128 = ((p.m + 255) / 256) * ((p.n + 127) / 128);
+      if (t256 * 16 >= (int64_t)cus * 9) {
+        const tlhip_kernel_config_t c = direct_cfg(256, 256, 2, 4);
+        if (gemm_direct_config_applicable(p, c, nullptr)) return c;
+      } else if (t256x128 * 4 >= (int64_t)cus * 3) {
+        const tlhip_kernel_config_t c = direct_cfg(256, 128, 2, 4);
+        if (gemm_direct_config_applicable(p, c, nullptr)) return c;
       }
-      return c;
+    }
+    // The LDS-staged kernel (the int8 formats): the 128 x 128 or the 64 x 128 tile, with K
+    // slices across workgroups where the tiles are few, whichever the model of a launch
+    // prices lowest: tiles x slices / CUs rounds (at least one) of the time a workgroup
+    // needs to walk its slice (52 us per 4096 of K for the 128-row tile, 42 us for the
+    // 64-row tile) plus the second launch that adds the slices.  Within 10 % of the best
+    // of every tile and slice count at 2048..28672 x 2048..14336, M = 32..2048; the 256 x
+    // 128 tile was up to 42 % slower.
+    {
+      tlhip_kernel_config_t best_c{};
+      double best_us = 0.0;
+      bool have = false;
+      for (const int bm : {128, 64}) {
+        const int64_t wgs = ((p.m + bm - 1) / bm) * ((p.n + 127) / 128);
+        const tlhip_kernel_config_t c = tiled_cfg(bm, 128, 64, 2, 2);
+        if (!gemm_config_applicable(p, c, nullptr)) continue;
+        for (int ks = 1; ks <= 8; ks *= 2) {
+          tlhip_kernel_config_t split = c;
+          if (ks > 1) {
+            // every slice at least 512 of K, and at most two workgroups to a CU (the model
+            // prices the crowding: 160 rows at 5120 x 5120 took 36 us in 4 slices, 320
+            // workgroups, against 42 us in 2)
+            if (wgs * ks > 2 * cus || (p.k / 64) % ks != 0 || p.k / ks < 512) continue;
+            split.p5 = ks;
+            if (!gemm_config_applicable(p, split, nullptr)) continue;
+          }
+          const double us = tiled_launch_us(p, split);
+          if (!have || us < best_us) {
+            best_c = split;
+            best_us = us;
+            have = true;
+          }
+        }
+      }
+      if (have) return best_c;
     }
   }
   // three or four rows of int4 weights with K up to 8192, from 8 MB of weights on: the
@@ -650,7 +698,8 @@ Route plan_route(const Problem& p, const tlhip_kernel_config_t& c) {
     const int64_t passes = (p.m + 15) / 16;
     const int64_t tiles = ((p.m + 127) / 128) * ((p.n + 127) / 128);
     const double rounds = tiles <= 512 ? 1.0 : (double)tiles / 512.0;
-    const double tiled_us = direct_round_us(p, c.p5 > 1 ? c.p5 : 1, c.variant == VARIANT_TILED_DIRECT ? 42.0 : 52.0) * rounds;
+    const double tiled_us =
+        direct_round_us(p, c.p5 > 1 ? c.p5 : 1, c.variant == VARIANT_TILED_DIRECT ? 42.0 : (c.p0 <= 64 ? 42.0 : 52.0)) * rounds;
     // Up to 64 rows per launch of the decode kernel: 1.2-1.6 times a 16-row pass for two
     // tiles of rows, 2.3-3.2 times for four (the activations a workgroup stages grow with
     // the rows, and their K slices are combined across workgroups).  More rows go 64 at a

@@ -18,14 +18,11 @@ struct TileMap {
   int nsb;                 // super-blocks in all
 };
 
-inline TileMap make_tile_map(int tiles_m, int tiles_n, int* grid) {
+// The map with super-blocks of 2^s_shift tiles: as tall as the tiles along M allow (up to 8).
+inline TileMap tile_map_with(int tiles_m, int tiles_n, int s_shift) {
   TileMap t;
   t.tiles_m = tiles_m;
   t.tiles_n = tiles_n;
-  const long total = (long)tiles_m * tiles_n;
-  // as large as 32 tiles, but at least 16 super-blocks so that every XCD gets work
-  int s_shift = 5;
-  while (s_shift > 0 && (total >> s_shift) < 16) --s_shift;
   int gm_shift = 0;
   while (gm_shift < 3 && gm_shift < s_shift && (2 << gm_shift) <= tiles_m) ++gm_shift;
   t.gm_shift = gm_shift;
@@ -34,6 +31,59 @@ inline TileMap make_tile_map(int tiles_m, int tiles_n, int* grid) {
   t.sbm = (tiles_m + gm - 1) / gm;
   const int sbn = (tiles_n + gn - 1) / gn;
   t.nsb = t.sbm * sbn;
+  return t;
+}
+
+// Tiles of the busiest XCD under a map (super-block sb goes to XCD sb % 8; the ones on the
+// edges hold fewer tiles than 2^s_shift).
+inline int64_t busiest_xcd_tiles(const TileMap& t) {
+  int64_t load[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  const int gm = 1 << t.gm_shift, gn = 1 << t.gn_shift;
+  for (int sb = 0; sb < t.nsb; ++sb) {
+    const int sb_n = sb / t.sbm, sb_m = sb - sb_n * t.sbm;
+    const int rows = t.tiles_m - sb_m * gm < gm ? t.tiles_m - sb_m * gm : gm;
+    const int cols = t.tiles_n - sb_n * gn < gn ? t.tiles_n - sb_n * gn : gn;
+    load[sb & 7] += (int64_t)rows * cols;
+  }
+  int64_t most = 0;
+  for (int64_t l : load) most = l > most ? l : most;
+  return most;
+}
+
+// Super-blocks as large as 32 tiles, but at least 16 of them so that every XCD gets work,
+// and no larger than keeps the XCDs level: partial super-blocks on the edges can all fall
+// to the same XCDs (12 x 20 tiles in super-blocks of 8 x 1: the even XCDs got 40 tiles
+// each, the odd ones 20, and a launch that fits the chip in one round took two), so the
+// super-blocks shrink until the busiest XCD needs no more rounds of its 32 CUs than the
+// whole launch needs of the chip, or, in a launch of more than two rounds, holds at most
+// 5 % more than its share.
+inline TileMap make_tile_map(int tiles_m, int tiles_n, int* grid) {
+  static thread_local struct {
+    int tiles_m = 0, tiles_n = 0, s_shift = 0;
+  } last;  // the loop below costs a few microseconds for thousands of tiles
+  const int64_t total = (int64_t)tiles_m * tiles_n;
+  int s_shift = 5;
+  if (last.tiles_m == tiles_m && last.tiles_n == tiles_n) {
+    s_shift = last.s_shift;
+  } else {
+    while (s_shift > 0 && (total >> s_shift) < 16) --s_shift;
+    const int64_t chip_rounds = (total + 255) / 256;
+    int best_shift = s_shift;
+    int64_t best_load = -1;
+    for (int s = s_shift; s >= 0; --s) {
+      const int64_t load = busiest_xcd_tiles(tile_map_with(tiles_m, tiles_n, s));
+      if (best_load < 0 || load < best_load) {
+        best_load = load;
+        best_shift = s;
+      }
+      if ((load + 31) / 32 <= chip_rounds || (chip_rounds > 2 && load * 8 * 20 <= total * 21)) break;
+    }
+    s_shift = best_shift;
+    last.tiles_m = tiles_m;
+    last.tiles_n = tiles_n;
+    last.s_shift = s_shift;
+  }
+  const TileMap t = tile_map_with(tiles_m, tiles_n, s_shift);
   *grid = ((t.nsb + 7) / 8) * 8 << s_shift;
   return t;
 }

@@ -66,13 +66,20 @@ struct DirectArgs {
 // WM x WN waves, each owning TM x TN MFMA tiles of 32 x 32.  G32: one scale per
 // 16-byte chunk (group size 32), the two scales of a lane's step come as one
 // 4-byte load.
-template <int WM, int WN, int TM, int TN, bool G32>
+// I8: int8 weights with one f16 scale per group of 64 or more (the reference's own
+// format).  A 128-k step of a row is 128 bytes = 8 chunks; a lane of the B operand reads
+// the 4 chunks of its k half and turns two words (8 weights) into an MFMA operand, in
+// natural k order (k = 64*lk + 8*kk for MFMA group kk: the same activation units as for
+// int4, without the int4 order inside a unit); the 1/127 of the format rides on alpha.
+template <int WM, int WN, int TM, int TN, bool G32, bool I8 = false>
 __global__ __launch_bounds__(WM * WN * 64, (TM * TN >= 16 ? 1 : 2)) void gemm_direct_kernel(const DirectArgs a) {
+  static_assert(!(G32 && I8), "int8 groups are 64 weights or more");
   constexpr int THREADS = WM * WN * 64;
   constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
+  constexpr int CPR = I8 ? 8 : 4;             // 16-byte chunks of a weight row per step
   constexpr int X_LOADS = BM * 16 / THREADS;  // 16-byte units of the X tile per thread per step
-  constexpr int W_LOADS = BN * 4 / THREADS;   // 16-byte chunks of the W tile per thread per step
-  static_assert(BM * 16 % THREADS == 0 && BN * 4 % THREADS == 0, "tiles must divide over the threads");
+  constexpr int W_LOADS = BN * CPR / THREADS; // 16-byte chunks of the W tile per thread per step
+  static_assert(BM * 16 % THREADS == 0 && BN * CPR % THREADS == 0, "tiles must divide over the threads");
   constexpr int X_UNITS = BM * HROW_UNITS;  // half a step of the X tile
   // The 256x128 tile of eight 128x32 waves issues its MFMA groups at raised priority,
   // so that the wave it shares a SIMD with (same workgroup, same barriers, the same
@@ -110,8 +117,8 @@ __global__ __launch_bounds__(WM * WN * 64, (TM * TN >= 16 ? 1 : 2)) void gemm_di
 #pragma unroll
     for (int i = 0; i < W_LOADS; ++i) {
       const int q = tid + i * THREADS;
-      const int row = min(n0 + (q >> 2), a.n - 1);
-      wr[i] = *(const u32x4*)(a.packed + (size_t)row * a.w_row_bytes + (size_t)st * 64 + (q & 3) * 16);
+      const int row = min(n0 + q / CPR, a.n - 1);
+      wr[i] = *(const u32x4*)(a.packed + (size_t)row * a.w_row_bytes + (size_t)st * (CPR * 16) + (q % CPR) * 16);
     }
   };
   auto store_w = [&]() {
@@ -119,8 +126,9 @@ __global__ __launch_bounds__(WM * WN * 64, (TM * TN >= 16 ? 1 : 2)) void gemm_di
 #pragma unroll
     for (int i = 0; i < W_LOADS; ++i) {
       const int q = tid + i * THREADS;
-      const int r = q >> 2;
-      ws[r * 4 + ((q & 3) ^ ((r >> 2) & 3))] = wr[i];
+      const int r = q / CPR;
+      if constexpr (I8) ws[r * 8 + ((q & 7) ^ (r & 7))] = wr[i];
+      else ws[r * 4 + ((q & 3) ^ ((r >> 2) & 3))] = wr[i];
     }
   };
   // The lane's scales: raw bits, two stages (this step, next step).
@@ -169,7 +177,7 @@ __global__ __launch_bounds__(WM * WN * 64, (TM * TN >= 16 ? 1 : 2)) void gemm_di
     for (int i = 0; i < XH; ++i) {
       const int u = tid + (part * XH + i) * THREADS;
       const int r = u >> 3, c = u & 7;
-      xs[r * HROW_UNITS + (c ^ ((r >> 1) & 7))] = permute_x_for_int4(xr[i]);
+      xs[r * HROW_UNITS + (c ^ ((r >> 1) & 7))] = I8 ? xr[i] : permute_x_for_int4(xr[i]);
     }
   };
 
@@ -188,13 +196,18 @@ __global__ __launch_bounds__(WM * WN * 64, (TM * TN >= 16 ? 1 : 2)) void gemm_di
   // kk+1 as soon as its last MFMA of group kk has been issued: an MFMA occupies
   // the matrix pipe for 8 passes and the wave can issue 7 other instructions
   // meanwhile, so the dequantisation and the LDS reads hide under the MFMAs.
-  u32x4 bw[TN][2];  // the lane's packed chunks c = 0, 1 of the step
+  // the lane's packed chunks of the step.  int4: c = 0, 1.  int8: four chunks through two
+  // register slots: chunks 0 and 1 at the top of the step, chunk 2 into slot 0 once MFMA
+  // group 1 has been dequantised (the last user of chunk 0), chunk 3 into slot 1 behind
+  // group 3; all four are read before the mid-step barrier that frees the W buffer.
+  u32x4 bw[TN][2];
   auto read_w = [&](int c) {
     const u32x4* ws = lds_w;
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
       const int r = (wn * TN + j) * 32 + lrow;
-      bw[j][c] = ws[r * 4 + ((lk * 2 + c) ^ ((r >> 2) & 3))];
+      if constexpr (I8) bw[j][c & 1] = ws[r * 8 + ((lk * 4 + c) ^ (r & 7))];
+      else bw[j][c] = ws[r * 4 + ((lk * 2 + c) ^ ((r >> 2) & 3))];
     }
   };
   auto dequant = [&](const Scales& sc, int kk, half8_t (&bf)[TN]) {
@@ -204,10 +217,17 @@ __global__ __launch_bounds__(WM * WN * 64, (TM * TN >= 16 ? 1 : 2)) void gemm_di
       const uint32_t bits = G32 ? (c ? (sc.s[j][0] >> 16) : (sc.s[j][0] & 0xffffu)) : sc.s[j][c];
       const _Float16 sh = __builtin_bit_cast(_Float16, (uint16_t)bits);
       const half2_t s2 = {sh, sh};
-      const u32x4 chunk = bw[j][c];
-      const uint32_t word = w == 0 ? chunk.x : (w == 1 ? chunk.y : (w == 2 ? chunk.z : chunk.w));
       half2_t h[4];
-      unpack_int4_word(word, h);
+      if constexpr (I8) {
+        // chunk kk / 2 of the lane's four, its words 0, 1 (kk even) or 2, 3 (kk odd)
+        const u32x4 chunk8 = bw[j][(kk >> 1) & 1];
+        unpack_int8_word((kk & 1) ? chunk8.z : chunk8.x, h);
+        unpack_int8_word((kk & 1) ? chunk8.w : chunk8.y, h + 2);
+      } else {
+        const u32x4 chunk = bw[j][c];
+        const uint32_t word = w == 0 ? chunk.x : (w == 1 ? chunk.y : (w == 2 ? chunk.z : chunk.w));
+        unpack_int4_word(word, h);
+      }
       half8_t v;
       const half2_t h0 = h[0] * s2, h1 = h[1] * s2, h2 = h[2] * s2, h3 = h[3] * s2;
       v[0] = h0[0]; v[1] = h0[1]; v[2] = h1[0]; v[3] = h1[1];
@@ -275,13 +295,17 @@ __global__ __launch_bounds__(WM * WN * 64, (TM * TN >= 16 ? 1 : 2)) void gemm_di
       dequant(sc, 0, bfA);
     }
     __builtin_amdgcn_sched_barrier(0);
-    dequant(sc, 1, bfB); group(bfA, 1);
+    dequant(sc, 1, bfB);
+    if constexpr (I8) read_w(2);
+    group(bfA, 1);
     dequant(sc, 2, bfA); group(bfB, 2);
     __builtin_amdgcn_sched_barrier(0);
     store_x(1, 0);
     load_x(s, 1, 1);
     __builtin_amdgcn_sched_barrier(0);
-    dequant(sc, 3, bfB); group(bfA, 3);
+    dequant(sc, 3, bfB);
+    if constexpr (I8) read_w(3);
+    group(bfA, 3);
     if constexpr (!CARRY) {
       // group 3 re-reads nothing: the second half of X is whole only behind the barrier
       dequant(sc, 4, bfA); group(bfB, -1);
@@ -421,12 +445,21 @@ int launch_direct_reduce(int ks, unsigned grid, const float* planes, const OutAr
   return TLHIP_OK;
 }
 
+// The tiles built for int8 weights (the others would only lengthen the build).
 template <int WM, int WN, int TM, int TN>
-int launch_direct_tile(const DirectArgs& a, bool g32, hipStream_t stream) {
+constexpr bool kInt8Tile = (WM == 2 && WN == 2 && TM == 2 && TN == 2) || (WM == 2 && WN == 4 && TM == 2 && TN == 2) ||
+                           (WM == 2 && WN == 4 && TM == 4 && TN == 1) || (WM == 2 && WN == 4 && TM == 4 && TN == 2);
+
+template <int WM, int WN, int TM, int TN>
+int launch_direct_tile(const DirectArgs& a, bool g32, bool int8, hipStream_t stream) {
   constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
   const void* fn = g32 ? (const void*)gemm_direct_kernel<WM, WN, TM, TN, true>
                        : (const void*)gemm_direct_kernel<WM, WN, TM, TN, false>;
-  size_t lds_bytes = (size_t)(2 * BM * HROW_UNITS + BN * 4) * 16;
+  if (int8) {
+    if constexpr (kInt8Tile<WM, WN, TM, TN>) fn = (const void*)gemm_direct_kernel<WM, WN, TM, TN, false, true>;
+    else return set_error(TLHIP_ERR_INVALID, "gemm_direct: this tile is not built for int8 weights");
+  }
+  size_t lds_bytes = (size_t)(2 * BM * HROW_UNITS + BN * (int8 ? 8 : 4)) * 16;
   const size_t patch_bytes = (size_t)WM * WN * 32 * (TN * 32 + 4) * sizeof(float);
   if (lds_bytes < patch_bytes) lds_bytes = patch_bytes;
   DirectArgs b = a;
@@ -468,7 +501,8 @@ int launch_k_slice_reduce(int ks, const float* planes, const OutArgs& o, hipStre
 bool gemm_direct_config_applicable(const Problem& p, const tlhip_kernel_config_t& c, const char** why) {
   static const char* reasons[] = {
       "not the tiled_direct variant",
-      "weights must be int4-grouped",
+      "weights must be int4-grouped, or int8-grouped with a group size that is a multiple of 64 on one of the tiles "
+      "128x128 2x2, 128x256 2x4, 256x128 2x4, 256x256 2x4",
       "activations must be f16",
       "K must be a multiple of 128",
       "group size must be a multiple of 32",
@@ -481,7 +515,13 @@ bool gemm_direct_config_applicable(const Problem& p, const tlhip_kernel_config_t
     return false;
   };
   if (c.variant != VARIANT_TILED_DIRECT) return fail(0);
-  if (p.format != TLHIP_FMT_INT4_GROUPED) return fail(1);
+  const bool int8 = p.format == TLHIP_FMT_INT8_GROUPED;
+  if (p.format != TLHIP_FMT_INT4_GROUPED && !int8) return fail(1);
+  if (int8) {
+    const bool tile_ok = (c.p0 == 128 && c.p1 == 128 && c.p3 == 2 && c.p4 == 2) || (c.p0 == 128 && c.p1 == 256 && c.p3 == 2 && c.p4 == 4) ||
+                         (c.p0 == 256 && c.p1 == 128 && c.p3 == 2 && c.p4 == 4) || (c.p0 == 256 && c.p1 == 256 && c.p3 == 2 && c.p4 == 4);
+    if (p.group_size % 64 != 0 || !tile_ok) return fail(1);
+  }
   if (p.x_dtype != TLHIP_F16) return fail(2);
   if (p.k % DK != 0 || p.k == 0) return fail(3);
   if (p.group_size % 32 != 0) return fail(4);
@@ -510,7 +550,7 @@ int launch_gemm_direct(const Problem& p, const tlhip_kernel_config_t& c, hipStre
   a.m = (int)p.m;
   a.n = (int)p.n;
   a.k = (int)p.k;
-  a.w_row_bytes = (int)(p.k / 2);
+  a.w_row_bytes = (int)(p.format == TLHIP_FMT_INT8_GROUPED ? p.k : p.k / 2);
   a.cpg_shift = __builtin_ctz((unsigned)(p.group_size / 32));
   a.groups_per_row = (int)(p.k / p.group_size);
   a.ksteps = (int)(p.k / DK);
@@ -528,16 +568,18 @@ int launch_gemm_direct(const Problem& p, const tlhip_kernel_config_t& c, hipStre
   a.out.n = (int)p.n;
   a.out.alpha = p.alpha;
   a.out.epi = p.epi;
-  const bool g32 = p.group_size == 32;
+  const bool int8 = p.format == TLHIP_FMT_INT8_GROUPED;
+  const bool g32 = !int8 && p.group_size == 32;
+  if (int8) a.out.alpha = p.alpha * (1.0f / 127.0f);  // the format's 1/127 (quantize.ts: q = round(w / absmax * 127))
   int rc;
-  if (c.p0 == 256 && c.p1 == 256 && c.p4 == 2) rc = launch_direct_tile<2, 2, 4, 4>(a, g32, stream);
-  else if (c.p0 == 256 && c.p1 == 256) rc = launch_direct_tile<2, 4, 4, 2>(a, g32, stream);
-  else if (c.p0 == 256 && c.p1 == 128 && c.p3 == 2) rc = launch_direct_tile<2, 4, 4, 1>(a, g32, stream);
-  else if (c.p0 == 128 && c.p1 == 256 && c.p3 == 1) rc = launch_direct_tile<1, 4, 4, 2>(a, g32, stream);
-  else if (c.p0 == 128 && c.p1 == 256) rc = launch_direct_tile<2, 4, 2, 2>(a, g32, stream);
-  else if (c.p0 == 128 && c.p1 == 128) rc = launch_direct_tile<2, 2, 2, 2>(a, g32, stream);
-  else if (c.p0 == 128 && c.p1 == 192) rc = launch_direct_tile<2, 2, 2, 3>(a, g32, stream);
-  else rc = launch_direct_tile<4, 2, 2, 2>(a, g32, stream);
+  if (c.p0 == 256 && c.p1 == 256 && c.p4 == 2) rc = launch_direct_tile<2, 2, 4, 4>(a, g32, int8, stream);
+  else if (c.p0 == 256 && c.p1 == 256) rc = launch_direct_tile<2, 4, 4, 2>(a, g32, int8, stream);
+  else if (c.p0 == 256 && c.p1 == 128 && c.p3 == 2) rc = launch_direct_tile<2, 4, 4, 1>(a, g32, int8, stream);
+  else if (c.p0 == 128 && c.p1 == 256 && c.p3 == 1) rc = launch_direct_tile<1, 4, 4, 2>(a, g32, int8, stream);
+  else if (c.p0 == 128 && c.p1 == 256) rc = launch_direct_tile<2, 4, 2, 2>(a, g32, int8, stream);
+  else if (c.p0 == 128 && c.p1 == 128) rc = launch_direct_tile<2, 2, 2, 2>(a, g32, int8, stream);
+  else if (c.p0 == 128 && c.p1 == 192) rc = launch_direct_tile<2, 2, 2, 3>(a, g32, int8, stream);
+  else rc = launch_direct_tile<4, 2, 2, 2>(a, g32, int8, stream);
   if (rc) return rc;
   TLHIP_CHECK_HIP(hipGetLastError());
   if (a.ksplit > 1) {
@@ -555,14 +597,21 @@ int prepare_gemm_direct_kernels() {
   a.m = a.n = 1;
   a.ksplit = 1;
   for (bool g32 : {true, false}) {
-    int rc = launch_direct_tile<2, 2, 4, 4>(a, g32, nullptr);
-    if (!rc) rc = launch_direct_tile<2, 4, 4, 2>(a, g32, nullptr);
-    if (!rc) rc = launch_direct_tile<2, 4, 4, 1>(a, g32, nullptr);
-    if (!rc) rc = launch_direct_tile<1, 4, 4, 2>(a, g32, nullptr);
-    if (!rc) rc = launch_direct_tile<2, 4, 2, 2>(a, g32, nullptr);
-    if (!rc) rc = launch_direct_tile<2, 2, 2, 2>(a, g32, nullptr);
-    if (!rc) rc = launch_direct_tile<2, 2, 2, 3>(a, g32, nullptr);
-    if (!rc) rc = launch_direct_tile<4, 2, 2, 2>(a, g32, nullptr);
+    int rc = launch_direct_tile<2, 2, 4, 4>(a, g32, false, nullptr);
+    if (!rc) rc = launch_direct_tile<2, 4, 4, 2>(a, g32, false, nullptr);
+    if (!rc) rc = launch_direct_tile<2, 4, 4, 1>(a, g32, false, nullptr);
+    if (!rc) rc = launch_direct_tile<1, 4, 4, 2>(a, g32, false, nullptr);
+    if (!rc) rc = launch_direct_tile<2, 4, 2, 2>(a, g32, false, nullptr);
+    if (!rc) rc = launch_direct_tile<2, 2, 2, 2>(a, g32, false, nullptr);
+    if (!rc) rc = launch_direct_tile<2, 2, 2, 3>(a, g32, false, nullptr);
+    if (!rc) rc = launch_direct_tile<4, 2, 2, 2>(a, g32, false, nullptr);
+    if (rc) return rc;
+  }
+  {
+    int rc = launch_direct_tile<2, 2, 2, 2>(a, false, true, nullptr);
+    if (!rc) rc = launch_direct_tile<2, 4, 2, 2>(a, false, true, nullptr);
+    if (!rc) rc = launch_direct_tile<2, 4, 4, 1>(a, false, true, nullptr);
+    if (!rc) rc = launch_direct_tile<2, 4, 4, 2>(a, false, true, nullptr);
     if (rc) return rc;
   }
   return TLHIP_OK;
