@@ -915,6 +915,21 @@ def main() -> int:
                           "config": list(be.selectedConfig(w, "f32", m, "f32").as_tuple())})
             out.destroy()
         details["prefill_gemm_int4_4096x12288_f32_activations"] = pre32
+        # the same GEMM on the reference's own format (int8, one f16 absmax per 64 weights),
+        # heuristic defaults (no entry of the tuning file covers it)
+        w8_pool, _ = B.weight_pool("int8-grouped", n, k, 64, "f16", pool_bytes=110e6)
+        pre8 = []
+        for m in (512, 2048):
+            x, _ = B.activations(m, k, std=0.5)
+            out = be._alloc([m, n], "f16")
+            us = B.median_time(B.make_call(w8_pool, x, m, out, epilogue=be.makeEpilogue(bias, "silu")), 20)
+            fl = 2.0 * m * n * k
+            pre8.append({"m": m, "epilogue": "bias+silu", "us": round(us, 1), "tflops": round(fl / us / 1e6, 1),
+                         "frac_of_f16_mfma_peak": round(fl / us / 1e6 / F16_MFMA_PEAK_TFLOPS, 4),
+                         "config": list(be.selectedConfig(w8_pool[0], "f16", m, "f16").as_tuple())})
+            out.destroy()
+            x.destroy()
+        details["prefill_gemm_int8_g64_4096x12288"] = pre8
 
         # config 1: int8-row 1024 x 1024, f32 activations and output, M = 1
         pool, _ = B.weight_pool("int8-row", 1024, 1024, 0, "f32", pool_bytes=64e6)
