@@ -356,9 +356,9 @@ int tlhip_topk(const float* logits, int64_t offset, int64_t length, int k, float
  * 3 = "tiled_direct" (prefill MFMA GEMM whose weights stay packed up to the
  * operand registers; fields as "tiled" with tile K 128; int4-grouped on the tiles
  * (M, N, waves M, waves N) 256x256 2x4, 256x128 2x4, 128x256 2x4, 256x128 4x2,
- * 128x128 2x2, 256x256 2x2, 128x256 1x4, 128x192 2x2; int8-grouped with a group
- * size that is a multiple of 64 on 256x256 2x4, 256x128 2x4, 128x256 2x4, 128x128
- * 2x2; p5 = 2, 4, 8 or 16: that many workgroups share a tile, each walking a
+ * 128x128 2x2, 256x256 2x2, 128x256 1x4, 128x192 2x2; int8-row, and int8-grouped
+ * with a group size that is a multiple of 64, on 256x256 2x4, 256x128 2x4, 128x256
+ * 2x4, 128x128 2x2; p5 = 2, 4, 8 or 16: that many workgroups share a tile, each walking a
  * slice of K, and a second launch adds their partial sums in slice order - for
  * launches of far fewer tiles than the chip has CUs),
  * 4 = "gemv_mfma_xreg" (skinny MFMA for int4 g32 with the activations held in

@@ -135,6 +135,50 @@ def test_tile_counts_whose_edge_blocks_would_crowd_some_xcds(be, m, n, cfg):
             assert e <= REL_L2_TOL, (r0, c0, e)
 
 
+@pytest.mark.parametrize("bm,bn,wm,wn", INT8_DIRECT_TILES)
+@pytest.mark.parametrize("m,n,k,ks", [(300, 333, 256, 0), (520, 777, 1152, 0), (64, 256, 512, 2), (130, 300, 2048, 8)])
+@pytest.mark.parametrize("ydt", ["f16", "f32"])
+def test_direct_weight_operand_gemm_on_int8_rows(be, m, n, k, ks, bm, bn, wm, wn, ydt):
+    """int8 weights with one f32 scale per row: the MFMA operand is the bare integer (exact
+    in f16) and the row's scale multiplies the sums in the epilogue (or in the launch that
+    adds the K slices), so the f32 output differs from the oracle only by the order of the
+    f32 sums: far closer than the 1e-3 bar, which the f16 output's rounding sets."""
+    rng = np.random.default_rng(bm + bn + k + ks)
+    packed, scales, deq = make_weight("int8-row", n, k, 0, rng)
+    x = make_x(m, k, "f16", rng, std=0.5)
+    bias = f16_round(rng.standard_normal(n) * 0.1)
+    cfg = L.KernelConfig.of(3, bm, bn, 128, wm, wn, ks)
+    before = T.getQuantGemmDispatchCount()
+    got = run(be, "int8-row", packed, scales, n, k, 0, x, ydt, bias=bias, act="gelu", config=cfg)
+    assert T.getQuantGemmDispatchCount() == before + 1
+    want = O.linear(x.astype(np.float32), deq, bias.astype(np.float32), "gelu", threads=8)
+    assert got.shape == (m, n)
+    assert rel_l2(got, want) <= (REL_L2_TOL if ydt == "f16" else 5e-6), rel_l2(got, want)
+    again = run(be, "int8-row", packed, scales, n, k, 0, x, ydt, bias=bias, act="gelu", config=cfg)
+    assert np.array_equal(again, got)
+
+
+def test_direct_gemm_int8_rows_extreme_scales(be):
+    """Row scales from denormal to 3e38, zero and negative zero among them: the scale never
+    enters f16 (the staged kernel's dequantised weight would overflow or vanish there)."""
+    rng = np.random.default_rng(11)
+    m, n, k = 70, 256, 256
+    packed, scales, _ = make_weight("int8-row", n, k, 0, rng)
+    scales = scales.copy()
+    scales[:8] = np.array([0.0, -0.0, 1e-40, 3e-39, 1e-30, 1e30, 3e38, 6.1e-5], np.float32)
+    q = packed.view(np.int8).reshape(n, k).astype(np.float64)
+    x = make_x(m, k, "f16", rng, std=0.01)
+    got = run(be, "int8-row", packed, scales, n, k, 0, x, "f32", config=L.KernelConfig.of(3, 128, 128, 128, 2, 2))
+    with np.errstate(over="ignore", under="ignore"):
+        want = ((x.astype(np.float64) @ q.T) * scales.astype(np.float64)[None, :]).astype(np.float32)
+    assert np.all(np.isfinite(got[:, 8:]))
+    for c in range(n):
+        if np.any(np.isinf(want[:, c])) or scales[c] < 1e-37:
+            continue  # past f32 on either side: the order of the multiplications decides
+        assert rel_l2(got[:, c], want[:, c]) <= 1e-5, (c, scales[c])
+    assert np.all(got[:, 0] == 0) and np.all(got[:, 1] == 0)
+
+
 def test_direct_gemm_rejects_what_it_does_not_cover(be):
     rng = np.random.default_rng(3)
     x = be.ops.tensorFromArray(make_x(32, 192, "f16", rng), [32, 192], "f16")
@@ -146,7 +190,7 @@ def test_direct_gemm_rejects_what_it_does_not_cover(be):
     w8 = be.createQuantizedWeight(packed8, scales8, 64, 256, T.resolveWeightFormat("int8-row", "f32"))
     x8 = be.ops.tensorFromArray(make_x(32, 256, "f16", rng), [32, 256], "f16")
     with pytest.raises(L.TlhipError, match="int4-grouped"):
-        be.linear(x8, w8, config=L.KernelConfig.of(3, 256, 256, 128, 2, 4))
+        be.linear(x8, w8, config=L.KernelConfig.of(3, 256, 256, 128, 2, 2))   # a tile not built for int8
     # int8 in groups: groups of 64 or more, and only the tiles built for it
     p32, s32, _ = make_weight("int8-grouped", 64, 256, 32, rng)
     w32 = be.createQuantizedWeight(p32, s32, 64, 256, T.resolveWeightFormat("int8-32", "f32"))

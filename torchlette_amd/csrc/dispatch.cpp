@@ -257,20 +257,20 @@ tlhip_kernel_config_t default_config(const Problem& p) {
       }
       if (gemm_direct_config_applicable(p, c, nullptr)) return c;
     }
-    // int8 in groups of 64 or more: the same kernel once its 256-row tiles fill the chip
-    // (2048..28672 x 2048..14336, M = 32..8192, groups of 64 and 128: the 256 x 256 tile
-    // was the best of every tile of both kernels from 144 tiles on, 4-23 % ahead of the
-    // staged kernel; 256 x 128 from 192 tiles on, 3-9 % ahead); with fewer tiles the
-    // staged kernel below is ahead by 3-40 %.
-    // Not where the rows fill less than 70 % of their 256-row tiles (128 rows on 28672
-    // columns: 78 us against 52 us).
-    if (p.format == TLHIP_FMT_INT8_GROUPED && p.m * 10 >= ((p.m + 255) / 256) * 256 * 7) {
+    // int8 per row, or in groups of 64 or more: the same kernel once its 256-row tiles fill
+    // the chip (2048..28672 x 2048..14336, M = 32..8192, per row and groups of 64 and 128:
+    // the 256 x 256 tile was the best of every tile of both kernels from 144 tiles on, 4-27 %
+    // ahead of the staged kernel; 256 x 128 from 160 tiles on, 3-15 % ahead); with fewer
+    // tiles the staged kernel below is ahead by 3-40 %.  Not where the rows fill less than
+    // 58 % of their 256-row tiles (128 rows on 28672 columns: 78 us against 52 us).
+    if ((p.format == TLHIP_FMT_INT8_GROUPED || p.format == TLHIP_FMT_INT8_ROW) &&
+        p.m * 100 >= ((p.m + 255) / 256) * 256 * 58) {
       const int64_t t256 = ((p.m + 255) / 256) * ((p.n + 255) / 256);
       const int64_t t256x128 = ((p.m + 255) / 256) * ((p.n + 127) / 128);
       if (t256 * 16 >= (int64_t)cus * 9) {
         const tlhip_kernel_config_t c = direct_cfg(256, 256, 2, 4);
         if (gemm_direct_config_applicable(p, c, nullptr)) return c;
-      } else if (t256x128 * 4 >= (int64_t)cus * 3) {
+      } else if (t256x128 * 8 >= (int64_t)cus * 5) {
         const tlhip_kernel_config_t c = direct_cfg(256, 128, 2, 4);
         if (gemm_direct_config_applicable(p, c, nullptr)) return c;
       }

@@ -1,6 +1,8 @@
 // Pieces shared by the two prefill GEMM kernels: the workgroup -> tile map and
 // the per-wave epilogue.
 #pragma once
+#include <algorithm>
+
 #include "device_utils.h"
 
 namespace tlhip {
@@ -10,7 +12,7 @@ namespace tlhip {
 // the CUs of an XCD) consecutive workgroups of an XCD takes one "super-block" of
 // 2^gm_shift x 2^gn_shift tiles, so the tiles that run together on an XCD share
 // their X row blocks and W column blocks through that XCD's L2: the L2 fill per
-// K step is (GM * BM + GN * BN) rows instead of (32 * BM + BN).
+// K step is GM row blocks of X and GN column blocks of W instead of 32 and 1.
 struct TileMap {
   int tiles_m, tiles_n;
   int gm_shift, gn_shift;  // super-block = 2^gm_shift x 2^gn_shift tiles
@@ -18,13 +20,34 @@ struct TileMap {
   int nsb;                 // super-blocks in all
 };
 
-// The map with super-blocks of 2^s_shift tiles: as tall as the tiles along M allow (up to 8).
-inline TileMap tile_map_with(int tiles_m, int tiles_n, int s_shift) {
+// Bytes per k that one more row of tiles (an X row block) and one more column of tiles (a
+// W column block) add to what an XCD's L2 has to fetch for a super-block.
+struct TileCost {
+  int x_bytes;  // tile M x 2 (f16 activations)
+  int w_bytes;  // tile N x bytes per packed weight
+};
+
+// The map with super-blocks of 2^s_shift tiles, of the shape (rows of tiles up to 8, a power
+// of two) that fetches the fewest bytes per k for the tiles it really holds; ties go to the
+// taller block.  4 x 8 tiles for the large problems of every format; a matrix of few column
+// tiles gets blocks as wide as it is (1024 columns on 256 x 128 tiles at M = 6000: 8 x 1
+// blocks read X once per column tile, 180 us; 2 x 4 blocks 127 us).
+inline TileMap tile_map_with(int tiles_m, int tiles_n, int s_shift, TileCost cost) {
   TileMap t;
   t.tiles_m = tiles_m;
   t.tiles_n = tiles_n;
   int gm_shift = 0;
-  while (gm_shift < 3 && gm_shift < s_shift && (2 << gm_shift) <= tiles_m) ++gm_shift;
+  int64_t best = -1;
+  for (int g = 0; g <= 3 && g <= s_shift; ++g) {
+    const int64_t rows = std::min<int64_t>(1 << g, tiles_m), cols = std::min<int64_t>(1 << (s_shift - g), tiles_n);
+    const int64_t bytes = rows * cost.x_bytes + cols * cost.w_bytes;
+    // per tile really held: a block clipped by the matrix must not look cheap
+    const int64_t per_tile = bytes * 1024 / (rows * cols);
+    if (best < 0 || per_tile <= best) {
+      best = per_tile;
+      gm_shift = g;
+    }
+  }
   t.gm_shift = gm_shift;
   t.gn_shift = s_shift - gm_shift;
   const int gm = 1 << t.gm_shift, gn = 1 << t.gn_shift;
@@ -57,13 +80,13 @@ inline int64_t busiest_xcd_tiles(const TileMap& t) {
 // super-blocks shrink until the busiest XCD needs no more rounds of its 32 CUs than the
 // whole launch needs of the chip, or, in a launch of more than two rounds, holds at most
 // 5 % more than its share.
-inline TileMap make_tile_map(int tiles_m, int tiles_n, int* grid) {
+inline TileMap make_tile_map(int tiles_m, int tiles_n, TileCost cost, int* grid) {
   static thread_local struct {
-    int tiles_m = 0, tiles_n = 0, s_shift = 0;
+    int tiles_m = 0, tiles_n = 0, x_bytes = 0, w_bytes = 0, s_shift = 0;
   } last;  // the loop below costs a few microseconds for thousands of tiles
   const int64_t total = (int64_t)tiles_m * tiles_n;
   int s_shift = 5;
-  if (last.tiles_m == tiles_m && last.tiles_n == tiles_n) {
+  if (last.tiles_m == tiles_m && last.tiles_n == tiles_n && last.x_bytes == cost.x_bytes && last.w_bytes == cost.w_bytes) {
     s_shift = last.s_shift;
   } else {
     while (s_shift > 0 && (total >> s_shift) < 16) --s_shift;
@@ -71,7 +94,7 @@ inline TileMap make_tile_map(int tiles_m, int tiles_n, int* grid) {
     int best_shift = s_shift;
     int64_t best_load = -1;
     for (int s = s_shift; s >= 0; --s) {
-      const int64_t load = busiest_xcd_tiles(tile_map_with(tiles_m, tiles_n, s));
+      const int64_t load = busiest_xcd_tiles(tile_map_with(tiles_m, tiles_n, s, cost));
       if (best_load < 0 || load < best_load) {
         best_load = load;
         best_shift = s;
@@ -81,9 +104,11 @@ inline TileMap make_tile_map(int tiles_m, int tiles_n, int* grid) {
     s_shift = best_shift;
     last.tiles_m = tiles_m;
     last.tiles_n = tiles_n;
+    last.x_bytes = cost.x_bytes;
+    last.w_bytes = cost.w_bytes;
     last.s_shift = s_shift;
   }
-  const TileMap t = tile_map_with(tiles_m, tiles_n, s_shift);
+  const TileMap t = tile_map_with(tiles_m, tiles_n, s_shift, cost);
   *grid = ((t.nsb + 7) / 8) * 8 << s_shift;
   return t;
 }
@@ -107,6 +132,7 @@ struct OutArgs {
   int m, n;
   float alpha;
   DevEpilogue epi;
+  const float* col_scale;  // null, or one f32 factor per output column, applied with alpha (int8-row: the row scales of W)
 };
 
 // Defined in gemm_direct.hip: the second launch of a K-sliced tiled GEMM.
@@ -125,7 +151,9 @@ int launch_k_slice_reduce(int ks, const float* planes, const OutArgs& o, hipStre
 // `o` would do the same, but a copy of the kernel arguments whose op arrays are indexed
 // at run time lands in scratch memory.)
 // PLANE = false: instances that never take K slices compile without the choice.
-template <int TN, bool PLANE = false>
+// COLSCALE: o.col_scale holds a factor per column (never null then); a K slice leaves it,
+// like alpha, to the launch that adds the planes.
+template <int TN, bool PLANE = false, bool COLSCALE = false>
 __device__ __forceinline__ void wave_epilogue(float* patch, const float16_t (&acc)[TN], int lane, int row0,
                                               int col0, const OutArgs& o, float* plane = nullptr) {
   const bool bare = PLANE && plane != nullptr;  // uniform
@@ -156,6 +184,15 @@ __device__ __forceinline__ void wave_epilogue(float* patch, const float16_t (&ac
   const int un_at = has_bias ? 1 : 0;
   const bool simple = n_ops <= un_at + 1 && (n_ops == un_at || o.epi.kind[un_at] == TLHIP_EPI_UNARY);
   const int unary = (simple && n_ops > un_at) ? o.epi.unary[un_at] : TLHIP_UNARY_NONE;
+  float cscale[COLSCALE ? 8 : 1];  // alpha x the lane's column factors
+  if constexpr (COLSCALE) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) cscale[e] = bare ? 1.f : o.alpha * o.col_scale[min(col + e, o.n - 1)];
+  }
+  auto scale_of = [&](int e) -> float {
+    if constexpr (COLSCALE) return cscale[e];
+    else return out_alpha();
+  };
   float bias[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) {
@@ -175,10 +212,10 @@ __device__ __forceinline__ void wave_epilogue(float* patch, const float16_t (&ac
     if (row < o.m && lane_used && p * RPP + rr0 < 32) {
       if (simple) {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) v[e] = apply_unary(unary, v[e] * out_alpha() + bias[e]);
+        for (int e = 0; e < 8; ++e) v[e] = apply_unary(unary, v[e] * scale_of(e) + bias[e]);
       } else {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) v[e] = apply_epilogue(o.epi, v[e] * out_alpha(), min(col + e, o.n - 1));
+        for (int e = 0; e < 8; ++e) v[e] = apply_epilogue(o.epi, v[e] * scale_of(e), min(col + e, o.n - 1));
       }
       if (vec) {
         const int64_t idx = (int64_t)row * o.n + col;

@@ -71,9 +71,13 @@ struct DirectArgs {
 // the 4 chunks of its k half and turns two words (8 weights) into an MFMA operand, in
 // natural k order (k = 64*lk + 8*kk for MFMA group kk: the same activation units as for
 // int4, without the int4 order inside a unit); the 1/127 of the format rides on alpha.
-template <int WM, int WN, int TM, int TN, bool G32, bool I8 = false>
+// ROW (with I8): int8 weights with one f32 scale per row.  The operand is the bare integer
+// (exact in f16, no multiplication, no scale loads in the loop) and the row's scale
+// multiplies the sums in the epilogue, as a factor per output column.
+template <int WM, int WN, int TM, int TN, bool G32, bool I8 = false, bool ROW = false>
 __global__ __launch_bounds__(WM * WN * 64, (TM * TN >= 16 ? 1 : 2)) void gemm_direct_kernel(const DirectArgs a) {
   static_assert(!(G32 && I8), "int8 groups are 64 weights or more");
+  static_assert(!ROW || I8, "per-row scales are an int8 format");
   constexpr int THREADS = WM * WN * 64;
   constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
   constexpr int CPR = I8 ? 8 : 4;             // 16-byte chunks of a weight row per step
@@ -142,6 +146,7 @@ __global__ __launch_bounds__(WM * WN * 64, (TM * TN >= 16 ? 1 : 2)) void gemm_di
     uint32_t s[TN][2];  // G32: s[j][0] holds both scales; else one 16-bit scale each
   };
   auto load_s = [&](int step, Scales& sc) {
+    if constexpr (ROW) return;
     const int st = step0 + min(step, nsteps - 1);
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
@@ -214,7 +219,7 @@ __global__ __launch_bounds__(WM * WN * 64, (TM * TN >= 16 ? 1 : 2)) void gemm_di
     const int c = kk >> 2, w = kk & 3;
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
-      const uint32_t bits = G32 ? (c ? (sc.s[j][0] >> 16) : (sc.s[j][0] & 0xffffu)) : sc.s[j][c];
+      const uint32_t bits = ROW ? 0x3c00u : (G32 ? (c ? (sc.s[j][0] >> 16) : (sc.s[j][0] & 0xffffu)) : sc.s[j][c]);
       const _Float16 sh = __builtin_bit_cast(_Float16, (uint16_t)bits);
       const half2_t s2 = {sh, sh};
       half2_t h[4];
@@ -229,7 +234,8 @@ __global__ __launch_bounds__(WM * WN * 64, (TM * TN >= 16 ? 1 : 2)) void gemm_di
         unpack_int4_word(word, h);
       }
       half8_t v;
-      const half2_t h0 = h[0] * s2, h1 = h[1] * s2, h2 = h[2] * s2, h3 = h[3] * s2;
+      const half2_t h0 = ROW ? h[0] : h[0] * s2, h1 = ROW ? h[1] : h[1] * s2, h2 = ROW ? h[2] : h[2] * s2,
+                    h3 = ROW ? h[3] : h[3] * s2;
       v[0] = h0[0]; v[1] = h0[1]; v[2] = h1[0]; v[3] = h1[1];
       v[4] = h2[0]; v[5] = h2[1]; v[6] = h3[0]; v[7] = h3[1];
       bf[j] = v;
@@ -357,14 +363,14 @@ __global__ __launch_bounds__(WM * WN * 64, (TM * TN >= 16 ? 1 : 2)) void gemm_di
   float* const plane = a.ksplit > 1 ? a.workspace + (size_t)slice * a.m * a.n : nullptr;
 #pragma unroll
   for (int i = 0; i < TM; ++i)
-    wave_epilogue<TN, true>(patch, acc[i], lane, m0 + (wm * TM + i) * 32, n0 + wn * TN * 32, a.out, plane);
+    wave_epilogue<TN, true, ROW>(patch, acc[i], lane, m0 + (wm * TM + i) * 32, n0 + wn * TN * 32, a.out, plane);
 }
 
 // v[e] = ops(alpha * v[e]) for the W consecutive columns from `col` on.
 template <int W>
 __device__ __forceinline__ void apply_epilogue_scaled(const OutArgs& o, float (&v)[W], int64_t col) {
 #pragma unroll
-  for (int e = 0; e < W; ++e) v[e] *= o.alpha;
+  for (int e = 0; e < W; ++e) v[e] *= o.col_scale ? o.alpha * o.col_scale[col + e] : o.alpha;
 #pragma unroll
   for (int i = 0; i < TLHIP_MAX_EPILOGUE_OPS; ++i) {
     if (i < o.epi.n_ops) {
@@ -456,7 +462,9 @@ int launch_direct_tile(const DirectArgs& a, bool g32, bool int8, hipStream_t str
   const void* fn = g32 ? (const void*)gemm_direct_kernel<WM, WN, TM, TN, true>
                        : (const void*)gemm_direct_kernel<WM, WN, TM, TN, false>;
   if (int8) {
-    if constexpr (kInt8Tile<WM, WN, TM, TN>) fn = (const void*)gemm_direct_kernel<WM, WN, TM, TN, false, true>;
+    if constexpr (kInt8Tile<WM, WN, TM, TN>)
+      fn = a.out.col_scale ? (const void*)gemm_direct_kernel<WM, WN, TM, TN, false, true, true>
+                           : (const void*)gemm_direct_kernel<WM, WN, TM, TN, false, true>;
     else return set_error(TLHIP_ERR_INVALID, "gemm_direct: this tile is not built for int8 weights");
   }
   size_t lds_bytes = (size_t)(2 * BM * HROW_UNITS + BN * (int8 ? 8 : 4)) * 16;
@@ -464,7 +472,7 @@ int launch_direct_tile(const DirectArgs& a, bool g32, bool int8, hipStream_t str
   if (lds_bytes < patch_bytes) lds_bytes = patch_bytes;
   DirectArgs b = a;
   int grid = 0;
-  b.map = make_tile_map((a.m + BM - 1) / BM, (a.n + BN - 1) / BN, &grid);
+  b.map = make_tile_map((a.m + BM - 1) / BM, (a.n + BN - 1) / BN, TileCost{BM * 2, int8 ? BN : BN / 2}, &grid);
   void* args[] = {(void*)&b};
   return launch_kernel(fn, dim3(grid * (a.ksplit > 1 ? a.ksplit : 1)), dim3(WM * WN * 64), args, lds_bytes, stream);
 }
@@ -501,7 +509,7 @@ int launch_k_slice_reduce(int ks, const float* planes, const OutArgs& o, hipStre
 bool gemm_direct_config_applicable(const Problem& p, const tlhip_kernel_config_t& c, const char** why) {
   static const char* reasons[] = {
       "not the tiled_direct variant",
-      "weights must be int4-grouped, or int8-grouped with a group size that is a multiple of 64 on one of the tiles "
+      "weights must be int4-grouped, or int8-row or int8-grouped with a group size that is a multiple of 64 on one of the tiles "
       "128x128 2x2, 128x256 2x4, 256x128 2x4, 256x256 2x4",
       "activations must be f16",
       "K must be a multiple of 128",
@@ -515,16 +523,17 @@ bool gemm_direct_config_applicable(const Problem& p, const tlhip_kernel_config_t
     return false;
   };
   if (c.variant != VARIANT_TILED_DIRECT) return fail(0);
-  const bool int8 = p.format == TLHIP_FMT_INT8_GROUPED;
+  const bool row = p.format == TLHIP_FMT_INT8_ROW;
+  const bool int8 = p.format == TLHIP_FMT_INT8_GROUPED || row;
   if (p.format != TLHIP_FMT_INT4_GROUPED && !int8) return fail(1);
   if (int8) {
     const bool tile_ok = (c.p0 == 128 && c.p1 == 128 && c.p3 == 2 && c.p4 == 2) || (c.p0 == 128 && c.p1 == 256 && c.p3 == 2 && c.p4 == 4) ||
                          (c.p0 == 256 && c.p1 == 128 && c.p3 == 2 && c.p4 == 4) || (c.p0 == 256 && c.p1 == 256 && c.p3 == 2 && c.p4 == 4);
-    if (p.group_size % 64 != 0 || !tile_ok) return fail(1);
+    if ((!row && p.group_size % 64 != 0) || !tile_ok) return fail(1);
   }
   if (p.x_dtype != TLHIP_F16) return fail(2);
   if (p.k % DK != 0 || p.k == 0) return fail(3);
-  if (p.group_size % 32 != 0) return fail(4);
+  if (!row && p.group_size % 32 != 0) return fail(4);
   if (c.p2 != DK) return fail(6);
   for (const auto& t : kDirectTiles)
     if (t.bm == c.p0 && t.bn == c.p1 && t.wm == c.p3 && t.wn == c.p4) {
@@ -550,9 +559,10 @@ int launch_gemm_direct(const Problem& p, const tlhip_kernel_config_t& c, hipStre
   a.m = (int)p.m;
   a.n = (int)p.n;
   a.k = (int)p.k;
-  a.w_row_bytes = (int)(p.format == TLHIP_FMT_INT8_GROUPED ? p.k : p.k / 2);
-  a.cpg_shift = __builtin_ctz((unsigned)(p.group_size / 32));
-  a.groups_per_row = (int)(p.k / p.group_size);
+  const bool row = p.format == TLHIP_FMT_INT8_ROW;
+  a.w_row_bytes = (int)(p.format == TLHIP_FMT_INT4_GROUPED ? p.k / 2 : p.k);
+  a.cpg_shift = row ? 0 : __builtin_ctz((unsigned)(p.group_size / 32));
+  a.groups_per_row = row ? 0 : (int)(p.k / p.group_size);
   a.ksteps = (int)(p.k / DK);
   a.ksplit = c.p5 < 1 ? 1 : c.p5;
   a.workspace = nullptr;
@@ -568,9 +578,11 @@ int launch_gemm_direct(const Problem& p, const tlhip_kernel_config_t& c, hipStre
   a.out.n = (int)p.n;
   a.out.alpha = p.alpha;
   a.out.epi = p.epi;
-  const bool int8 = p.format == TLHIP_FMT_INT8_GROUPED;
+  a.out.col_scale = row ? (const float*)p.scales : nullptr;  // int8-row: w = q * scale[n], applied to the sums
+  const bool int8 = p.format == TLHIP_FMT_INT8_GROUPED || row;
   const bool g32 = !int8 && p.group_size == 32;
-  if (int8) a.out.alpha = p.alpha * (1.0f / 127.0f);  // the format's 1/127 (quantize.ts: q = round(w / absmax * 127))
+  // the grouped format's 1/127 (quantize.ts: q = round(w / absmax * 127))
+  if (p.format == TLHIP_FMT_INT8_GROUPED) a.out.alpha = p.alpha * (1.0f / 127.0f);
   int rc;
   if (c.p0 == 256 && c.p1 == 256 && c.p4 == 2) rc = launch_direct_tile<2, 2, 4, 4>(a, g32, int8, stream);
   else if (c.p0 == 256 && c.p1 == 256) rc = launch_direct_tile<2, 4, 4, 2>(a, g32, int8, stream);
@@ -607,7 +619,9 @@ int prepare_gemm_direct_kernels() {
     if (!rc) rc = launch_direct_tile<4, 2, 2, 2>(a, g32, false, nullptr);
     if (rc) return rc;
   }
-  {
+  static const float one = 1.f;
+  for (const float* cs : {(const float*)nullptr, &one}) {  // int8 in groups, int8 per row
+    a.out.col_scale = cs;
     int rc = launch_direct_tile<2, 2, 2, 2>(a, false, true, nullptr);
     if (!rc) rc = launch_direct_tile<2, 4, 2, 2>(a, false, true, nullptr);
     if (!rc) rc = launch_direct_tile<2, 4, 4, 1>(a, false, true, nullptr);

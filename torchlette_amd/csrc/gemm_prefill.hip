@@ -263,7 +263,7 @@ int launch_tile(const GemmArgs& a, hipStream_t stream) {
   if (lds_bytes < patch_bytes) lds_bytes = patch_bytes;
   GemmArgs b = a;
   int grid = 0;
-  b.map = make_tile_map((a.m + BM - 1) / BM, (a.n + BN - 1) / BN, &grid);
+  b.map = make_tile_map((a.m + BM - 1) / BM, (a.n + BN - 1) / BN, TileCost{BM * 2, FMT == TLHIP_FMT_INT4_GROUPED ? BN / 2 : BN}, &grid);
   void* args[] = {(void*)&b};
   return launch_kernel(fn, dim3(grid * (a.ksplit > 1 ? a.ksplit : 1)), dim3(256), args, lds_bytes, stream);
 }
@@ -346,6 +346,7 @@ int launch_gemm(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t st
   a.out.n = (int)p.n;
   a.out.alpha = p.alpha;
   a.out.epi = p.epi;
+  a.out.col_scale = nullptr;
   int rc;
   switch (p.format) {
     case TLHIP_FMT_INT4_GROUPED: rc = launch_fmt<TLHIP_FMT_INT4_GROUPED>(c.p0, c.p1, a, stream); break;
