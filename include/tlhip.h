@@ -97,10 +97,12 @@ typedef struct {
  *           same bytes);  INT8_ROW: f32 [N] */
 /* Limits.  packed and scales are 16-byte aligned.  K <= 2^24, N <= 2^30.  The decode
  * kernels keep activation rows in LDS: K <= 57344 for f16 activations, K <= 28672 for f32
- * activations (longer rows: TLHIP_ERR_INVALID).  The prefill GEMMs (m > 16) round each
- * dequantised weight q*s once to f16 before the matrix cores, so |q*s| must stay inside
- * f16's normal range: scales between 6.2e-5 / 1 and 65504 / 8 (int4) or 65504 / 127
- * (int8); the decode kernels (m <= 16) apply the scale in f32 and have no such limit. */
+ * activations (longer rows: TLHIP_ERR_INVALID).  For the grouped formats the prefill
+ * GEMMs (m > 16) round each dequantised weight q*s once to f16 before the matrix cores,
+ * so |q*s| must stay inside f16's normal range: scales between 6.2e-5 / 1 and 65504 / 8
+ * (int4) or 65504 / 127 (int8-grouped).  The decode kernels (m <= 16) apply the scale in
+ * f32 and have no such limit, and neither has INT8_ROW at any m (its prefill GEMMs
+ * multiply the bare integers and apply the row's scale to the f32 sums). */
 typedef struct {
   int32_t format;     /* tlhip_format_t */
   int32_t group_size; /* G along K; ignored for INT8_ROW */

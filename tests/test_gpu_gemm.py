@@ -158,9 +158,12 @@ def test_direct_weight_operand_gemm_on_int8_rows(be, m, n, k, ks, bm, bn, wm, wn
     assert np.array_equal(again, got)
 
 
-def test_direct_gemm_int8_rows_extreme_scales(be):
-    """Row scales from denormal to 3e38, zero and negative zero among them: the scale never
-    enters f16 (the staged kernel's dequantised weight would overflow or vanish there)."""
+@pytest.mark.parametrize("cfg", [(3, 128, 128, 128, 2, 2), (3, 256, 128, 128, 2, 4, 2), (2, 128, 128, 64, 2, 2),
+                                 (2, 64, 128, 64, 2, 2, 2), None])
+def test_int8_rows_extreme_scales_above_16_rows(be, cfg):
+    """Row scales from denormal to 3e38, zero and negative zero among them: both prefill
+    kernels feed the bare integers to the matrix cores and apply the row's scale to the f32
+    sums, so the scale never enters f16 (a dequantised f16 weight would overflow or vanish)."""
     rng = np.random.default_rng(11)
     m, n, k = 70, 256, 256
     packed, scales, _ = make_weight("int8-row", n, k, 0, rng)
@@ -168,7 +171,7 @@ def test_direct_gemm_int8_rows_extreme_scales(be):
     scales[:8] = np.array([0.0, -0.0, 1e-40, 3e-39, 1e-30, 1e30, 3e38, 6.1e-5], np.float32)
     q = packed.view(np.int8).reshape(n, k).astype(np.float64)
     x = make_x(m, k, "f16", rng, std=0.01)
-    got = run(be, "int8-row", packed, scales, n, k, 0, x, "f32", config=L.KernelConfig.of(3, 128, 128, 128, 2, 2))
+    got = run(be, "int8-row", packed, scales, n, k, 0, x, "f32", config=L.KernelConfig.of(*cfg) if cfg else None)
     with np.errstate(over="ignore", under="ignore"):
         want = ((x.astype(np.float64) @ q.T) * scales.astype(np.float64)[None, :]).astype(np.float32)
     assert np.all(np.isfinite(got[:, 8:]))

@@ -81,8 +81,8 @@ template <int FMT>
 struct WChunkInt8 {
   static constexpr int WEIGHTS = 16;
   static constexpr int UNITS = 2;
-  // The scale multiplies in f32 here (int8-row scales are f32 and (q/127)*s is
-  // not an f16 product); one rounding to f16 per weight.
+  // The scale multiplies in f32 here ((q/127)*s is not an f16 product); one rounding to
+  // f16 per weight.
   __device__ static __forceinline__ void dequant(const u32x4& w, float scale, u32x4 (&out)[UNITS]) {
     const uint32_t words[4] = {w.x, w.y, w.z, w.w};
     uint32_t packed[8];
@@ -103,8 +103,27 @@ struct WChunkInt8 {
 };
 template <>
 struct WChunk<TLHIP_FMT_INT8_GROUPED> : WChunkInt8<TLHIP_FMT_INT8_GROUPED> {};
+// int8 with one f32 scale per row: the bare integers go to the matrix cores (exact in f16)
+// and the row's scale multiplies the f32 sums in the epilogue, as a factor per output
+// column: no rounding of q * s to f16, and no scale that f16 could not hold.
 template <>
-struct WChunk<TLHIP_FMT_INT8_ROW> : WChunkInt8<TLHIP_FMT_INT8_ROW> {};
+struct WChunk<TLHIP_FMT_INT8_ROW> {
+  static constexpr int WEIGHTS = 16;
+  static constexpr int UNITS = 2;
+  __device__ static __forceinline__ void dequant(const u32x4& w, float, u32x4 (&out)[UNITS]) {
+    const uint32_t words[4] = {w.x, w.y, w.z, w.w};
+    uint32_t packed[8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      half2_t h[2];
+      unpack_int8_word(words[i], h);
+      packed[2 * i] = __builtin_bit_cast(uint32_t, h[0]);
+      packed[2 * i + 1] = __builtin_bit_cast(uint32_t, h[1]);
+    }
+    out[0] = (u32x4){packed[0], packed[1], packed[2], packed[3]};
+    out[1] = (u32x4){packed[4], packed[5], packed[6], packed[7]};
+  }
+};
 
 // SPLIT: the instances that take K slices across workgroups (the 64- and 128-row tiles
 // with 128 columns, the ones a launch of few tiles uses); the others compile as without.
@@ -162,7 +181,7 @@ __global__ __launch_bounds__(256) void gemm_prefill_kernel(const GemmArgs a) {
       const int chunk = k0 / WC::WEIGHTS + c;
       ws[i] = *(const u32x4*)(a.packed + (size_t)row * a.w_row_bytes + (size_t)chunk * 16);
       if (GROUPED) ss[i] = ((const uint16_t*)a.scales)[(size_t)row * a.groups_per_row + (chunk >> a.cpg_shift)];
-      else ss[i] = ((const uint32_t*)a.scales)[row];
+      else ss[i] = 0;  // int8-row: the row scales are the epilogue's
     }
   };
 
@@ -247,7 +266,8 @@ __global__ __launch_bounds__(256) void gemm_prefill_kernel(const GemmArgs a) {
   float* const plane = SPLIT ? a.workspace + (size_t)slice * a.m * a.n : nullptr;
 #pragma unroll
   for (int i = 0; i < TM; ++i)
-    wave_epilogue<TN, SPLIT>(patch, acc[i], lane, m0 + wm * (BM / 2) + i * 32, n0 + wn * (BN / 2), a.out, plane);
+    wave_epilogue<TN, SPLIT, FMT == TLHIP_FMT_INT8_ROW>(patch, acc[i], lane, m0 + wm * (BM / 2) + i * 32, n0 + wn * (BN / 2),
+                                                         a.out, plane);
 }
 
 template <int FMT, int BM, int BN>
@@ -346,7 +366,7 @@ int launch_gemm(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t st
   a.out.n = (int)p.n;
   a.out.alpha = p.alpha;
   a.out.epi = p.epi;
-  a.out.col_scale = nullptr;
+  a.out.col_scale = p.format == TLHIP_FMT_INT8_ROW ? (const float*)p.scales : nullptr;
   int rc;
   switch (p.format) {
     case TLHIP_FMT_INT4_GROUPED: rc = launch_fmt<TLHIP_FMT_INT4_GROUPED>(c.p0, c.p1, a, stream); break;
