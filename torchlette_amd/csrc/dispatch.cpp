@@ -199,21 +199,20 @@ double direct_round_us(const Problem& p, int ks, double walk_4096_us = 42.0) {
   return walk + 6.0 + 0.6 * (double)ks * (double)p.m * (double)p.n * 4.0 / 1e6;
 }
 
-// Time of a launch of a tiled configuration by the same model, in microseconds: a round of
-// the direct kernel's 128 x 128 tiles walks 4096 of K in 42 us, of the staged kernel's in
-// 52 us, of its 64 x 128 tiles in 42 us; x = tiles x slices / CUs up to 1 is one round,
-// beyond that 0.45 + 0.78 x rounds (workgroups that share a CU slow each other down: the
-// staged kernel measured 1.38 / 1.56 / 1.83 / 2.73 / 5.2 rounds at x = 1.125 / 1.5 / 2 / 3 / 6).
-double tiled_launch_us(const Problem& p, const tlhip_kernel_config_t& c) {
+// Time of a launch of the staged GEMM's 128 x 128 or 64 x 128 tiles by the same model, in
+// microseconds: a round of the 128-row tiles walks 4096 of K in 52 us, of the 64-row tiles
+// in 42 us; x = tiles x slices / CUs up to 1 is one round, beyond that 0.45 + 0.78 x rounds
+// (workgroups that share a CU slow each other down: measured 1.38 / 1.56 / 1.83 / 2.73 / 5.2
+// rounds at x = 1.125 / 1.5 / 2 / 3 / 6).
+double staged_launch_us(const Problem& p, const tlhip_kernel_config_t& c) {
   const int cus = device_cu_count() > 0 ? device_cu_count() : 256;
   const int ks = c.p5 > 1 ? c.p5 : 1;
   const int64_t tiles = ((p.m + c.p0 - 1) / c.p0) * ((p.n + c.p1 - 1) / c.p1);
-  const double walk = c.variant == VARIANT_TILED_DIRECT ? 42.0 : (c.p0 <= 64 ? 42.0 : 52.0);
   const double fill = (double)(tiles * ks) / (double)cus;
   const double rounds = fill <= 1.0 ? 1.0 : 0.45 + 0.78 * fill;
-  const double area = (double)c.p0 * c.p1 / (c.p0 <= 64 ? 64.0 * 128.0 : 128.0 * 128.0);  // larger tiles walk longer
-  const double sum_us = ks > 1 ? 6.0 + 0.6 * (double)ks * (double)p.m * (double)p.n * 4.0 / 1e6 : 0.0;
-  return rounds * walk * area * (double)p.k / 4096.0 / ks + sum_us;
+  const double walk_us = (c.p0 <= 64 ? 42.0 : 52.0) * (double)p.k / 4096.0 / ks;
+  const double sum_us = direct_round_us(p, ks, 0.0);  // the second launch of a K-sliced one
+  return rounds * walk_us + sum_us;
 }
 
 // K slices across workgroups for a launch of 128 x 128 tiles of the direct GEMM: of 1, 2,
@@ -300,7 +299,7 @@ tlhip_kernel_config_t default_config(const Problem& p) {
             split.p5 = ks;
             if (!gemm_config_applicable(p, split, nullptr)) continue;
           }
-          const double us = tiled_launch_us(p, split);
+          const double us = staged_launch_us(p, split);
           if (!have || us < best_us) {
             best_c = split;
             best_us = us;
