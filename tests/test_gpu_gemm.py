@@ -451,3 +451,28 @@ def test_prefill_scale_range(be, lo, hi, cfg):
     want = O.linear(x.astype(np.float32), deq, threads=8)
     assert np.isfinite(got).all()
     assert rel_l2(got, want) <= REL_L2_TOL, rel_l2(got, want)
+
+
+@pytest.mark.parametrize("m,cfg", [(300, None), (2100, None), (300, (3, 128, 128, 128, 2, 2)), (300, (2, 128, 128, 64, 2, 2))])
+def test_lm_head_sized_prefill_on_sampled_columns(be, m, cfg):
+    """256000 x 2304 int8-row (the Gemma-shaped LM head) above 16 rows: 2000 column tiles,
+    up to 2.1 GB of f32 logits.  The oracle runs on sampled blocks of 256 columns (the first,
+    the last, and six in between) of the first and the last 300 rows."""
+    rng = np.random.default_rng(m)
+    n, k = 256000, 2304
+    q = rng.integers(-127, 128, (n, k), dtype=np.int8)
+    packed = O.np_pack_int8(q)
+    rs = rng.uniform(0.002, 0.01, n).astype(np.float32)
+    x = make_x(m, k, "f16", rng, std=0.5)
+    w = be.createQuantizedWeight(packed, rs, n, k, T.resolveWeightFormat("int8-row", "f32"))
+    xt = be.ops.tensorFromArray(x, [m, k], "f16")
+    y = be.linear(xt, w, config=L.KernelConfig.of(*cfg) if cfg else None)
+    got = y.numpy()
+    assert got.shape == (m, n) and got.dtype == np.float32
+    rows = np.unique(np.concatenate([np.arange(min(m, 300)), np.arange(max(0, m - 300), m)]))
+    for c0 in [0, n - 256] + [int(c) * 256 for c in rng.integers(1, n // 256 - 1, 6)]:
+        deq = O.dequant_int8_row(packed.reshape(n, k // 4)[c0:c0 + 256].reshape(-1), rs[c0:c0 + 256], 256, k)
+        want = O.linear(x[rows].astype(np.float32), deq, threads=8)
+        assert rel_l2(got[rows][:, c0:c0 + 256], want) <= 5e-6, c0
+    for t in (y, xt, w):
+        t.destroy()
