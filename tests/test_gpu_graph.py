@@ -87,6 +87,63 @@ def test_graph_with_k_slices_and_topk_replays_bit_exact(be):
         t.destroy()
 
 
+@pytest.mark.parametrize("fmt,g,cfg", [("int4-grouped", 32, (3, 128, 128, 128, 2, 2, 4)),
+                                       ("int8-grouped", 64, (3, 256, 128, 128, 2, 4, 2)),
+                                       ("int8-row", 0, (2, 64, 128, 64, 2, 2, 8)),
+                                       ("int8-row", 0, None)])
+def test_graph_with_k_sliced_tiled_gemm_replays_bit_exact(be, fmt, g, cfg):
+    """A tiled GEMM whose K slices leave their partial sums in the stream's workspace and a
+    second launch adds them (or, with no configuration named, whatever the routing picks for
+    150 rows of f32 activations: a cast into the same workspace, then tiles): captured,
+    replayed five times with eager K-sliced work on the same workspace in between, every
+    replay bit-equal to the eager result."""
+    rng = np.random.default_rng(7)
+    m, n, k = 150, 640, 2048
+    packed, scales, deq = make_weight(fmt, n, k, g, rng)
+    xdt = "f16" if cfg else "f32"
+    x = make_x(m, k, xdt, rng, std=0.5)
+    name = "int8-row" if fmt == "int8-row" else f"{fmt.split('-')[0]}-{g}"
+    w = be.createQuantizedWeight(packed, scales, n, k, T.resolveWeightFormat(name, "f32"))
+    xt = be.ops.tensorFromArray(x, [m, k], xdt)
+    bias = be.ops.tensorFromArray(rng.standard_normal(n).astype(np.float32), [n], "f32")
+    y = be._alloc([m, n], "f32")
+    qw = be._qweight(w, False)
+    ep = be.makeEpilogue(bias, "gelu")
+    kc = L.KernelConfig.of(*cfg) if cfg else None
+
+    def enqueue():
+        if kc is not None:
+            L.check(L.load().tlhip_matmul_quantized_config(C.byref(qw), xt.ptr, L.F16, m, y.ptr, L.F32, 1.0,
+                                                           C.byref(ep), C.byref(kc), None))
+        else:
+            L.check(L.load().tlhip_matmul_quantized(C.byref(qw), xt.ptr, L.F32, m, y.ptr, L.F32, 1.0, C.byref(ep), None))
+
+    enqueue()
+    ref = y.numpy()
+    want = O.linear(x.astype(np.float32), deq, bias.numpy(), "gelu", threads=8)
+    assert rel_l2(ref, want) <= 1e-3
+    graph = C.c_void_p()
+    L.call("tlhip_graph_begin_capture", None)
+    enqueue()
+    L.call("tlhip_graph_end_capture", None, C.byref(graph))
+    w2, xt2, want2 = _problem(be, 1040, 12288, 8, 4)
+    cfg2 = L.KernelConfig.of(L.VARIANT_GEMV_MFMA, 8, 2, 4, 2)
+    try:
+        for replay in range(5):
+            L.call("tlhip_memset", y.ptr, 0xFF, y.nbytes, None)
+            out2 = be._alloc([8, 1040], "f32")
+            L.check(_gemv(be, w2, xt2, 8, out2, cfg2))
+            assert rel_l2(out2.numpy(), want2) <= 2e-6
+            out2.destroy()
+            be.synchronize()
+            L.call("tlhip_graph_launch", graph, None)
+            assert np.array_equal(y.numpy().view(np.uint32), ref.view(np.uint32)), replay
+    finally:
+        L.call("tlhip_graph_destroy", graph)
+    for t in (y, xt, w, bias):
+        t.destroy()
+
+
 def test_capture_rules(be):
     n, k, m = 512, 12288, 16
     w, xt, want = _problem(be, n, k, m, 5)
