@@ -42,7 +42,6 @@ struct GemmArgs {
   int cpg_shift;          // log2(16-byte chunks per scale group)
   int groups_per_row;
   int ksteps;
-  float scale_mul;
   TileMap map;
   OutArgs out;
   int ksplit;             // workgroups that share a tile, each walking ksteps / ksplit steps of K (1 = none)
@@ -77,32 +76,28 @@ struct WChunk<TLHIP_FMT_INT4_GROUPED> {
   }
 };
 
-template <int FMT>
-struct WChunkInt8 {
+// int8 with an f16 scale per group: the integer (exact in f16) times the scale as it is
+// stored, one rounding to f16 per weight; the format's 1/127 rides on alpha.
+template <>
+struct WChunk<TLHIP_FMT_INT8_GROUPED> {
   static constexpr int WEIGHTS = 16;
   static constexpr int UNITS = 2;
-  // The scale multiplies in f32 here ((q/127)*s is not an f16 product); one rounding to
-  // f16 per weight.
   __device__ static __forceinline__ void dequant(const u32x4& w, float scale, u32x4 (&out)[UNITS]) {
+    const _Float16 sh = (_Float16)scale;  // the scale is an f16 value: exact
+    const half2_t s2 = {sh, sh};
     const uint32_t words[4] = {w.x, w.y, w.z, w.w};
     uint32_t packed[8];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const float f0 = (float)(int8_t)(words[i] & 0xffu) * scale;
-      const float f1 = (float)(int8_t)((words[i] >> 8) & 0xffu) * scale;
-      const float f2 = (float)(int8_t)((words[i] >> 16) & 0xffu) * scale;
-      const float f3 = (float)(int8_t)(words[i] >> 24) * scale;
-      const half2_t a = {(_Float16)f0, (_Float16)f1};
-      const half2_t b = {(_Float16)f2, (_Float16)f3};
-      packed[2 * i] = __builtin_bit_cast(uint32_t, a);
-      packed[2 * i + 1] = __builtin_bit_cast(uint32_t, b);
+      half2_t h[2];
+      unpack_int8_word(words[i], h);
+      packed[2 * i] = __builtin_bit_cast(uint32_t, h[0] * s2);
+      packed[2 * i + 1] = __builtin_bit_cast(uint32_t, h[1] * s2);
     }
     out[0] = (u32x4){packed[0], packed[1], packed[2], packed[3]};
     out[1] = (u32x4){packed[4], packed[5], packed[6], packed[7]};
   }
 };
-template <>
-struct WChunk<TLHIP_FMT_INT8_GROUPED> : WChunkInt8<TLHIP_FMT_INT8_GROUPED> {};
 // int8 with one f32 scale per row: the bare integers go to the matrix cores (exact in f16)
 // and the row's scale multiplies the f32 sums in the epilogue, as a factor per output
 // column: no rounding of q * s to f16, and no scale that f16 could not hold.
@@ -200,7 +195,7 @@ __global__ __launch_bounds__(256) void gemm_prefill_kernel(const GemmArgs a) {
     for (int i = 0; i < W_LOADS; ++i) {
       const int u = tid + i * 256;
       const int r = u / W_CHUNKS_PER_ROW, c = u - r * W_CHUNKS_PER_ROW;
-      const float s = (GROUPED ? half_bits_to_float(sv[i]) : as_float(sv[i])) * a.scale_mul;
+      const float s = GROUPED ? half_bits_to_float(sv[i]) : 1.f;  // int8-row: the row scales are the epilogue's
       u32x4 out[WC::UNITS];
       WC::dequant(wv[i], s, out);
 #pragma unroll
@@ -358,13 +353,13 @@ int launch_gemm(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t st
     const int rc = split_workspace(stream, &a.workspace, &counters);
     if (rc) return rc;
   }
-  a.scale_mul = p.format == TLHIP_FMT_INT8_GROUPED ? (1.0f / 127.0f) : 1.0f;
   a.out.y = p.y;
   a.out.y_dtype = p.y_dtype;
   a.out.vec_ok = (p.n % 8 == 0) && ((uintptr_t)p.y % 16 == 0);
   a.out.m = (int)p.m;
   a.out.n = (int)p.n;
-  a.out.alpha = p.alpha;
+  // the grouped int8 format's 1/127 (quantize.ts: q = round(w / absmax * 127)) rides on alpha
+  a.out.alpha = p.format == TLHIP_FMT_INT8_GROUPED ? p.alpha * (1.0f / 127.0f) : p.alpha;
   a.out.epi = p.epi;
   a.out.col_scale = p.format == TLHIP_FMT_INT8_ROW ? (const float*)p.scales : nullptr;
   int rc;
