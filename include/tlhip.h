@@ -66,18 +66,31 @@ typedef enum {
   TLHIP_UNARY_TANH = 6
 } tlhip_unary_t;
 
-typedef enum { TLHIP_EPI_NONE = 0, TLHIP_EPI_BIAS = 1, TLHIP_EPI_UNARY = 2 } tlhip_epilogue_kind_t;
+typedef enum {
+  TLHIP_EPI_NONE = 0,
+  TLHIP_EPI_BIAS = 1,
+  TLHIP_EPI_UNARY = 2,
+  TLHIP_EPI_BINARY = 3,  /* add / sub / mul with an [M,N] input, indexed by output element */
+  TLHIP_EPI_CAST_F16 = 4 /* {kind: "cast", toDtype: "f16"}: the value is rounded to f16 at this point of the chain */
+} tlhip_epilogue_kind_t;
+
+/* The op of a BINARY step (`op` of {kind: "binary"}: "add", "sub", "mul";
+ * src/schedule/matmul-skeleton.ts:934-955). */
+typedef enum { TLHIP_BINARY_ADD = 0, TLHIP_BINARY_SUB = 1, TLHIP_BINARY_MUL = 2 } tlhip_binary_t;
 
 #define TLHIP_MAX_EPILOGUE_OPS 4
 
 /* One step of an epilogue chain: EpilogueOp
  * (src/backend/webgpu/matmul/types.ts:13-24).  BIAS adds input[n] (indexed by
- * output column); UNARY applies `unary`. */
+ * output column); UNARY applies `unary`; BINARY combines the value with
+ * input[m*N + n] (an [M,N] tensor, contiguous: value + input, value - input or
+ * value * input; a residual add, a gate; the library sees a pointer, so that it
+ * holds M*N elements is the caller's to ensure); CAST_F16 rounds the value to f16. */
 typedef struct {
   int32_t kind;        /* tlhip_epilogue_kind_t */
-  int32_t unary;       /* tlhip_unary_t, for kind == UNARY */
-  const void* input;   /* device [N], for kind == BIAS */
-  int32_t input_dtype; /* tlhip_dtype_t of input */
+  int32_t unary;       /* tlhip_unary_t for kind == UNARY, tlhip_binary_t for kind == BINARY */
+  const void* input;   /* device [N] for kind == BIAS, device [M,N] for kind == BINARY */
+  int32_t input_dtype; /* tlhip_dtype_t of input (f32 or f16) */
   int32_t reserved;
 } tlhip_epilogue_op_t;
 

@@ -107,12 +107,25 @@ for (const c of manifest.cases) {
     r.dtype = y1.dtype;
     r.plan = D.planBareMatmul(x, be.ops.transpose(w));
     [y1, y2, y3, y4].forEach((y, i) => save(c.out + i, be.readSync(y)));
-    try {
+    // matmul -> bias -> unary -> add residual: a binary step with an [M,N] input
+    const residual = tensor(be, c.residual, [c.m, c.n], "f32");
+    const chain = { ops: [{ kind: "bias", inputIndex: 0 }, { kind: "unary", op: c.act }, { kind: "binary", op: "add", inputIndex: 1 }],
+                    additionalInputCount: 2, outputDtype: c.out_dtype };
+    save(c.out + "_residual", be.readSync(D.dispatchMatmul(x, be.ops.transpose(w), false, false, undefined,
+      { epilogue: chain, epilogueInputs: [bias, residual] })));
+    try {   // an [N] tensor where the [M,N] one belongs must be refused, not read out of bounds
       D.dispatchMatmul(x, be.ops.transpose(w), false, false, undefined,
         { epilogue: { ops: [{ kind: "binary", op: "mul", inputIndex: 0 }], additionalInputCount: 1, outputDtype: "f32" }, epilogueInputs: [bias] });
       r.binary_error = null;
     } catch (e) {
       r.binary_error = e.message;
+    }
+    try {
+      D.dispatchMatmul(x, be.ops.transpose(w), false, false, undefined,
+        { epilogue: { ops: [{ kind: "binary", op: "div", inputIndex: 0 }], additionalInputCount: 1, outputDtype: "f32" }, epilogueInputs: [residual] });
+      r.binary_op_error = null;
+    } catch (e) {
+      r.binary_op_error = e.message;
     }
   } else if (c.kind === "topk") {
     const logits = tensor(be, c.logits, [c.length], "f32");

@@ -123,11 +123,14 @@ def run(tmp_path_factory):
         packed, scales, deq = make_weight("int4-grouped", n, k, g, rng)
         x = make_x(m, k, xdt, rng)
         bias = rng.standard_normal(n).astype(np.float32)
+        residual = rng.standard_normal((m, n)).astype(np.float32)
         cases.append({"kind": "side_door", "name": name, "format": "int4-32", "element": "f16", "n": n, "k": k, "m": m,
                       "xdtype": xdt, "act": "silu", "out_dtype": out_dtype, "packed": put(name + ".packed", packed),
                       "scales": put(name + ".scales", scales), "x": put(name + ".x", x.astype(np.float32)),
-                      "bias": put(name + ".bias", bias), "out": name + ".y"})
-        want[name] = (O.linear(x.astype(np.float32), deq, bias, "silu"), out_dtype, (m, n))
+                      "bias": put(name + ".bias", bias), "residual": put(name + ".residual", residual), "out": name + ".y"})
+        lin = O.linear(x.astype(np.float32), deq, bias, "silu")
+        want[name] = (lin, out_dtype, (m, n))
+        want[name + "_residual"] = (lin + residual).astype(np.float32)
 
     rng = seeded("addon", "topk")
     logits = rng.standard_normal(50000).astype(np.float32)
@@ -194,7 +197,13 @@ def test_fused_side_door(run, name):
     r = run["results"]["cases"][name]
     assert r["launches"] == 1 and r["dtype"] == dtype and r["donated_reused"] is True
     assert r["plan"] == "quantized-operand"           # planBareMatmul: webgpu/dispatch.ts:826
-    assert "binary" in r["binary_error"]
+    if shape[0] > 1:
+        assert "[M,N]" in r["binary_error"]              # an [N] tensor as a binary step's input is refused
+    else:
+        assert r["binary_error"] is None                 # one row: [N] is [M,N]
+    assert "Unsupported binary epilogue: div" in r["binary_op_error"]   # matmul-skeleton.ts:953
+    yr = run["get"](f"{name}.y_residual").reshape(shape)
+    assert rel_l2(yr, run["want"][name + "_residual"]) <= (1e-5 if dtype == "f32" else 1e-3)
     ys = [run["get"](f"{name}.y{i}").reshape(shape) for i in range(4)]
     for y in ys:
         assert rel_l2(y, want) <= (1e-5 if dtype == "f32" else 1e-3)

@@ -20,7 +20,8 @@ FMT_INT8_GROUPED, FMT_INT8_ROW, FMT_INT4_GROUPED = 0, 1, 2
 F32, F16, I32 = 0, 1, 2
 UNARY = {"none": 0, "relu": 1, "silu": 2, "gelu": 3, "gelu_tanh": 3, "gelu_erf": 4,
          "sigmoid": 5, "tanh": 6}
-EPI_NONE, EPI_BIAS, EPI_UNARY = 0, 1, 2
+EPI_NONE, EPI_BIAS, EPI_UNARY, EPI_BINARY, EPI_CAST_F16 = 0, 1, 2, 3, 4
+BINARY = {"add": 0, "sub": 1, "mul": 2}
 MAX_EPILOGUE_OPS = 4
 VARIANT_GEMV, VARIANT_GEMV_MFMA, VARIANT_TILED, VARIANT_TILED_DIRECT, VARIANT_GEMV_XREG = 0, 1, 2, 3, 4
 

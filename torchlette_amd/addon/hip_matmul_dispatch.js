@@ -14,11 +14,13 @@ const tl = H.native;
 
 const DT = { f32: 0, f16: 1 };
 const UNARY = { relu: 1, silu: 2, gelu: 3, gelu_tanh: 3, gelu_erf: 4, sigmoid: 5, tanh: 6 };
-const EPI_BIAS = 1, EPI_UNARY = 2;
+const EPI_BIAS = 1, EPI_UNARY = 2, EPI_BINARY = 3, EPI_CAST_F16 = 4;
+const BINARY = { add: 0, sub: 1, mul: 2 };
 
-/** EpilogueConfig.ops (matmul/types.ts:13-24) -> the addon's op list.  `cast` may only
- *  close the chain and must name the output dtype; `binary` is not part of this path. */
-function lowerEpilogue(epilogue, epilogueInputs, outputDtype) {
+/** EpilogueConfig.ops (matmul/types.ts:13-24) -> the addon's op list.  `binary` takes an
+ *  [M,N] input (add, sub, mul: matmul-skeleton.ts:934-955); a `cast` to f16 in the middle of
+ *  the chain rounds the value there, one that closes the chain must name the output dtype. */
+function lowerEpilogue(epilogue, epilogueInputs, outputDtype, m, n) {
   const ops = [];
   const list = (epilogue && epilogue.ops) || [];
   list.forEach((op, i) => {
@@ -31,9 +33,22 @@ function lowerEpilogue(epilogue, epilogueInputs, outputDtype) {
     } else if (op.kind === "unary") {
       if (!(op.op in UNARY)) throw new Error(`hip dispatchMatmul: unary epilogue op ${op.op} is not built`);
       ops.push([EPI_UNARY, UNARY[op.op], null, 0]);
+    } else if (op.kind === "binary") {
+      const t = epilogueInputs[op.inputIndex];
+      if (!t) throw new Error(`hip dispatchMatmul: epilogue input ${op.inputIndex} missing`);
+      if (!(t.dtype in DT)) throw new Error(`hip dispatchMatmul: binary epilogue input dtype ${t.dtype}`);
+      if (!(op.op in BINARY)) throw new Error(`Unsupported binary epilogue: ${op.op}`);
+      // the kernels index it by output element: anything but M*N elements would be read out of bounds
+      const count = t.size !== undefined ? t.size : t.nbytes / (t.dtype === "f16" ? 2 : 4);
+      if (count !== m * n || !t.isContiguous)
+        throw new Error(`hip dispatchMatmul: a binary epilogue input must be a contiguous [M,N] = [${m},${n}] tensor`);
+      ops.push([EPI_BINARY, BINARY[op.op], t.ptr, DT[t.dtype]]);
     } else if (op.kind === "cast") {
-      if (i !== list.length - 1 || op.toDtype !== outputDtype)
-        throw new Error("hip dispatchMatmul: a cast may only close the chain, to the output dtype");
+      if (i === list.length - 1) {
+        if (op.toDtype !== outputDtype) throw new Error("hip dispatchMatmul: the cast that closes the chain must name the output dtype");
+      } else if (op.toDtype === "f16") {
+        ops.push([EPI_CAST_F16, 0, null, 0]);
+      }  // a cast to f32 in the chain changes nothing: the chain computes in f32
     } else {
       throw new Error(`hip dispatchMatmul: epilogue op kind ${op.kind} is not built`);
     }
@@ -55,9 +70,9 @@ function dispatchMatmul(a, b, transA, transB, donatedBuffer, epilogueOpts) {
   if (!a.isContiguous) throw new Error("matmulQuantizedB: strided activations");
   const promoted = a.dtype === "f16" && b.format.elementType === "f16" ? "f16" : "f32";
   const outputDtype = (epilogueOpts && epilogueOpts.epilogue && epilogueOpts.epilogue.outputDtype) || promoted;
-  const ops = epilogueOpts ? lowerEpilogue(epilogueOpts.epilogue, epilogueOpts.epilogueInputs || [], outputDtype) : [];
-  const outShape = a.shape.slice(0, -1).concat([n]);
   const m = k ? a.size / k : 0;
+  const ops = epilogueOpts ? lowerEpilogue(epilogueOpts.epilogue, epilogueOpts.epilogueInputs || [], outputDtype, m, n) : [];
+  const outShape = a.shape.slice(0, -1).concat([n]);
   const need = outShape.reduce((p, c) => p * c, 1) * (outputDtype === "f16" ? 2 : 4);
   let out;
   if (donatedBuffer && donatedBuffer.nbytes >= need) {
@@ -78,7 +93,7 @@ function dispatchMatmulDirect(bufA, bufB, config) {
   if (!p) throw new Error("hip dispatchMatmulDirect: config.packing is required");
   const be = H.getBackend();
   const FMT = { "int8-grouped": 0, "int8-row": 1, "int4-grouped": 2 };
-  const ops = lowerEpilogue(config.epilogueConfig, config.epilogueBuffers || [], config.outputDtype);
+  const ops = lowerEpilogue(config.epilogueConfig, config.epilogueBuffers || [], config.outputDtype, config.m, config.n);
   const out = be._alloc(config.outShape, config.outputDtype);
   tl.matmulQuantizedOps(FMT[p.scheme], p.groupSize, config.n, config.k, bufB.ptr, config.scales.ptr, bufA.ptr,
     DT[config.dtypeA], config.m, out.ptr, DT[config.outputDtype], ops);

@@ -496,6 +496,9 @@ class HipBackend:
         out_shape = (a.shape[:-1] if len(a.shape) > 1 else []) + [qw.n]
         if len(a.shape) == 1:
             out_shape = [qw.n]
+        for size in getattr(epilogue, "_binary_sizes", []):
+            if size != m * qw.n:
+                raise ValueError(f"a binary epilogue input must be an [M,N] = [{m},{qw.n}] tensor")
         out = self._alloc(out_shape, out_dtype)
         ep = C.byref(epilogue) if epilogue is not None else None
         if config is None:
@@ -507,17 +510,40 @@ class HipBackend:
         return out
 
     @staticmethod
-    def makeEpilogue(bias: Optional[HipTensor] = None, activation: Optional[str] = None) -> L.Epilogue:
-        """EpilogueConfig {ops: [bias?, unary?]} (matmul/types.ts:13-24)."""
+    def makeEpilogue(bias: Optional[HipTensor] = None, activation: Optional[str] = None,
+                     binary: Optional[Sequence] = None) -> L.Epilogue:
+        """EpilogueConfig {ops: [bias?, unary?, binary?]} (matmul/types.ts:13-24); `binary` is
+        (op, tensor) with op in add / sub / mul and an [M,N] tensor (a residual, a gate)."""
+        return HipBackend.makeEpilogueChain(([("bias", bias)] if bias is not None else []) +
+                                            ([("unary", activation)] if activation and activation != "none" else []) +
+                                            ([("binary",) + tuple(binary)] if binary is not None else []))
+
+    @staticmethod
+    def makeEpilogueChain(ops: Sequence[Sequence]) -> L.Epilogue:
+        """EpilogueConfig.ops in the caller's order: ("bias", tensor[N]), ("unary", name),
+        ("binary", op, tensor[M,N]), ("cast", "f16") (matmul-skeleton.ts:916-966)."""
+        if len(ops) > L.MAX_EPILOGUE_OPS:
+            raise ValueError(f"at most {L.MAX_EPILOGUE_OPS} epilogue ops")
         ep = L.Epilogue()
-        i = 0
-        if bias is not None:
-            ep.ops[i] = L.EpilogueOp(L.EPI_BIAS, 0, bias.ptr, _DT_CODE[bias.dtype], 0)
-            i += 1
-        if activation and activation != "none":
-            ep.ops[i] = L.EpilogueOp(L.EPI_UNARY, L.UNARY[activation], None, 0, 0)
-            i += 1
-        ep.n_ops = i
+        binary_sizes = []   # checked against M * N at the call: the kernels index these inputs by output element
+        for i, op in enumerate(ops):
+            if op[0] == "bias":
+                ep.ops[i] = L.EpilogueOp(L.EPI_BIAS, 0, op[1].ptr, _DT_CODE[op[1].dtype], 0)
+            elif op[0] == "unary":
+                ep.ops[i] = L.EpilogueOp(L.EPI_UNARY, L.UNARY[op[1]], None, 0, 0)
+            elif op[0] == "binary":
+                if op[1] not in L.BINARY:
+                    raise ValueError(f"Unsupported binary epilogue: {op[1]}")
+                if not op[2].isContiguous:
+                    raise ValueError("a binary epilogue input must be contiguous")
+                ep.ops[i] = L.EpilogueOp(L.EPI_BINARY, L.BINARY[op[1]], op[2].ptr, _DT_CODE[op[2].dtype], 0)
+                binary_sizes.append(op[2].size)
+            elif op[0] == "cast":
+                ep.ops[i] = L.EpilogueOp(L.EPI_CAST_F16 if op[1] == "f16" else L.EPI_NONE, 0, None, 0, 0)
+            else:
+                raise ValueError(f"unknown epilogue op {op[0]}")
+        ep.n_ops = len(ops)
+        ep._binary_sizes = binary_sizes
         return ep
 
     def linear(self, input: HipTensor, weight: HipTensor, bias: Optional[HipTensor] = None,

@@ -42,6 +42,15 @@ struct DevEpilogue {
   const void* input[TLHIP_MAX_EPILOGUE_OPS];
 };
 
+// The epilogue of the rows from m0 on of a problem with n columns: a binary step's [M,N]
+// input starts m0 rows further, like the output.
+inline DevEpilogue epilogue_from_row(DevEpilogue e, int64_t m0, int64_t n) {
+  for (int i = 0; i < e.n_ops; ++i)
+    if (e.kind[i] == TLHIP_EPI_BINARY && e.input[i])
+      e.input[i] = (const char*)e.input[i] + m0 * n * (e.input_dtype[i] == TLHIP_F16 ? 2 : 4);
+  return e;
+}
+
 // Prologue of the VALU decode GEMV (tlhip_prologue_t as the kernel takes it).
 struct DevPrologue {
   int kind;

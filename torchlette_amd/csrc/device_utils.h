@@ -60,27 +60,36 @@ __device__ __forceinline__ float apply_unary(int op, float v) {
   }
 }
 
-// acc*alpha, then the ops in order; `col` is the output column n.
-__device__ __forceinline__ float apply_epilogue(const DevEpilogue& ep, float v, int64_t col) {
-  for (int i = 0; i < ep.n_ops; ++i) {
-    if (ep.kind[i] == TLHIP_EPI_BIAS) {
-      float b;
-      if (ep.input_dtype[i] == TLHIP_F16) b = (float)((const _Float16*)ep.input[i])[col];
-      else b = ((const float*)ep.input[i])[col];
-      v += b;
-    } else if (ep.kind[i] == TLHIP_EPI_UNARY) {
-      v = apply_unary(ep.unary[i], v);
-    }
+// One step of the chain on one value: `col` is the output column n, `idx` the output
+// element m*N + n (what a binary step's [M,N] input is indexed by).
+__device__ __forceinline__ float apply_epilogue_step(int kind, int op, const void* input, int input_dtype, float v,
+                                                     int64_t col, int64_t idx) {
+  if (kind == TLHIP_EPI_BIAS || kind == TLHIP_EPI_BINARY) {
+    const int64_t at = kind == TLHIP_EPI_BIAS ? col : idx;
+    float b;
+    if (input_dtype == TLHIP_F16) b = (float)((const _Float16*)input)[at];
+    else b = ((const float*)input)[at];
+    if (kind == TLHIP_EPI_BIAS || op == TLHIP_BINARY_ADD) return v + b;
+    return op == TLHIP_BINARY_SUB ? v - b : v * b;
   }
+  if (kind == TLHIP_EPI_UNARY) return apply_unary(op, v);
+  if (kind == TLHIP_EPI_CAST_F16) return (float)(_Float16)v;
   return v;
 }
 
-// The same on COUNT values of one output column: the ops are the outer loop, unrolled
-// over the fixed capacity with constant indices, so that the epilogue's fields stay in
-// scalar registers however many values the caller holds (a run-time index into the
-// kernel arguments makes the compiler copy them to scratch memory).
-template <int COUNT>
-__device__ __forceinline__ void apply_epilogue_all(const DevEpilogue& ep, float (&v)[COUNT], int64_t col) {
+// acc*alpha, then the ops in order.
+__device__ __forceinline__ float apply_epilogue(const DevEpilogue& ep, float v, int64_t col, int64_t idx) {
+  for (int i = 0; i < ep.n_ops; ++i) v = apply_epilogue_step(ep.kind[i], ep.unary[i], ep.input[i], ep.input_dtype[i], v, col, idx);
+  return v;
+}
+
+// The same on COUNT values of one output column (element_of(j): the output element of
+// value j, or -1 for a value that will not be stored): the ops are the outer loop,
+// unrolled over the fixed capacity with constant indices, so that the epilogue's fields
+// stay in scalar registers however many values the caller holds (a run-time index into
+// the kernel arguments makes the compiler copy them to scratch memory).
+template <int COUNT, typename ElementOf>
+__device__ __forceinline__ void apply_epilogue_all(const DevEpilogue& ep, float (&v)[COUNT], int64_t col, ElementOf element_of) {
 #pragma unroll
   for (int i = 0; i < TLHIP_MAX_EPILOGUE_OPS; ++i) {
     if (i < ep.n_ops) {
@@ -93,6 +102,12 @@ __device__ __forceinline__ void apply_epilogue_all(const DevEpilogue& ep, float 
       } else if (ep.kind[i] == TLHIP_EPI_UNARY) {
 #pragma unroll
         for (int j = 0; j < COUNT; ++j) v[j] = apply_unary(ep.unary[i], v[j]);
+      } else if (ep.kind[i] != TLHIP_EPI_NONE) {
+#pragma unroll
+        for (int j = 0; j < COUNT; ++j) {
+          const int64_t idx = element_of(j);
+          if (idx >= 0) v[j] = apply_epilogue_step(ep.kind[i], ep.unary[i], ep.input[i], ep.input_dtype[i], v[j], col, idx);
+        }
       }
     }
   }

@@ -602,6 +602,7 @@ bool f32_rows_through_tiled(const Problem& p, hipStream_t stream, int* rc) {
     if (*rc) return true;
     q.x = workspace;
     q.y = (char*)p.y + m0 * p.n * yb;
+    q.epi = epilogue_from_row(p.epi, m0, p.n);
     *rc = run_config(q, c, stream);
     if (*rc) return true;
   }
@@ -623,6 +624,7 @@ int matmul_with(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t st
     q.m = std::min<int64_t>(16, p.m - m0);
     q.x = (const char*)p.x + m0 * p.k * xb;
     q.y = (char*)p.y + m0 * p.n * yb;
+    q.epi = epilogue_from_row(p.epi, m0, p.n);
     int rc = run_config(q, c, stream);
     if (rc) return rc;
   }
@@ -740,6 +742,7 @@ int run_selected(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t s
     q.m = std::min<int64_t>(r.chunk, p.m - m0);
     q.x = (const char*)p.x + m0 * p.k * xb;
     q.y = (char*)p.y + m0 * p.n * yb;
+    q.epi = epilogue_from_row(p.epi, m0, p.n);
     const int rc = matmul_with(q, q.m == r.chunk ? r.first : r.last, stream);
     if (rc) return rc;
   }
@@ -1095,8 +1098,15 @@ int make_problem(const tlhip_qweight_t* w, const void* x, int x_dtype, int64_t m
     p->epi.n_ops = epilogue->n_ops;
     for (int i = 0; i < epilogue->n_ops; ++i) {
       const tlhip_epilogue_op_t& op = epilogue->ops[i];
-      if (op.kind != TLHIP_EPI_NONE && op.kind != TLHIP_EPI_BIAS && op.kind != TLHIP_EPI_UNARY)
+      if (op.kind < TLHIP_EPI_NONE || op.kind > TLHIP_EPI_CAST_F16)
         return set_error(TLHIP_ERR_INVALID, "%s: unknown epilogue op kind %d", who, op.kind);
+      if (op.kind == TLHIP_EPI_BINARY) {
+        if (!op.input && w->n > 0 && m > 0) return set_error(TLHIP_ERR_INVALID, "%s: binary epilogue without input", who);
+        if (op.input_dtype != TLHIP_F32 && op.input_dtype != TLHIP_F16)
+          return set_error(TLHIP_ERR_INVALID, "%s: bad binary epilogue input dtype %d", who, op.input_dtype);
+        if (op.unary < TLHIP_BINARY_ADD || op.unary > TLHIP_BINARY_MUL)
+          return set_error(TLHIP_ERR_INVALID, "%s: unknown binary epilogue op %d (add, sub, mul)", who, op.unary);
+      }
       if (op.kind == TLHIP_EPI_BIAS) {
         if (!op.input && w->n > 0) return set_error(TLHIP_ERR_INVALID, "%s: bias epilogue without input", who);
         if (op.input_dtype != TLHIP_F32 && op.input_dtype != TLHIP_F16)

@@ -215,7 +215,10 @@ __device__ __forceinline__ void wave_epilogue(float* patch, const float16_t (&ac
         for (int e = 0; e < 8; ++e) v[e] = apply_unary(unary, v[e] * scale_of(e) + bias[e]);
       } else {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) v[e] = apply_epilogue(o.epi, v[e] * scale_of(e), min(col + e, o.n - 1));
+        for (int e = 0; e < 8; ++e) {
+          const int c = min(col + e, o.n - 1);
+          v[e] = apply_epilogue(o.epi, v[e] * scale_of(e), c, (int64_t)row * o.n + c);
+        }
       }
       if (vec) {
         const int64_t idx = (int64_t)row * o.n + col;

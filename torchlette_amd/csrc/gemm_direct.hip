@@ -366,9 +366,10 @@ __global__ __launch_bounds__(WM * WN * 64, (TM * TN >= 16 ? 1 : 2)) void gemm_di
     wave_epilogue<TN, true, ROW>(patch, acc[i], lane, m0 + (wm * TM + i) * 32, n0 + wn * TN * 32, a.out, plane);
 }
 
-// v[e] = ops(alpha * v[e]) for the W consecutive columns from `col` on.
+// v[e] = ops(alpha * v[e]) for the W consecutive columns from `col` on (output elements
+// from `idx` on).
 template <int W>
-__device__ __forceinline__ void apply_epilogue_scaled(const OutArgs& o, float (&v)[W], int64_t col) {
+__device__ __forceinline__ void apply_epilogue_scaled(const OutArgs& o, float (&v)[W], int64_t col, int64_t idx) {
 #pragma unroll
   for (int e = 0; e < W; ++e) v[e] *= o.col_scale ? o.alpha * o.col_scale[col + e] : o.alpha;
 #pragma unroll
@@ -383,6 +384,10 @@ __device__ __forceinline__ void apply_epilogue_scaled(const OutArgs& o, float (&
       } else if (o.epi.kind[i] == TLHIP_EPI_UNARY) {
 #pragma unroll
         for (int e = 0; e < W; ++e) v[e] = apply_unary(o.epi.unary[i], v[e]);
+      } else if (o.epi.kind[i] != TLHIP_EPI_NONE) {
+#pragma unroll
+        for (int e = 0; e < W; ++e)
+          v[e] = apply_epilogue_step(o.epi.kind[i], o.epi.unary[i], o.epi.input[i], o.epi.input_dtype[i], v[e], col + e, idx + e);
       }
     }
   }
@@ -423,7 +428,7 @@ __global__ __launch_bounds__(256) void direct_reduce_kernel(const float* __restr
     for (int sl = 0; sl < KS; ++sl) v[e] += part[sl][e];  // slice order
   }
   const int64_t col = idx % o.n;
-  apply_epilogue_scaled(o, v, col);
+  apply_epilogue_scaled(o, v, col, idx);
   if constexpr (VEC) {
     if (o.y_dtype == TLHIP_F16) {
       half8_t h;

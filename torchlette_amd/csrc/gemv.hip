@@ -83,7 +83,7 @@ static void fill_args(const Problem& p, const tlhip_kernel_config_t& c, int64_t 
   a.alpha = p.alpha;
   a.scale_mul = p.format == TLHIP_FMT_INT8_GROUPED ? (1.0f / 127.0f) : 1.0f;
   a.y_dtype = p.y_dtype;
-  a.epi = p.epi;
+  a.epi = epilogue_from_row(p.epi, m0, p.n);  // this pass starts at row m0, like y
   a.pro = p.pro;
   if (a.pro.kind == TLHIP_PRO_GATED_MUL) a.pro.operand = (const char*)p.pro.operand + m0 * p.k * xbytes;
   // LDS: staged x (mt rows) + split-K partials

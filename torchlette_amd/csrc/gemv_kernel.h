@@ -334,7 +334,7 @@ __device__ __forceinline__ void gemv_body(const GemvArgs& a, const int bid, cons
           for (int m = 0; m < MT; ++m) {
             if (m < a.m) {
               float v = acc[r][m] * (row_scale[r] * a.scale_mul) * a.alpha;
-              v = apply_epilogue(a.epi, v, row);
+              v = apply_epilogue(a.epi, v, row, (int64_t)m * a.n + row);
               store_out(a.y, a.y_dtype, (int64_t)m * a.n + row, v);
             }
           }

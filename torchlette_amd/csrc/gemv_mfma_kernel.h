@@ -434,7 +434,7 @@ __global__ __launch_bounds__(MAXT) void gemv_mfma_kernel(const MfmaArgs a) {
           for (int r = 0; r < 4; ++r) {
             const int m = 4 * g + r;
             if (m < mrows) {
-              const float v = apply_epilogue(P.epi, tile[0][r] * rs, orow);
+              const float v = apply_epilogue(P.epi, tile[0][r] * rs, orow, (int64_t)m * P.n + orow);
               store_out(P.y, a.y_dtype, (int64_t)m * P.n + orow, v);
             }
           }
@@ -444,7 +444,10 @@ __global__ __launch_bounds__(MAXT) void gemv_mfma_kernel(const MfmaArgs a) {
           for (int t = 0; t < MT; ++t)
 #pragma unroll
             for (int r = 0; r < 4; ++r) v[4 * t + r] = tile[t][r] * rs;
-          apply_epilogue_all(P.epi, v, orow);
+          apply_epilogue_all(P.epi, v, orow, [&](int j) -> int64_t {
+            const int m = 16 * (j >> 2) + 4 * g + (j & 3);
+            return m < mrows ? (int64_t)m * P.n + orow : (int64_t)-1;
+          });
 #pragma unroll
           for (int t = 0; t < MT; ++t)
 #pragma unroll

@@ -277,7 +277,7 @@ __global__ __launch_bounds__(MAXT) void gemv_xreg_kernel(const XregArgs a) {
         for (int q = 0; q < 4; ++q) {
           const int m = 4 * g + q;
           if (m < mrows) {
-            const float v = apply_epilogue(P.epi, sum[q] * a.alpha, orow);
+            const float v = apply_epilogue(P.epi, sum[q] * a.alpha, orow, (int64_t)m * P.n + orow);
             store_out(P.y, a.y_dtype, (int64_t)m * P.n + orow, v);
           }
         }
