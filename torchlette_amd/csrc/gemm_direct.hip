@@ -1,8 +1,10 @@
-// Prefill GEMM over packed int4 weights, second form: the weights stay PACKED
-// until they are in the operand registers.  Y[M,N] = epilogue(alpha * X[M,K] *
-// W[N,K]^T); same contract and reference route as gemm_prefill.hip
+// Prefill GEMM over packed weights, second form: the weights stay PACKED until they
+// are in the operand registers.  Y[M,N] = epilogue(alpha * X[M,K] * W[N,K]^T); same
+// contract and reference route as gemm_prefill.hip
 // (src/backend/webgpu/ops/matmul-ops.ts:163-181;
-// src/schedule/matmul-skeleton.ts:738-966).
+// src/schedule/matmul-skeleton.ts:738-966).  Written for int4 in groups, described
+// below; the int8 forms (groups of 64 or more, and one scale per row) are the same
+// pipeline on 128 bytes per row and step, described at the kernel's template flags.
 //
 // Why a second form: with the dequantised f16 weights staged through LDS a tile
 // moves about 1 KB of LDS traffic per MFMA and the kernel is bound by LDS, not
