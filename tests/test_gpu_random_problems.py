@@ -1,7 +1,9 @@
 """Seeded random problems through the seam call with NO configuration named: whatever the
 library's routing picks for a shape (VALU or matrix-core GEMV, rows in one or several
 launches, K slices of equal or unequal length, tiled launches with or without K slices
-across workgroups, the f32 routes) must give the oracle's result.
+across workgroups, the f32 routes) must give the oracle's result; a third of the problems
+end their epilogue with a binary step on an [M,N] input, which has to move with every slice
+of rows a route makes.
 
 Tolerances: rel-L2 <= 1e-3 (the stated bar) everywhere; f16 activations with f32 output on
 at most 16 rows <= 2e-6 (exact products, f32 accumulate: order noise only)."""
@@ -44,6 +46,12 @@ def draw(seed):
     return rng, fmt, g, m, n, k, xdt, ydt, bias, act
 
 
+def draw_binary(rng):
+    """A third of the problems close their chain with a binary step on an [M,N] input (a
+    residual add, or a gate), drawn after everything else so that the other draws stay."""
+    return [None, None, "add", "mul", None, None][rng.integers(6)]
+
+
 @pytest.fixture(scope="module")
 def be():
     return T.getBackend()
@@ -60,10 +68,20 @@ def test_whatever_the_routing_picks_matches_the_oracle(be, seed):
     bias = f16_round(rng.standard_normal(n) * 0.1).astype(np.float32) if has_bias else None
     bt = be.ops.tensorFromArray(bias, [n], "f32") if has_bias else None
     sel = be.selectedConfig(w, xdt, m, ydt).as_tuple()
-    y = be.linear(xt, w, bt, act, fused=True)
+    binary = draw_binary(rng)
+    other = f16_round(rng.standard_normal((m, n))).astype(np.float32) if binary else None
+    ot = be.ops.tensorFromArray(other, [m, n], "f32") if binary else None
+
+    def linear():
+        ep = be.makeEpilogue(bt, act, (binary, ot) if binary else None)
+        return be._matmulQuantizedB(xt, be.ops.transpose(w), ep, None)
+
+    y = linear()
     got = y.numpy()
     want = O.linear(x.astype(np.float32), deq, bias, act or "none", threads=8)
-    what = (fmt, g, m, n, k, xdt, ydt, has_bias, act, sel)
+    if binary:
+        want = (want + other if binary == "add" else want * other).astype(np.float32)
+    what = (fmt, g, m, n, k, xdt, ydt, has_bias, act, binary, sel)
     assert got.shape == (m, n), what
     assert got.dtype == (np.float16 if ydt == "f16" else np.float32), what
     assert np.isfinite(got).all(), what
@@ -72,9 +90,9 @@ def test_whatever_the_routing_picks_matches_the_oracle(be, seed):
     if xdt == "f16" and ydt == "f32" and m <= 16:
         assert err <= 2e-6, (err, what)
     # the same call again gives the same bits (no route depends on arrival order)
-    y2 = be.linear(xt, w, bt, act, fused=True)
+    y2 = linear()
     assert np.array_equal(y2.numpy(), got), what
-    for t in (y, y2, xt, w) + ((bt,) if bt is not None else ()):
+    for t in (y, y2, xt, w) + ((bt,) if bt is not None else ()) + ((ot,) if ot is not None else ()):
         t.destroy()
 
 
