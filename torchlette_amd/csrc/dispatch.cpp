@@ -342,6 +342,19 @@ tlhip_kernel_config_t default_config(const Problem& p) {
     // whole-line loads, four iterations in flight where they fit (tuned winner for all
     // three int8 formats at M = 4..16: 12.0-14.6 us against 14.2-17.4 us without)
     const bool int8 = p.format != TLHIP_FMT_INT4_GROUPED;
+    // first the full form (eight or four K-split waves, four iterations in flight) with as
+    // few K slices as let it fit: where 16 rows of K = 4096 leave no room for it in one
+    // slice, two slices take 14.4-14.7 us at 12288 x 4096 against 16.8-17.7 us for what
+    // does fit in one (two K-split waves, two iterations in flight)
+    if (int8 && p.n < 32768)
+      for (int ks = 1; ks <= 4; ks *= 2)
+        for (int i = 0; i < 2; ++i) {
+          // eight K-split waves first, four first where a workgroup walks a slice of more than 2048 of K
+          const int kw = (ks > 1 && p.k / ks > 2048) == (i == 0) ? 4 : 8;
+          tlhip_kernel_config_t c = mfma_cfg(8, 4, kw, ks);
+          c.p5 = 1;
+          if (gemv_mfma_config_applicable(p, c, nullptr)) return c;
+        }
     if (int8)
       for (int ks = 1; ks <= 4; ks *= 2) {  // one more K slice rather than no whole-line loads (14.3 against 17.4 us)
         const int preferred = p.n >= 32768 ? 1 : (ks > 1 ? 4 : 8);
