@@ -168,3 +168,32 @@ def test_format_names_resolve_like_the_reference():
     assert T.resolveWeightFormat("int8-128", "f32").packing.groupSize == 128
     assert T.resolveWeightFormat("int4-32").packing == T.QuantPacking("int4-grouped", 32, "f16")
     assert T.resolveWeightFormat("int8-row").packing.scheme == "int8-row"
+
+
+def test_enum_values_of_the_header_match_both_bindings():
+    """The ctypes mirror and the JavaScript files carry the header's enum values as plain
+    numbers: every one of them is checked against include/tlhip.h."""
+    import re
+    here = os.path.dirname(os.path.abspath(__file__))
+    header = open(os.path.join(here, "..", "include", "tlhip.h")).read()
+    enums = {name: int(value) for name, value in re.findall(r"\b(TLHIP_[A-Z0-9_]+)\s*=\s*(-?\d+)", header)}
+    assert enums["TLHIP_EPI_BINARY"] == 3 and enums["TLHIP_BINARY_MUL"] == 2   # the regex sees them
+    from torchlette_amd import _lib as L
+    assert (L.EPI_NONE, L.EPI_BIAS, L.EPI_UNARY, L.EPI_BINARY, L.EPI_CAST_F16) == tuple(
+        enums[n] for n in ("TLHIP_EPI_NONE", "TLHIP_EPI_BIAS", "TLHIP_EPI_UNARY", "TLHIP_EPI_BINARY", "TLHIP_EPI_CAST_F16"))
+    assert L.BINARY == {"add": enums["TLHIP_BINARY_ADD"], "sub": enums["TLHIP_BINARY_SUB"], "mul": enums["TLHIP_BINARY_MUL"]}
+    unary = {"none": "NONE", "relu": "RELU", "silu": "SILU", "gelu": "GELU_TANH", "gelu_tanh": "GELU_TANH",
+             "gelu_erf": "GELU_ERF", "sigmoid": "SIGMOID", "tanh": "TANH"}
+    assert L.UNARY == {k: enums["TLHIP_UNARY_" + v] for k, v in unary.items()}
+    assert (L.FMT_INT8_GROUPED, L.FMT_INT8_ROW, L.FMT_INT4_GROUPED) == (
+        enums["TLHIP_FMT_INT8_GROUPED"], enums["TLHIP_FMT_INT8_ROW"], enums["TLHIP_FMT_INT4_GROUPED"])
+    assert (L.F32, L.F16, L.I32) == (enums["TLHIP_F32"], enums["TLHIP_F16"], enums["TLHIP_I32"])
+    # the side door's constants (a JavaScript file: read as text)
+    js = open(os.path.join(here, "..", "torchlette_amd", "addon", "hip_matmul_dispatch.js")).read()
+    m = re.search(r"const EPI_BIAS = (\d+), EPI_UNARY = (\d+), EPI_BINARY = (\d+), EPI_CAST_F16 = (\d+);", js)
+    assert m and tuple(int(v) for v in m.groups()) == (L.EPI_BIAS, L.EPI_UNARY, L.EPI_BINARY, L.EPI_CAST_F16)
+    m = re.search(r"const BINARY = \{ add: (\d+), sub: (\d+), mul: (\d+) \};", js)
+    assert m and tuple(int(v) for v in m.groups()) == (L.BINARY["add"], L.BINARY["sub"], L.BINARY["mul"])
+    m = re.search(r"const UNARY = \{([^}]*)\};", js)
+    js_unary = {k.strip(): int(v) for k, v in (item.split(":") for item in m.group(1).split(","))}
+    assert js_unary == {k: v for k, v in L.UNARY.items() if k != "none"}
