@@ -901,6 +901,15 @@ def main() -> int:
                 pre.append({"m": m, "epilogue": f"bias+{act}", "us": round(us, 1), "tflops": round(fl / us / 1e6, 1),
                             "frac_of_f16_mfma_peak": round(fl / us / 1e6 / F16_MFMA_PEAK_TFLOPS, 4),
                             "config": list(cfg.as_tuple())})
+            if m == 2048:
+                # the chain a decoder block hands over: bias, activation, residual add ([M,N], f16)
+                res = be._alloc([m, n], "f16")
+                ep = be.makeEpilogue(bias, "silu", ("add", res))
+                us = B.median_time(B.make_call([w], x, m, out, epilogue=ep), 20)
+                pre.append({"m": m, "epilogue": "bias+silu+add[M,N]", "us": round(us, 1), "tflops": round(fl / us / 1e6, 1),
+                            "frac_of_f16_mfma_peak": round(fl / us / 1e6 / F16_MFMA_PEAK_TFLOPS, 4),
+                            "config": list(cfg.as_tuple())})
+                res.destroy()
             out.destroy()
         details["prefill_gemm_int4_4096x12288"] = pre
         # the same GEMM on f32 activations with f32 output (the reference's default

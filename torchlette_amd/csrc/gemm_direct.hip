@@ -369,29 +369,16 @@ __global__ __launch_bounds__(WM * WN * 64, (TM * TN >= 16 ? 1 : 2)) void gemm_di
 }
 
 // v[e] = ops(alpha * v[e]) for the W consecutive columns from `col` on (output elements
-// from `idx` on).
+// from `idx` on); W = 8: whole 16-byte pieces of the inputs, W = 1: one element.
 template <int W>
 __device__ __forceinline__ void apply_epilogue_scaled(const OutArgs& o, float (&v)[W], int64_t col, int64_t idx) {
 #pragma unroll
   for (int e = 0; e < W; ++e) v[e] *= o.col_scale ? o.alpha * o.col_scale[col + e] : o.alpha;
+  if constexpr (W == 8) {
+    apply_epilogue_row8(o.epi, v, col, idx, true, o.n - 1);
+  } else {
 #pragma unroll
-  for (int i = 0; i < TLHIP_MAX_EPILOGUE_OPS; ++i) {
-    if (i < o.epi.n_ops) {
-      if (o.epi.kind[i] == TLHIP_EPI_BIAS) {
-#pragma unroll
-        for (int e = 0; e < W; ++e) {
-          if (o.epi.input_dtype[i] == TLHIP_F16) v[e] += (float)((const _Float16*)o.epi.input[i])[col + e];
-          else v[e] += ((const float*)o.epi.input[i])[col + e];
-        }
-      } else if (o.epi.kind[i] == TLHIP_EPI_UNARY) {
-#pragma unroll
-        for (int e = 0; e < W; ++e) v[e] = apply_unary(o.epi.unary[i], v[e]);
-      } else if (o.epi.kind[i] != TLHIP_EPI_NONE) {
-#pragma unroll
-        for (int e = 0; e < W; ++e)
-          v[e] = apply_epilogue_step(o.epi.kind[i], o.epi.unary[i], o.epi.input[i], o.epi.input_dtype[i], v[e], col + e, idx + e);
-      }
-    }
+    for (int e = 0; e < W; ++e) v[e] = apply_epilogue(o.epi, v[e], col + e, idx + e);
   }
 }
 
