@@ -38,6 +38,7 @@
 // 14 / TM VALU instructions on dequantisation.
 #include <cstring>
 #include <type_traits>
+#include <utility>
 
 #include "gemm_common.h"
 
@@ -64,6 +65,14 @@ struct DirectArgs {
   TileMap map;
   OutArgs out;
 };
+
+// The epilogue of a wave's TM row blocks of 32 rows, one call each.
+template <int TN, bool ROW, int... I>
+__device__ __forceinline__ void epilogue_of_row_blocks(std::integer_sequence<int, I...>, float* patch,
+                                                       const float16_t (&acc)[sizeof...(I)][TN], int lane, int row0, int col0,
+                                                       const OutArgs& o, float* plane) {
+  (wave_epilogue<TN, true, ROW>(patch, acc[I], lane, row0 + I * 32, col0, o, plane), ...);
+}
 
 // WM x WN waves, each owning TM x TN MFMA tiles of 32 x 32.  G32: one scale per
 // 16-byte chunk (group size 32), the two scales of a lane's step come as one
@@ -363,9 +372,11 @@ __global__ __launch_bounds__(WM * WN * 64, (TM * TN >= 16 ? 1 : 2)) void gemm_di
   // a K slice leaves its bare partial sums, f32, row-major, in this slice's M x N plane of
   // the workspace; the reduce launch adds the planes in slice order and runs the epilogue
   float* const plane = a.ksplit > 1 ? a.workspace + (size_t)slice * a.m * a.n : nullptr;
-#pragma unroll
-  for (int i = 0; i < TM; ++i)
-    wave_epilogue<TN, true, ROW>(patch, acc[i], lane, m0 + (wm * TM + i) * 32, n0 + wn * TN * 32, a.out, plane);
+  // One call per row block, written out at compile time (a loop here is only unrolled while
+  // its unrolled size stays under the compiler's threshold; left as a loop it indexes the
+  // accumulators at run time, and they move to scratch memory for the whole kernel).
+  epilogue_of_row_blocks<TN, ROW>(std::make_integer_sequence<int, TM>{}, patch, acc, lane, m0 + wm * TM * 32, n0 + wn * TN * 32,
+                                  a.out, plane);
 }
 
 // v[e] = ops(alpha * v[e]) for the W consecutive columns from `col` on (output elements
