@@ -108,6 +108,8 @@ int launch_gemv_xreg(const Problem& p, const tlhip_kernel_config_t& c, hipStream
 // up to 4 problems that share activations, rows and shape class in one launch
 bool gemv_xreg_group_applicable(const Problem* ps, int count, const tlhip_kernel_config_t& c, const char** why);
 int launch_gemv_xreg_group(const Problem* ps, int count, const tlhip_kernel_config_t& c, hipStream_t stream);
+bool gemv_wave_config_applicable(const Problem& p, const tlhip_kernel_config_t& c, const char** why);
+int launch_gemv_wave(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t stream);
 bool gemm_config_applicable(const Problem& p, const tlhip_kernel_config_t& c, const char** why);
 int launch_gemm(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t stream);
 bool gemm_direct_config_applicable(const Problem& p, const tlhip_kernel_config_t& c, const char** why);
@@ -155,6 +157,7 @@ int prepare_all_kernels();
 int prepare_gemv_kernels();       // gemv.hip (+ the per-format units)
 int prepare_gemv_mfma_kernels();  // gemv_mfma.hip
 int prepare_gemv_xreg_kernels();  // gemv_mfma_xreg.hip
+int prepare_gemv_wave_kernels();  // gemv_wave.hip
 int prepare_gemm_kernels();       // gemm_prefill.hip
 int prepare_gemm_direct_kernels();  // gemm_direct.hip
 
@@ -164,6 +167,6 @@ void count_gemm_dispatch();
 void count_dequant_dispatch();
 void count_autotune_run();
 
-enum { VARIANT_GEMV = 0, VARIANT_GEMV_MFMA = 1, VARIANT_TILED = 2, VARIANT_TILED_DIRECT = 3, VARIANT_GEMV_XREG = 4 };
+enum { VARIANT_GEMV = 0, VARIANT_GEMV_MFMA = 1, VARIANT_TILED = 2, VARIANT_TILED_DIRECT = 3, VARIANT_GEMV_XREG = 4, VARIANT_GEMV_WAVE = 5 };
 
 }  // namespace tlhip

@@ -160,6 +160,17 @@ tlhip_kernel_config_t xreg_cfg(int waves, int unroll, int per_cu, int ks, int up
   return c;
 }
 
+tlhip_kernel_config_t wave_cfg(int waves, int depth, int per_cu, int unroll) {
+  tlhip_kernel_config_t c;
+  memset(&c, 0, sizeof c);
+  c.variant = VARIANT_GEMV_WAVE;
+  c.p0 = waves;
+  c.p1 = depth;
+  c.p2 = per_cu;
+  c.p3 = unroll;
+  return c;
+}
+
 tlhip_kernel_config_t tiled_cfg(int tm, int tn, int tk, int wm, int wn) {
   tlhip_kernel_config_t c;
   memset(&c, 0, sizeof c);
@@ -184,6 +195,7 @@ bool config_applicable(const Problem& p, const tlhip_kernel_config_t& c, const c
   if (c.variant == VARIANT_TILED) return gemm_config_applicable(p, c, why);
   if (c.variant == VARIANT_GEMV_MFMA) return gemv_mfma_config_applicable(p, c, why);
   if (c.variant == VARIANT_GEMV_XREG) return gemv_xreg_config_applicable(p, c, why);
+  if (c.variant == VARIANT_GEMV_WAVE) return gemv_wave_config_applicable(p, c, why);
   return gemv_config_applicable(p, c, why);
 }
 
@@ -464,6 +476,15 @@ std::vector<tlhip_kernel_config_t> candidates(const Problem& p) {
                 tlhip_kernel_config_t c = xreg_cfg(waves, unroll, per_cu, ks, upfront, xbar);
                 if (gemv_xreg_config_applicable(p, c, nullptr)) out.push_back(c);
               }
+    for (int waves : {4, 8})
+      for (int depth : {2, 3, 4})
+        for (int per_cu : {1, 2})
+          for (int unroll : {1, 2}) {
+            tlhip_kernel_config_t c = wave_cfg(waves, depth, per_cu, unroll);
+            if (gemv_wave_config_applicable(p, c, nullptr)) out.push_back(c);
+            c.p5 = 1;  // whole-line weight loads
+            if (gemv_wave_config_applicable(p, c, nullptr)) out.push_back(c);
+          }
   }
   if (p.x_dtype == TLHIP_F16 && p.m >= 16) {
     static const int tiles[][5] = {
@@ -575,6 +596,7 @@ int run_config(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t str
   if (c.variant == VARIANT_TILED) return launch_gemm(p, c, stream);
   if (c.variant == VARIANT_GEMV_MFMA) return launch_gemv_mfma(p, c, stream);
   if (c.variant == VARIANT_GEMV_XREG) return launch_gemv_xreg(p, c, stream);
+  if (c.variant == VARIANT_GEMV_WAVE) return launch_gemv_wave(p, c, stream);
   return launch_gemv(p, c, stream);
 }
 
@@ -799,6 +821,13 @@ std::vector<tlhip_kernel_config_t> neighbour_candidates(const Problem& p, const 
       vary(1, {1, 2, 4});
       vary(2, {1, 2, 4, 8, 16});
       vary(3, {1, 2, 4, 8});
+      vary(5, {0, 1});
+      break;
+    case VARIANT_GEMV_WAVE:
+      vary(0, {4, 8});
+      vary(1, {2, 3, 4});
+      vary(2, {1, 2});
+      vary(3, {1, 2});
       vary(5, {0, 1});
       break;
     case VARIANT_GEMV_XREG:

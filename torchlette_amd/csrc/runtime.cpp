@@ -156,6 +156,7 @@ int prepare_all_kernels() {
   int rc = prepare_gemv_kernels();
   if (!rc) rc = prepare_gemv_mfma_kernels();
   if (!rc) rc = prepare_gemv_xreg_kernels();
+  if (!rc) rc = prepare_gemv_wave_kernels();
   if (!rc) rc = prepare_gemm_kernels();
   if (!rc) rc = prepare_gemm_direct_kernels();
   t_prepare_mode = false;
