@@ -267,6 +267,52 @@ int tlhip_gemv_grouped(const tlhip_gemv_problem_t* problems, int count, int x_dt
 int tlhip_gemv_grouped_rows(const tlhip_gemv_problem_t* problems, int count, int x_dtype, int64_t m,
                             int y_dtype, float alpha, tlhip_stream_t stream);
 
+/* A SEQUENCE of decode Linears in ONE launch.  The reference issues a decoder layer's
+ * Linears one after the other, each its own dispatch, with the elementwise op of the MLP
+ * between them (packages/qwen3-browser/src/model.ts:341-361: q/k/v, o, then
+ * down(mul(silu(gate(x)), up(x))); packages/gemma2-browser/src/model.ts:411-415 with gelu);
+ * at decode sizes every launch costs as much as the weights it streams.  Here up to 16 steps
+ * run as one launch: the weight stream never stops between them, and a step whose
+ * activations (or epilogue inputs) are written by an earlier step of the call (`wait`) is
+ * ordered behind ALL earlier steps inside the kernel.  A step without `wait` must not read
+ * or write anything an earlier step of the call writes, nor write what one reads.
+ * A GATED step computes y = epilogue(x w^T) * (x w_up^T) on two weights of one shape (the
+ * MLP's act(gate) * up: the epilogue carries the activation) and writes only the product.
+ * All steps: int4 weights with group size 32, K a multiple of 256 between 2048 (3072 for
+ * M <= 8) and 12288, f16 activations, the same m <= 16; anything else is
+ * TLHIP_ERR_UNSUPPORTED (run the steps through tlhip_gemv instead).  Results are those of
+ * the same steps through tlhip_gemv (f32 accumulation of exact products: the order of the
+ * sums differs), bit-identical from launch to launch.
+ * The waits inside the kernel are bounded: if one expires (it cannot while every workgroup
+ * of the launch is resident, which the library ensures by launching one workgroup per CU)
+ * the kernel sets an error word and leaves; tlhip_sequence_status reports it.  Like a
+ * K-sliced GEMV, a stream's first sequence call must not happen under graph capture. */
+typedef struct {
+  tlhip_qweight_t w;      /* the weight; of a gated step: the gate projection */
+  tlhip_qweight_t w_up;   /* gated steps only: the up projection (same format and shape as w) */
+  const void* x;          /* device [m, K] f16 */
+  void* y;                /* device [m, N] */
+  const tlhip_epilogue_t* epilogue; /* may be NULL; gated: applied to the gate side */
+  int32_t y_dtype;        /* tlhip_dtype_t of y (f16 or f32) */
+  int32_t gated;          /* nonzero: y = epilogue(x w^T) * (x w_up^T) */
+  int32_t wait;           /* nonzero: starts only when all earlier steps of the call are complete */
+  int32_t reserved;
+} tlhip_sequence_step_t;
+int tlhip_gemv_sequence(const tlhip_sequence_step_t* steps, int count, int x_dtype, int64_t m, float alpha,
+                        tlhip_stream_t stream);
+/* The MLP block of a decoder layer as one sequence launch:
+ * h = unary(x gate^T) * (x up^T)  (f16 [m, gate.N], caller-provided),  y = epilogue(h down^T). */
+int tlhip_mlp_decode(const tlhip_qweight_t* gate, const tlhip_qweight_t* up, const tlhip_qweight_t* down, int unary,
+                     const void* x, int x_dtype, int64_t m, void* h, void* y, int y_dtype,
+                     const tlhip_epilogue_t* down_epilogue, tlhip_stream_t stream);
+/* Waits for `stream` and reports whether a sequence launch on it gave up a wait
+ * (*error != 0, return TLHIP_ERR_DEVICE; the state is cleared for the next launch). */
+int tlhip_sequence_status(tlhip_stream_t stream, int* error);
+/* Test hook: fault != 0 makes every wait of later sequence launches unsatisfiable, and
+ * spin_limit (0 = the default) bounds the polls of a wait, so that the give-up path can be
+ * exercised from the host with every workgroup still leaving normally. */
+int tlhip_debug_sequence(int fault, uint32_t spin_limit);
+
 /* Prefill GEMM with dequant fused into the LDS stage: same contract as
  * tlhip_gemv for any m >= 1; x must be f16.  Stands in for the explicit
  * dequant + stock matmul the reference runs when M > 1

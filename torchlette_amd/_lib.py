@@ -23,7 +23,7 @@ UNARY = {"none": 0, "relu": 1, "silu": 2, "gelu": 3, "gelu_tanh": 3, "gelu_erf":
 EPI_NONE, EPI_BIAS, EPI_UNARY, EPI_BINARY, EPI_CAST_F16 = 0, 1, 2, 3, 4
 BINARY = {"add": 0, "sub": 1, "mul": 2}
 MAX_EPILOGUE_OPS = 4
-VARIANT_GEMV, VARIANT_GEMV_MFMA, VARIANT_TILED, VARIANT_TILED_DIRECT, VARIANT_GEMV_XREG = 0, 1, 2, 3, 4
+VARIANT_GEMV, VARIANT_GEMV_MFMA, VARIANT_TILED, VARIANT_TILED_DIRECT, VARIANT_GEMV_XREG, VARIANT_GEMV_WAVE = 0, 1, 2, 3, 4, 5
 
 
 class TlhipError(RuntimeError):
@@ -84,6 +84,12 @@ class GemvProblem(C.Structure):
     _fields_ = [("w", QWeight), ("x", C.c_void_p), ("y", C.c_void_p), ("epilogue", C.POINTER(Epilogue))]
 
 
+class SequenceStep(C.Structure):
+    _fields_ = [("w", QWeight), ("w_up", QWeight), ("x", C.c_void_p), ("y", C.c_void_p),
+                ("epilogue", C.POINTER(Epilogue)), ("y_dtype", C.c_int32), ("gated", C.c_int32),
+                ("wait", C.c_int32), ("reserved", C.c_int32)]
+
+
 # name -> (restype, argtypes); every symbol include/tlhip.h declares.
 _vp, _i, _i64, _sz, _f = C.c_void_p, C.c_int, C.c_int64, C.c_size_t, C.c_float
 _QW, _EP, _KC = C.POINTER(QWeight), C.POINTER(Epilogue), C.POINTER(KernelConfig)
@@ -121,6 +127,10 @@ SIGNATURES = {
     "tlhip_gemv_noalloc": (_i, [_QW, _vp, _i, _i64, _vp, _i, _f, _EP, _vp]),
     "tlhip_gemv_grouped": (_i, [C.POINTER(GemvProblem), _i, _i, _i, _f, _vp]),
     "tlhip_gemv_grouped_rows": (_i, [C.POINTER(GemvProblem), _i, _i, _i64, _i, _f, _vp]),
+    "tlhip_gemv_sequence": (_i, [C.POINTER(SequenceStep), _i, _i, _i64, _f, _vp]),
+    "tlhip_mlp_decode": (_i, [_QW, _QW, _QW, _i, _vp, _i, _i64, _vp, _vp, _i, _EP, _vp]),
+    "tlhip_sequence_status": (_i, [_vp, C.POINTER(_i)]),
+    "tlhip_debug_sequence": (_i, [_i, C.c_uint32]),
     "tlhip_gemv_prologue": (_i, [_QW, C.POINTER(Prologue), _vp, _i, _i64, _vp, _i, _f, _EP, _vp]),
     "tlhip_gemv_grouped_prologue": (_i, [C.POINTER(GemvProblem), _i, C.POINTER(Prologue), _i, _i, _f, _vp]),
     "tlhip_rmsnorm": (_i, [_vp, _i, _vp, _vp, _i, _i64, _i64, _f, _vp]),

@@ -599,6 +599,76 @@ class HipBackend:
                    self.stream)
         return outs
 
+    # several Linears in one launch ------------------------------------------
+    def linearSequence(self, steps: Sequence[dict]) -> List[HipTensor]:
+        """A sequence of decode Linears as ONE launch (tlhip_gemv_sequence).  Each step is a
+        dict: ``input`` (HipTensor [m, K] f16), ``weight``, optional ``up`` (a second weight:
+        the step computes ``act(input w^T) * (input up^T)``), ``bias``, ``activation``,
+        ``binary`` ((op, tensor[m, N])), ``wait`` (the step reads what an earlier step of the
+        call writes), ``out`` (an existing tensor to write, e.g. one a later step reads).
+        Returns the outputs in order."""
+        if not 1 <= len(steps) <= 16:
+            raise ValueError("linearSequence: 1..16 steps")
+        arr = (L.SequenceStep * len(steps))()
+        outs, keep = [], []
+        m = None
+        for i, st in enumerate(steps):
+            x, w = st["input"], st["weight"]
+            qw = self._qweight(w, transposed=False)
+            if x.dtype != "f16" or not x.isContiguous or x.shape[-1] != qw.k:
+                raise ValueError("linearSequence: activations must be contiguous [m, K] f16")
+            mi = x.size // qw.k
+            if m is None:
+                m = mi
+            if mi != m or not 1 <= m <= 16:
+                raise ValueError("linearSequence: every step takes the same 1..16 rows")
+            out_dtype = "f16" if w.format.elementType == "f16" else "f32"
+            out = st.get("out")
+            if out is None:
+                out = self._alloc(list(x.shape[:-1]) + [qw.n], out_dtype)
+            elif out.size != m * qw.n or not out.isContiguous:
+                raise ValueError("linearSequence: out must be a contiguous [m, N] tensor")
+            ep = self.makeEpilogue(st.get("bias"), st.get("activation"), st.get("binary"))
+            if any(sz != m * qw.n for sz in ep._binary_sizes):
+                raise ValueError("a binary epilogue input must hold M*N elements")
+            keep.append(ep)
+            arr[i].w = qw
+            if st.get("up") is not None:
+                arr[i].w_up = self._qweight(st["up"], transposed=False)
+                arr[i].gated = 1
+            arr[i].x = x.ptr
+            arr[i].y = out.ptr
+            arr[i].epilogue = C.pointer(ep)
+            arr[i].y_dtype = _DT_CODE[out.dtype]
+            arr[i].wait = 1 if st.get("wait") else 0
+            outs.append(out)
+        L.call("tlhip_gemv_sequence", arr, len(steps), L.F16, m, 1.0, self.stream)
+        return outs
+
+    def mlpDecode(self, input: HipTensor, gate: HipTensor, up: HipTensor, down: HipTensor,
+                  activation: str = "silu") -> HipTensor:
+        """down(act(gate(x)) * up(x)) (packages/qwen3-browser/src/model.ts:357-361) as one launch."""
+        qg, qu, qd = (self._qweight(w, transposed=False) for w in (gate, up, down))
+        if input.dtype != "f16" or not input.isContiguous or input.shape[-1] != qg.k:
+            raise ValueError("mlpDecode: activations must be contiguous [m, K] f16")
+        m = input.size // qg.k
+        h = self._alloc([m, qg.n], "f16")
+        out_dtype = "f16" if down.format.elementType == "f16" else "f32"
+        y = self._alloc(list(input.shape[:-1]) + [qd.n], out_dtype)
+        act = "gelu_tanh" if activation == "gelu" else activation
+        try:
+            L.call("tlhip_mlp_decode", C.byref(qg), C.byref(qu), C.byref(qd), L.UNARY[act], input.ptr, L.F16, m, h.ptr,
+                   y.ptr, _DT_CODE[out_dtype], None, self.stream)
+        finally:
+            h.destroy()  # tlhip_free waits for the device: the launch that reads h is over by then
+        return y
+
+    def sequenceStatus(self) -> int:
+        """Waits for the stream; raises if a sequence launch gave up a wait."""
+        err = C.c_int()
+        L.call("tlhip_sequence_status", self.stream, C.byref(err))
+        return err.value
+
     # the producers of a decode Linear's input, fused into its GEMV ------------
     def _prologue(self, kind: int, operand: HipTensor, activation: str = "none", eps: float = 0.0) -> L.Prologue:
         act = "gelu_tanh" if activation == "gelu" else activation

@@ -104,10 +104,11 @@ int split_workspace(hipStream_t stream, float** workspace, int** counters) {
                        "capture: run the same call once on this stream before capturing");
     SplitWorkspace w{nullptr, nullptr, 0, true};
     TLHIP_CHECK_HIP(hipMalloc((void**)&w.workspace, kSplitWorkspaceFloats * sizeof(float)));
-    hipError_t e = hipMalloc((void**)&w.counters, kSplitCounters * sizeof(int));
+    // + 4 words behind the counters: the state of sequence launches on this stream
+    hipError_t e = hipMalloc((void**)&w.counters, (kSplitCounters + 4) * sizeof(int));
     // on the stream that will use them (not capturing: checked above), so the clear is
     // ordered in front of the first launch whatever the stream's flags are
-    if (e == hipSuccess) e = hipMemsetAsync(w.counters, 0, kSplitCounters * sizeof(int), stream);
+    if (e == hipSuccess) e = hipMemsetAsync(w.counters, 0, (kSplitCounters + 4) * sizeof(int), stream);
     if (e != hipSuccess) {
       (void)hipFree(w.workspace);
       if (w.counters) (void)hipFree(w.counters);
@@ -117,6 +118,17 @@ int split_workspace(hipStream_t stream, float** workspace, int** counters) {
   }
   *workspace = it->second.workspace;
   *counters = it->second.counters;
+  return TLHIP_OK;
+}
+
+// The device state of sequence launches on `stream` (gemv_seq.hip): four words behind the
+// stream's split-K counters, zero between launches.
+int sequence_state(hipStream_t stream, void** state) {
+  float* workspace = nullptr;
+  int* counters = nullptr;
+  const int rc = split_workspace(stream, &workspace, &counters);
+  if (rc) return rc;
+  *state = counters + kSplitCounters;
   return TLHIP_OK;
 }
 
@@ -151,12 +163,15 @@ int launch_kernel(const void* fn, dim3 grid, dim3 block, void** args, size_t lds
   return TLHIP_OK;
 }
 
+int prepare_gemv_seq_kernels();  // gemv_seq.hip
+
 int prepare_all_kernels() {
   t_prepare_mode = true;
   int rc = prepare_gemv_kernels();
   if (!rc) rc = prepare_gemv_mfma_kernels();
   if (!rc) rc = prepare_gemv_xreg_kernels();
   if (!rc) rc = prepare_gemv_wave_kernels();
+  if (!rc) rc = prepare_gemv_seq_kernels();
   if (!rc) rc = prepare_gemm_kernels();
   if (!rc) rc = prepare_gemm_direct_kernels();
   t_prepare_mode = false;
