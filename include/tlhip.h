@@ -278,8 +278,8 @@ int tlhip_gemv_grouped_rows(const tlhip_gemv_problem_t* problems, int count, int
  * or write anything an earlier step of the call writes, nor write what one reads.
  * A GATED step computes y = epilogue(x w^T) * (x w_up^T) on two weights of one shape (the
  * MLP's act(gate) * up: the epilogue carries the activation) and writes only the product.
- * All steps: int4 weights with group size 32, K a multiple of 256 between 2048 (3072 for
- * M <= 8) and 12288, f16 activations, the same m <= 16; anything else is
+ * All steps: int4 weights with group size 32, K a multiple of 256 up to 12288, f16
+ * activations, the same m <= 16; anything else is
  * TLHIP_ERR_UNSUPPORTED (run the steps through tlhip_gemv instead).  Results are those of
  * the same steps through tlhip_gemv (f32 accumulation of exact products: the order of the
  * sums differs), bit-identical from launch to launch.

@@ -35,7 +35,7 @@ def test_independent_steps_match_the_oracle_and_separate_launches(be, m):
     """Five Linears of different shapes (ragged row blocks, K of 2048..12288, one with a
     bias and an activation, one with a residual) as one launch."""
     rng = np.random.default_rng(zlib.crc32(repr(("seq", m)).encode()))
-    shapes = [(4096, 4096), (1000, 3072), (2048, 12288), (24, 4096), (5000, 3584 if m <= 8 else 2048)]
+    shapes = [(4096, 4096), (1000, 3072), (2048, 12288), (24, 4096), (5000, 3584), (13000, 1024), (20000, 256)]
     steps, wants = [], []
     for i, (n, k) in enumerate(shapes):
         w, deq = weight(be, n, k, rng)
@@ -122,9 +122,9 @@ def test_a_wait_that_cannot_be_satisfied_gives_up_and_reports(be):
 
 def test_sequence_refuses_what_it_is_not_built_for(be):
     rng = np.random.default_rng(2)
-    w, _ = weight(be, 256, 1024, rng)
-    x = be.ops.tensorFromArray(make_x(2, 1024, "f16", rng), [2, 1024], "f16")
-    with pytest.raises(L.TlhipError, match="K must be at least"):
+    w, _ = weight(be, 256, 1152, rng)
+    x = be.ops.tensorFromArray(make_x(2, 1152, "f16", rng), [2, 1152], "f16")
+    with pytest.raises(L.TlhipError, match="multiple of 256"):
         be.linearSequence([{"input": x, "weight": w}])
     w2, _ = weight(be, 256, 4096, rng)
     x2 = be.ops.tensorFromArray(make_x(2, 4096, "f16", rng), [2, 4096], "f16")

@@ -5,7 +5,7 @@
 #include "gemv_seq_kernel.h"
 
 namespace tlhip {
-int sequence_state(hipStream_t stream, void** state);  // runtime.cpp
+int sequence_state(hipStream_t stream, void** state, uint32_t** base);  // runtime.cpp
 
 namespace {
 
@@ -17,16 +17,16 @@ std::atomic<uint32_t> g_seq_spin_limit{kSeqSpinLimit};
 
 const void* seq_fn(int mq) {
   switch (mq) {
-    case 1: return (const void*)gemv_seq_kernel<1, 3>;
-    case 2: return (const void*)gemv_seq_kernel<2, 3>;
+    case 1: return (const void*)gemv_seq_kernel<1, 2>;
+    case 2: return (const void*)gemv_seq_kernel<2, 2>;
     case 4: return (const void*)gemv_seq_kernel<4, 2>;
   }
   return nullptr;
 }
-int seq_depth(int mq) { return mq == 4 ? 2 : 3; }
 
 size_t seq_lds_bytes() {
-  return (size_t)kSeqWaves * (16 * 17 + kSeqScaleLoads * 64) * 16 + (size_t)2 * kSeqWaves * kSeqSlots * 1024 + 16;
+  return (size_t)kSeqWaves * (16 * 17 + kSeqScaleLoads * 64) * 16 + (size_t)2 * kSeqWaves * kSeqSlots * 1024 + 16 +
+         sizeof(SeqProblem) * kSeqMaxProblems;
 }
 
 }  // namespace
@@ -55,7 +55,7 @@ int tlhip_gemv_sequence(const tlhip_sequence_step_t* steps, int count, int x_dty
   if (m < 1 || m > 16) return set_error(TLHIP_ERR_UNSUPPORTED, "gemv_sequence: M must be 1..16");
   int mq = 1;
   while (mq * 4 < m) mq *= 2;
-  const int depth = seq_depth(mq);
+  const int cus = device_cu_count() > 0 ? device_cu_count() : 256;
   SeqTable t;
   memset(&t, 0, sizeof t);
   t.count = count;
@@ -96,9 +96,6 @@ int tlhip_gemv_sequence(const tlhip_sequence_step_t* steps, int count, int x_dty
     P.kb = (int)(p.k / 2);
     P.nsteps = (int)(p.k / 128);
     P.steps = (P.nsteps + kSeqWaves - 1) / kSeqWaves;
-    if (P.steps < depth)
-      return set_error(TLHIP_ERR_UNSUPPORTED, "gemv_sequence: K must be at least %d (a wave's K range holds its steps in flight)",
-                       depth * kSeqWaves * 128);
     P.spr = (((P.steps & 1) ? 8 : 0) + P.steps * 8 + 15) / 16;
     if (32 * P.spr > (kSeqScaleLoads / 2) * 64)
       return set_error(TLHIP_ERR_UNSUPPORTED, "gemv_sequence: K above 12288 (the scales of a wave's K range are loaded up front)");
@@ -112,22 +109,38 @@ int tlhip_gemv_sequence(const tlhip_sequence_step_t* steps, int count, int x_dty
     P.y_dtype = s.y_dtype;
     P.alpha = alpha;
     P.epi = p.epi;
+    // Row blocks per unit: as few as still give every CU a unit (a problem of 256 row blocks
+    // on 256 CUs goes one block to a unit; more blocks per unit share the unit's activation
+    // loads), at most what the kernel's four slots hold (a gated row block takes two).
     const int64_t nblocks = (p.n + 15) / 16;
-    const int per_unit = s.gated ? 2 : 4;
+    int64_t per_unit = (nblocks + cus - 1) / cus;
+    const int64_t most = s.gated ? 2 : 4;
+    if (per_unit > most) per_unit = most;
+    P.nrb = (int)(s.gated ? 2 * per_unit : per_unit);
     units += (nblocks + per_unit - 1) / per_unit;
   }
   if (units >= ((int64_t)1 << 30)) return set_error(TLHIP_ERR_UNSUPPORTED, "gemv_sequence: too many rows");
   t.total_units = (int)units;
   t.fault = g_seq_fault.load();
+  t.counting = last_wait >= 0 ? 1 : 0;
   hipStream_t hs = resolve_stream(stream);
   void* state = nullptr;
-  int rc = sequence_state(hs, &state);
+  uint32_t* base = nullptr;  // host copy of what the stream's unit counters add up to
+  int rc = sequence_state(hs, &state, &base);
   if (rc) return rc;
   t.state = (SeqState*)state;
+  if (t.counting) {
+    // the counters' value is baked into the launch: a captured launch would replay with a stale one
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    TLHIP_CHECK_HIP(hipStreamIsCapturing(hs, &status));
+    if (status != hipStreamCaptureStatusNone)
+      return set_error(TLHIP_ERR_STATE, "gemv_sequence: a sequence with a waiting step cannot be captured into a graph");
+    t.base = *base;
+    *base += (uint32_t)units;
+  }
   t.spin_limit = g_seq_spin_limit.load();
   // Every workgroup must be resident (a unit may wait for units of other workgroups): one
   // per CU (the kernel's LDS lets no second one in), and never more than there are units.
-  const int cus = device_cu_count() > 0 ? device_cu_count() : 256;
   const int grid = (int)(units < cus ? units : cus);
   const void* fn = seq_fn(mq);
   void* args[] = {(void*)&t};
@@ -175,16 +188,18 @@ int tlhip_sequence_status(tlhip_stream_t stream, int* error) {
   if (!error) return set_error(TLHIP_ERR_INVALID, "sequence_status: null argument");
   hipStream_t hs = resolve_stream(stream);
   void* state = nullptr;
-  const int rc = sequence_state(hs, &state);
+  uint32_t* base = nullptr;
+  const int rc = sequence_state(hs, &state, &base);
   if (rc) return rc;
-  SeqState host;
-  TLHIP_CHECK_HIP(hipMemcpyAsync(&host, state, sizeof host, hipMemcpyDeviceToHost, hs));
+  uint32_t err = 0;
+  TLHIP_CHECK_HIP(hipMemcpyAsync(&err, &((SeqState*)state)->error, sizeof err, hipMemcpyDeviceToHost, hs));
   TLHIP_CHECK_HIP(hipStreamSynchronize(hs));
-  *error = (int)host.error;
-  if (host.error) {
-    // a wait expired: some workgroups left early, so the counters may not have been cleared
-    TLHIP_CHECK_HIP(hipMemsetAsync(state, 0, sizeof host, hs));
+  *error = (int)err;
+  if (err) {
+    // a wait expired: some workgroups left early, so the counters are behind the host's sum
+    TLHIP_CHECK_HIP(hipMemsetAsync(state, 0, sizeof(SeqState), hs));
     TLHIP_CHECK_HIP(hipStreamSynchronize(hs));
+    *base = 0;
     return set_error(TLHIP_ERR_DEVICE, "gemv_sequence: a wait for earlier steps of a launch expired; its results are incomplete");
   }
   return TLHIP_OK;

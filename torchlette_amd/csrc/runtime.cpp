@@ -51,6 +51,7 @@ namespace {
 struct SplitWorkspace {
   float* workspace;
   int* counters;
+  uint32_t seq_base;  // what the unit counters of the stream's sequence launches add up to
   int graphs;
   bool stream_alive;
 };
@@ -102,13 +103,13 @@ int split_workspace(hipStream_t stream, float** workspace, int** counters) {
       return set_error(TLHIP_ERR_STATE,
                        "split-K workspace of this stream does not exist yet and cannot be created during "
                        "capture: run the same call once on this stream before capturing");
-    SplitWorkspace w{nullptr, nullptr, 0, true};
+    SplitWorkspace w{nullptr, nullptr, 0, 0, true};
     TLHIP_CHECK_HIP(hipMalloc((void**)&w.workspace, kSplitWorkspaceFloats * sizeof(float)));
-    // + 4 words behind the counters: the state of sequence launches on this stream
-    hipError_t e = hipMalloc((void**)&w.counters, (kSplitCounters + 4) * sizeof(int));
+    // + 512 words behind the counters: the state of sequence launches on this stream
+    hipError_t e = hipMalloc((void**)&w.counters, (kSplitCounters + 512) * sizeof(int));
     // on the stream that will use them (not capturing: checked above), so the clear is
     // ordered in front of the first launch whatever the stream's flags are
-    if (e == hipSuccess) e = hipMemsetAsync(w.counters, 0, (kSplitCounters + 4) * sizeof(int), stream);
+    if (e == hipSuccess) e = hipMemsetAsync(w.counters, 0, (kSplitCounters + 512) * sizeof(int), stream);
     if (e != hipSuccess) {
       (void)hipFree(w.workspace);
       if (w.counters) (void)hipFree(w.counters);
@@ -121,14 +122,16 @@ int split_workspace(hipStream_t stream, float** workspace, int** counters) {
   return TLHIP_OK;
 }
 
-// The device state of sequence launches on `stream` (gemv_seq.hip): four words behind the
-// stream's split-K counters, zero between launches.
-int sequence_state(hipStream_t stream, void** state) {
+// The device state of sequence launches on `stream` (gemv_seq.hip): 512 words behind the
+// stream's split-K counters, and the host's running sum of its unit counters.
+int sequence_state(hipStream_t stream, void** state, uint32_t** base) {
   float* workspace = nullptr;
   int* counters = nullptr;
   const int rc = split_workspace(stream, &workspace, &counters);
   if (rc) return rc;
   *state = counters + kSplitCounters;
+  std::lock_guard<std::mutex> lock(g_ws_mutex);
+  *base = &g_workspaces.find(stream)->second.seq_base;  // the map's nodes do not move
   return TLHIP_OK;
 }
 
