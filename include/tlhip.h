@@ -84,14 +84,18 @@ typedef enum { TLHIP_BINARY_ADD = 0, TLHIP_BINARY_SUB = 1, TLHIP_BINARY_MUL = 2 
  * (src/backend/webgpu/matmul/types.ts:13-24).  BIAS adds input[n] (indexed by
  * output column); UNARY applies `unary`; BINARY combines the value with
  * input[m*N + n] (an [M,N] tensor, contiguous: value + input, value - input or
- * value * input; a residual add, a gate; the library sees a pointer, so that it
- * holds M*N elements is the caller's to ensure); CAST_F16 rounds the value to f16. */
+ * value * input; a residual add, a gate); CAST_F16 rounds the value to f16.
+ * The reference's op names a typed tensor (`inputIndex`); the C ABI sees a pointer, so
+ * the caller states the input's shape in `rows` ([rows, N], contiguous) and every entry
+ * point refuses, before any launch, a BIAS whose rows is not 1 and a BINARY whose rows is
+ * not the call's m (TLHIP_ERR_INVALID): the kernels index a BINARY input by output
+ * element, and a shorter buffer would be read past its end. */
 typedef struct {
   int32_t kind;        /* tlhip_epilogue_kind_t */
   int32_t unary;       /* tlhip_unary_t for kind == UNARY, tlhip_binary_t for kind == BINARY */
   const void* input;   /* device [N] for kind == BIAS, device [M,N] for kind == BINARY */
   int32_t input_dtype; /* tlhip_dtype_t of input (f32 or f16) */
-  int32_t reserved;
+  int32_t rows;        /* rows of input: 1 for BIAS, the call's m for BINARY; ignored otherwise */
 } tlhip_epilogue_op_t;
 
 /* EpilogueConfig: ops are applied in order to acc*alpha in f32, then the value
@@ -102,6 +106,9 @@ typedef struct {
   tlhip_epilogue_op_t ops[TLHIP_MAX_EPILOGUE_OPS];
 } tlhip_epilogue_t;
 
+/* The checks every compute entry point makes on (weight, m, epilogue) before it launches
+ * anything, on their own: needs no device and no tlhip_init.  TLHIP_OK or
+ * TLHIP_ERR_INVALID with the message in tlhip_last_error. */
 /* A packed weight operand: what BackendTensor.format + .scales describe
  * (src/backend/types.ts:5-28) for the logical [N,K] Linear weight.
  *   packed  u32 words, row-major [N, K/4] (int8) or [N, K/8] (int4)
@@ -124,6 +131,8 @@ typedef struct {
   const void* packed;
   const void* scales;
 } tlhip_qweight_t;
+
+int tlhip_epilogue_check(const tlhip_qweight_t* w, int64_t m, const tlhip_epilogue_t* epilogue);
 
 typedef struct {
   char name[64];     /* device name */
@@ -463,6 +472,13 @@ int tlhip_candidate_get(const tlhip_qweight_t* w, int x_dtype, int64_t m, int y_
  * dispatch.ts:171-192.  Every level is re-gated on applicability.  Where the rows
  * go in several launches (see tlhip_matmul_quantized) it is the configuration of
  * the first launch. */
+/* The whole route: `chunk_rows` rows per launch with configuration `first` (0: all rows in
+ * one launch, or the kernel's own passes) and `last` for the rows that remain.  Which route
+ * is taken between decode and prefill sizes depends on a cost model whose fitted numbers
+ * travel with the tuning cache (the "model" object of tlhip_tune_cache_export / import;
+ * tlhip_tune_cache_clear returns to the built-in values).  Needs no device. */
+int tlhip_selected_route(const tlhip_qweight_t* w, int x_dtype, int64_t m, int y_dtype, int64_t* chunk_rows,
+                         tlhip_kernel_config_t* first, tlhip_kernel_config_t* last);
 int tlhip_selected_config(const tlhip_qweight_t* w, int x_dtype, int64_t m, int y_dtype,
                           tlhip_kernel_config_t* host_out);
 

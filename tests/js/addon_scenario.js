@@ -87,6 +87,20 @@ for (const c of manifest.cases) {
     if (c.out_noalloc) {
       const out = be.ops.zeros([c.m, c.weights[0].n], "f16");
       save(c.out_noalloc, be.readSync(be.linearInto(out, x, ws[0], null, "none")));
+      // an output or a bias shorter than the shapes say is refused before anything is launched
+      r.into_errors = r.into_errors || [];
+      try {
+        be.linearInto(be.ops.zeros([Math.max(1, (x.size / ws[0].shape[1]) * ws[0].shape[0] - 1)], out.dtype), x, ws[0], null, "none");
+        r.into_errors.push(null);
+      } catch (e) {
+        r.into_errors.push(e.message);
+      }
+      try {
+        be.linearInto(out, x, ws[0], be.ops.zeros([ws[0].shape[0] - 1], "f32"), "none");
+        r.into_errors.push(null);
+      } catch (e) {
+        r.into_errors.push(e.message);
+      }
     }
   } else if (c.kind === "side_door") {
     // the fused path's call for matmul -> bias -> unary (-> cast): executor.ts:2959-3049

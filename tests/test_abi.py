@@ -2,6 +2,7 @@
 symbol include/tlhip.h declares, fails loudly without a GPU, and its host-side
 functions (f16 codec, quantizer) match the oracle bit for bit."""
 import ctypes
+import json
 import os
 import re
 
@@ -127,9 +128,10 @@ def test_tuning_cache_json_round_trip_and_autotune_toggle():
            '"512_12288_4096_int4-grouped_g32_f16_f16":[2,128,128,64,2,2,0,0]}}'
     T.importTuningCache(text)
     out = T.exportTuningCache()
-    assert out == text
+    assert out.startswith(text[:-1] + ',"model":{')      # the entries as imported, then the routing model
+    assert json.loads(out)["entries"] == json.loads(text)["entries"]
     T.clearTuningCache()
-    assert T.exportTuningCache() == '{"version":1,"entries":{}}'
+    assert json.loads(T.exportTuningCache())["entries"] == {}
     with pytest.raises(L.TlhipError, match="entries"):
         T.importTuningCache("{}")
 
@@ -141,15 +143,18 @@ def test_tuning_cache_import_survives_malformed_text():
     T.clearTuningCache()
     entries = {"1_4096_4096_int4-grouped_g32_f16_f16": [0, 64, 1, 4, 1, 0, 0, 0],
                "16_4096_12288_int4-grouped_g32_f16_f16": [1, 8, 4, 4, 2, 0, 1, 0]}
-    text = json.dumps({"version": 1, "entries": entries}, separators=(",", ":"))
+    model = {"rows_break_even": 0.5, "pass_base_us": 4.0}
+    text = json.dumps({"version": 1, "entries": entries, "model": model}, separators=(",", ":"))
+    whole_entries = text.index(',"model"')
+    empty = T.exportTuningCache()
     for cut in range(len(text)):
         try:
             T.importTuningCache(text[:cut])
-            # only a text whose entries object is whole is taken (the parser reads no further)
-            assert cut >= len(text) - 1, cut
+            # only a text whose entries object is whole is taken, and a model object only whole
+            assert cut >= len(text) - 1 or whole_entries <= cut <= whole_entries + len(',"model'), cut
             T.clearTuningCache()
         except L.TlhipError:
-            assert T.exportTuningCache() == '{"version":1,"entries":{}}', cut
+            assert T.exportTuningCache() == empty, cut   # neither entries nor model numbers were taken
     T.importTuningCache(json.dumps({"version": 1, "entries": entries}, indent=2))   # as json.dump writes it
     assert json.loads(T.exportTuningCache())["entries"] == entries
     T.clearTuningCache()
@@ -197,3 +202,76 @@ def test_enum_values_of_the_header_match_both_bindings():
     m = re.search(r"const UNARY = \{([^}]*)\};", js)
     js_unary = {k.strip(): int(v) for k, v in (item.split(":") for item in m.group(1).split(","))}
     assert js_unary == {k: v for k, v in L.UNARY.items() if k != "none"}
+
+
+def test_an_epilogue_input_of_the_wrong_shape_is_refused_before_any_launch():
+    """EpilogueOp names a typed tensor in the reference (matmul/types.ts:13-24); the C ABI
+    sees a pointer, so each step states its input's rows and the library checks them against
+    the call: a BINARY step indexes its input by output element, and an [N] tensor handed to
+    it at M > 1 would be read past its end.  The check needs no device."""
+    lib = L.load()
+    w = L.QWeight(L.FMT_INT4_GROUPED, 32, 64, 256, None, None)
+    buf = ctypes.create_string_buffer(64)  # never dereferenced: the check looks at shapes only
+    ptr = ctypes.cast(buf, ctypes.c_void_p).value
+
+    def check(m, *ops):
+        ep = L.Epilogue()
+        ep.n_ops = len(ops)
+        for i, op in enumerate(ops):
+            ep.ops[i] = L.EpilogueOp(*op)
+        return lib.tlhip_epilogue_check(ctypes.byref(w), m, ctypes.byref(ep)), L.last_error()
+
+    assert check(8, (L.EPI_BIAS, 0, ptr, L.F32, 1), (L.EPI_UNARY, L.UNARY["silu"], None, 0, 0), (L.EPI_BINARY, 0, ptr, L.F32, 8))[0] == 0
+    rc, msg = check(8, (L.EPI_BINARY, 0, ptr, L.F32, 1))       # an [N] tensor as a residual at 8 rows
+    assert rc == L.ERR_INVALID and "binary epilogue input must be [M,N] = [8,64]" in msg
+    rc, msg = check(8, (L.EPI_BINARY, 0, ptr, L.F32, 0))       # the field left at zero
+    assert rc == L.ERR_INVALID and "rows field says 0" in msg
+    rc, msg = check(1, (L.EPI_BINARY, 0, ptr, L.F32, 1))       # one row: [N] is [M,N]
+    assert rc == 0
+    rc, msg = check(8, (L.EPI_BIAS, 0, ptr, L.F32, 8))         # an [M,N] tensor as a bias
+    assert rc == L.ERR_INVALID and "bias epilogue input must be [N] = [64]" in msg
+    rc, msg = check(8, (L.EPI_BIAS, 0, ptr, L.F32, 0))
+    assert rc == L.ERR_INVALID
+
+
+def _routes(lib):
+    """The default route of a grid of problems between decode and prefill sizes."""
+    out = []
+    buf = ctypes.create_string_buffer(64)
+    ptr = ctypes.cast(buf, ctypes.c_void_p).value
+    for fmt, g in ((L.FMT_INT4_GROUPED, 32), (L.FMT_INT8_GROUPED, 64), (L.FMT_INT8_ROW, 0)):
+        for n, k in ((4096, 4096), (12288, 4096), (4096, 12288), (2048, 2048), (28672, 8192), (256000, 2304)):
+            for m in (1, 4, 9, 16, 17, 40, 64, 100, 128, 200, 256, 512, 1000, 2048):
+                w = L.QWeight(fmt, g, n, k, ptr, ptr)
+                chunk, first, last = ctypes.c_int64(), L.KernelConfig(), L.KernelConfig()
+                assert lib.tlhip_selected_route(ctypes.byref(w), L.F16, m, L.F16, ctypes.byref(chunk), ctypes.byref(first),
+                                                ctypes.byref(last)) == 0, L.last_error()
+                out.append((fmt, n, k, m, chunk.value, first.as_tuple(), last.as_tuple()))
+    return out
+
+
+def test_the_routing_model_travels_with_the_tuning_cache():
+    """The fitted numbers of the default routing are data, not code: without any tuning file
+    and with only the shipped file's model the routes agree (the file carries the built-in
+    values), the export writes the model back, and a changed number changes routes."""
+    lib = L.load()
+    shipped = json.load(open(os.path.join(os.path.dirname(T.__file__), "tuning", "mi355x.json")))
+    before = T.exportTuningCache()
+    try:
+        T.clearTuningCache()                       # what TLHIP_TUNING_FILE=none leaves: built-in model, no entries
+        builtin = _routes(lib)
+        T.importTuningCache(json.dumps({"version": 1, "entries": {}, "model": shipped["model"]}))
+        assert _routes(lib) == builtin
+        exported = json.loads(T.exportTuningCache())["model"]
+        assert exported == {k: float(v) for k, v in shipped["model"].items()}
+        assert any(chunk == 64 for (_, _, _, _, chunk, _, _) in builtin)      # some rows go 64 at a time ...
+        T.importTuningCache(json.dumps({"version": 1, "entries": {}, "model": {"rows_break_even": 1e-6, "passes_break_even": 1e-6}}))
+        changed = _routes(lib)
+        assert changed != builtin and not any(chunk == 64 for (_, _, _, _, chunk, _, _) in changed)  # ... until the model says no
+        with pytest.raises(L.TlhipError, match="unknown model field"):
+            T.importTuningCache('{"version":1,"entries":{},"model":{"no_such_number":1}}')
+        T.clearTuningCache()
+        assert _routes(lib) == builtin
+    finally:
+        T.clearTuningCache()
+        T.importTuningCache(before)

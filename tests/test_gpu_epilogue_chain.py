@@ -121,11 +121,11 @@ def test_epilogue_chain_rejects(be):
     xt = be.ops.tensorFromArray(make_x(2, 256, "f16", rng), [2, 256], "f16")
     ep = L.Epilogue()
     ep.n_ops = 1
-    ep.ops[0] = L.EpilogueOp(L.EPI_BINARY, 0, None, L.F32, 0)
+    ep.ops[0] = L.EpilogueOp(L.EPI_BINARY, 0, None, L.F32, 2)
     with pytest.raises(L.TlhipError, match="binary epilogue without input"):
         be._matmulQuantizedB(xt, be.ops.transpose(w), ep, None)
     r = be.ops.tensorFromArray(np.zeros((2, 64), np.float32), [2, 64], "f32")
-    ep.ops[0] = L.EpilogueOp(L.EPI_BINARY, 7, r.ptr, L.F32, 0)
+    ep.ops[0] = L.EpilogueOp(L.EPI_BINARY, 7, r.ptr, L.F32, 2)
     with pytest.raises(L.TlhipError, match="unknown binary epilogue op"):
         be._matmulQuantizedB(xt, be.ops.transpose(w), ep, None)
     ep.ops[0] = L.EpilogueOp(9, 0, None, 0, 0)

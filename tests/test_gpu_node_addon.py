@@ -222,6 +222,10 @@ def test_grouped_launch_of_a_batched_step_and_the_no_alloc_entry_point(run):
         assert rel_l2(run["get"](f"g8_{i}.y").reshape(want.shape), want) <= 1e-3
     want = run["want"]["grouped8_0"]
     assert rel_l2(run["get"]("g8.noalloc").reshape(want.shape), want) <= 1e-3
+    # linearInto writes a buffer of the caller's: one that is too short, or a bias that is,
+    # is refused before anything is launched
+    errors = run["results"]["cases"]["grouped8"]["into_errors"]
+    assert len(errors) == 2 and "out must be a contiguous tensor of at least" in errors[0] and "bias must hold N" in errors[1]
 
 
 def test_topk(run):

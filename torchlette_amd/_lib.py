@@ -34,7 +34,7 @@ class TlhipError(RuntimeError):
 
 class EpilogueOp(C.Structure):
     _fields_ = [("kind", C.c_int32), ("unary", C.c_int32), ("input", C.c_void_p),
-                ("input_dtype", C.c_int32), ("reserved", C.c_int32)]
+                ("input_dtype", C.c_int32), ("rows", C.c_int32)]
 
 
 class Epilogue(C.Structure):
@@ -122,6 +122,7 @@ SIGNATURES = {
     "tlhip_f16_bits_to_f32": (_f, [C.c_uint16]),
     "tlhip_quantize_int8_grouped_device": (_i, [_vp, _i64, _i64, _i64, _vp, _vp, _vp]),
     "tlhip_quantize_int8_grouped": (_i, [_vp, _i64, _i64, _i64, _vp, _vp]),
+    "tlhip_epilogue_check": (_i, [_QW, _i64, _EP]),
     "tlhip_dequant": (_i, [_QW, _vp, _vp]),
     "tlhip_gemv": (_i, [_QW, _vp, _i, _i64, _vp, _i, _f, _EP, _vp]),
     "tlhip_gemv_noalloc": (_i, [_QW, _vp, _i, _i64, _vp, _i, _f, _EP, _vp]),
@@ -146,6 +147,7 @@ SIGNATURES = {
     "tlhip_candidate_count": (_i, [_QW, _i, _i64, _i, C.POINTER(_i)]),
     "tlhip_candidate_get": (_i, [_QW, _i, _i64, _i, _i, _KC]),
     "tlhip_selected_config": (_i, [_QW, _i, _i64, _i, _KC]),
+    "tlhip_selected_route": (_i, [_QW, _i, _i64, _i, C.POINTER(_i64), _KC, _KC]),
     "tlhip_set_autotune_enabled": (_i, [_i]),
     "tlhip_is_autotune_enabled": (_i, []),
     "tlhip_autotune": (_i, [_QW, _vp, _i, _i64, _vp, _i, C.POINTER(C.c_double)]),

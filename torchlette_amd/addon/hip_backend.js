@@ -497,7 +497,15 @@ class HipBackend {
    *  device memory (tlhip_gemv_noalloc; `out` is the caller's): for code under graph capture. */
   linearInto(out, input, weight, bias, activation) {
     const wa = this._weightArgs(weight, false);
-    const m = input.size / wa[3];
+    const n = wa[2], k = wa[3];
+    const m = input.size / k;
+    // `out` and `bias` are the caller's buffers and the kernel sees only pointers: anything
+    // shorter than the shapes say would be read or written past its end, so refuse it here
+    if (!Number.isInteger(m) || m < 1 || m > 16) throw new Error("linearInto: 1..16 activation rows");
+    if (!(input.dtype in DT) || !input.isContiguous) throw new Error("linearInto: activations must be contiguous f32 or f16");
+    if (!(out.dtype in DT) || !out.isContiguous || out.nbytes < m * n * (out.dtype === "f16" ? 2 : 4))
+      throw new Error(`linearInto: out must be a contiguous tensor of at least [${m},${n}] ${out.dtype} elements`);
+    if (bias && (!(bias.dtype in DT) || !bias.isContiguous || bias.size !== n)) throw new Error(`linearInto: bias must hold N = ${n} elements`);
     const act = UNARY[activation === "gelu" ? "gelu_tanh" : activation || "none"];
     tl.gemvNoalloc.apply(null, wa.concat([input.ptr, DT[input.dtype], m, out.ptr, DT[out.dtype], bias ? bias.ptr : null,
                                           bias ? DT[bias.dtype] : 0, act]));

@@ -29,10 +29,12 @@ function lowerEpilogue(epilogue, epilogueInputs, outputDtype, m, n) {
       const t = epilogueInputs[op.inputIndex];
       if (!t) throw new Error(`hip dispatchMatmul: epilogue input ${op.inputIndex} missing`);
       if (!(t.dtype in DT)) throw new Error(`hip dispatchMatmul: bias dtype ${t.dtype}`);
-      ops.push([EPI_BIAS, 0, t.ptr, DT[t.dtype]]);
+      const biasCount = t.size !== undefined ? t.size : t.nbytes / (t.dtype === "f16" ? 2 : 4);
+      if (biasCount !== n) throw new Error(`hip dispatchMatmul: a bias epilogue input must hold N = ${n} elements`);
+      ops.push([EPI_BIAS, 0, t.ptr, DT[t.dtype], 1]);
     } else if (op.kind === "unary") {
       if (!(op.op in UNARY)) throw new Error(`hip dispatchMatmul: unary epilogue op ${op.op} is not built`);
-      ops.push([EPI_UNARY, UNARY[op.op], null, 0]);
+      ops.push([EPI_UNARY, UNARY[op.op], null, 0, 0]);
     } else if (op.kind === "binary") {
       const t = epilogueInputs[op.inputIndex];
       if (!t) throw new Error(`hip dispatchMatmul: epilogue input ${op.inputIndex} missing`);
@@ -42,12 +44,12 @@ function lowerEpilogue(epilogue, epilogueInputs, outputDtype, m, n) {
       const count = t.size !== undefined ? t.size : t.nbytes / (t.dtype === "f16" ? 2 : 4);
       if (count !== m * n || !t.isContiguous)
         throw new Error(`hip dispatchMatmul: a binary epilogue input must be a contiguous [M,N] = [${m},${n}] tensor`);
-      ops.push([EPI_BINARY, BINARY[op.op], t.ptr, DT[t.dtype]]);
+      ops.push([EPI_BINARY, BINARY[op.op], t.ptr, DT[t.dtype], m]);
     } else if (op.kind === "cast") {
       if (i === list.length - 1) {
         if (op.toDtype !== outputDtype) throw new Error("hip dispatchMatmul: the cast that closes the chain must name the output dtype");
       } else if (op.toDtype === "f16") {
-        ops.push([EPI_CAST_F16, 0, null, 0]);
+        ops.push([EPI_CAST_F16, 0, null, 0, 0]);
       }  // a cast to f32 in the chain changes nothing: the chain computes in f32
     } else {
       throw new Error(`hip dispatchMatmul: epilogue op kind ${op.kind} is not built`);

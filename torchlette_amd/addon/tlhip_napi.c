@@ -147,6 +147,7 @@ static void make_epilogue(void* bias, int32_t bias_dtype, int32_t unary, tlhip_e
     ep->ops[ep->n_ops].kind = TLHIP_EPI_BIAS;
     ep->ops[ep->n_ops].input = bias;
     ep->ops[ep->n_ops].input_dtype = bias_dtype;
+    ep->ops[ep->n_ops].rows = 1;
     ep->n_ops++;
   }
   if (unary) {
@@ -363,7 +364,7 @@ static napi_value MatmulQuantized(napi_env env, napi_callback_info info) {
   return undefined(env);
 }
 /* matmulQuantizedOps(format, groupSize, n, k, packed, scales, xPtr, xDtype, m, yPtr, yDtype,
- *                    [[kind, unary, inputPtr | null, inputDtype], ...])
+ *                    [[kind, unary, inputPtr | null, inputDtype, inputRows], ...])
  * An epilogue chain of up to TLHIP_MAX_EPILOGUE_OPS steps in the caller's order: the
  * EpilogueConfig.ops of the fused path (src/backend/webgpu/matmul/types.ts:13-24). */
 static napi_value MatmulQuantizedOps(napi_env env, napi_callback_info info) {
@@ -382,21 +383,23 @@ static napi_value MatmulQuantizedOps(napi_env env, napi_callback_info info) {
   tlhip_epilogue_t ep;
   memset(&ep, 0, sizeof ep);
   for (uint32_t i = 0; i < count; ++i) {
-    napi_value row, f[4];
+    napi_value row, f[5];
     uint32_t len = 0;
     napi_get_element(env, a[11], i, &row);
-    if (napi_is_array(env, row, &is_array) != napi_ok || !is_array) return throw_type(env, "tlhip: an op is [kind, unary, input, inputDtype]");
+    if (napi_is_array(env, row, &is_array) != napi_ok || !is_array) return throw_type(env, "tlhip: an op is [kind, unary, input, inputDtype, inputRows]");
     napi_get_array_length(env, row, &len);
-    if (len != 4) return throw_type(env, "tlhip: an op is [kind, unary, input, inputDtype]");
-    for (uint32_t j = 0; j < 4; ++j) napi_get_element(env, row, j, &f[j]);
-    int32_t kind, unary, idt;
+    if (len != 5) return throw_type(env, "tlhip: an op is [kind, unary, input, inputDtype, inputRows]");
+    for (uint32_t j = 0; j < 5; ++j) napi_get_element(env, row, j, &f[j]);
+    int32_t kind, unary, idt, rows;
     void* input;
-    if (!get_i32(env, f[0], &kind) || !get_i32(env, f[1], &unary) || !get_ptr(env, f[2], &input) || !get_i32(env, f[3], &idt))
-      return throw_type(env, "tlhip: an op is [kind, unary, input, inputDtype]");
+    if (!get_i32(env, f[0], &kind) || !get_i32(env, f[1], &unary) || !get_ptr(env, f[2], &input) || !get_i32(env, f[3], &idt) ||
+        !get_i32(env, f[4], &rows))
+      return throw_type(env, "tlhip: an op is [kind, unary, input, inputDtype, inputRows]");
     ep.ops[i].kind = kind;
     ep.ops[i].unary = unary;
     ep.ops[i].input = input;
     ep.ops[i].input_dtype = idt;
+    ep.ops[i].rows = rows;
   }
   ep.n_ops = (int32_t)count;
   CHECK(tlhip_matmul_quantized(&w, x, xd, m, y, yd, 1.0f, count ? &ep : NULL, NULL));

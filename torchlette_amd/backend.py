@@ -528,7 +528,7 @@ class HipBackend:
         binary_sizes = []   # checked against M * N at the call: the kernels index these inputs by output element
         for i, op in enumerate(ops):
             if op[0] == "bias":
-                ep.ops[i] = L.EpilogueOp(L.EPI_BIAS, 0, op[1].ptr, _DT_CODE[op[1].dtype], 0)
+                ep.ops[i] = L.EpilogueOp(L.EPI_BIAS, 0, op[1].ptr, _DT_CODE[op[1].dtype], 1 if len(op[1].shape) <= 1 else op[1].size // op[1].shape[-1])
             elif op[0] == "unary":
                 ep.ops[i] = L.EpilogueOp(L.EPI_UNARY, L.UNARY[op[1]], None, 0, 0)
             elif op[0] == "binary":
@@ -536,7 +536,8 @@ class HipBackend:
                     raise ValueError(f"Unsupported binary epilogue: {op[1]}")
                 if not op[2].isContiguous:
                     raise ValueError("a binary epilogue input must be contiguous")
-                ep.ops[i] = L.EpilogueOp(L.EPI_BINARY, L.BINARY[op[1]], op[2].ptr, _DT_CODE[op[2].dtype], 0)
+                ep.ops[i] = L.EpilogueOp(L.EPI_BINARY, L.BINARY[op[1]], op[2].ptr, _DT_CODE[op[2].dtype],
+                                         op[2].size // op[2].shape[-1] if op[2].shape and op[2].shape[-1] else 0)
                 binary_sizes.append(op[2].size)
             elif op[0] == "cast":
                 ep.ops[i] = L.EpilogueOp(L.EPI_CAST_F16 if op[1] == "f16" else L.EPI_NONE, 0, None, 0, 0)

@@ -201,14 +201,57 @@ bool config_applicable(const Problem& p, const tlhip_kernel_config_t& c, const c
 
 tlhip_kernel_config_t default_valu_config(const Problem& p);
 
+// The numbers the default routing was fitted with on MI355X: measurements, not structure.
+// They live next to the tuned entries: the tuning file may carry a "model" object that
+// overrides any of them by name (tlhip_tune_cache_import), the export writes them back,
+// and tlhip_tune_cache_clear returns to the built-in values below.
+struct RouteModel {
+  double walk_direct_us = 42.0;      // a workgroup of the direct GEMM walks 4096 of K in this time
+  double walk_staged128_us = 52.0;   // ... of the staged GEMM's 128-row tile
+  double walk_staged64_us = 42.0;    // ... of its 64-row tile
+  double reduce_base_us = 6.0;       // the launch that adds K slices: base
+  double reduce_us_per_mb = 0.6;     // ... per MB of f32 planes
+  double crowd_base = 0.45;          // rounds of a crowded launch: base + slope x (workgroups / CUs)
+  double crowd_slope = 0.78;
+  double pass_base_us = 3.0;         // a 16-row pass of the decode kernel: base
+  double pass_mb_per_us = 3.2;       // ... plus packed MB / this
+  double rows32_factor = 1.5;        // 17..32 rows in one launch of the decode kernel, in 16-row passes
+  double rows64_factor = 2.7;        // 33..64 rows
+  double rows_break_even = 0.9;      // rows through the decode kernel while below this x the tiled time
+  double passes_break_even = 0.8;    // 16-row passes while below this x the tiled time
+  double resident_tiles = 512.0;     // 128 x 128 tiles that run at once
+  double int4_256_rounds = 2.0;      // int4: 256 x 256 tiles from this many per CU on
+  double int4_128x256_tiles = 160.0; // int4: 128 x 256 tiles from this many on
+  double int8_256_fill = 0.5625;     // int8: 256 x 256 tiles once they are this fraction of the CUs
+  double int8_256x128_fill = 0.625;  // int8: 256 x 128 tiles likewise
+  double int8_row_fill = 0.58;       // int8 direct kernel only if the rows fill this much of their 256-row tiles
+};
+RouteModel g_model;
+struct ModelField {
+  const char* name;
+  double RouteModel::*field;
+};
+const ModelField kModelFields[] = {
+    {"walk_direct_us", &RouteModel::walk_direct_us},       {"walk_staged128_us", &RouteModel::walk_staged128_us},
+    {"walk_staged64_us", &RouteModel::walk_staged64_us},   {"reduce_base_us", &RouteModel::reduce_base_us},
+    {"reduce_us_per_mb", &RouteModel::reduce_us_per_mb},   {"crowd_base", &RouteModel::crowd_base},
+    {"crowd_slope", &RouteModel::crowd_slope},             {"pass_base_us", &RouteModel::pass_base_us},
+    {"pass_mb_per_us", &RouteModel::pass_mb_per_us},       {"rows32_factor", &RouteModel::rows32_factor},
+    {"rows64_factor", &RouteModel::rows64_factor},         {"rows_break_even", &RouteModel::rows_break_even},
+    {"passes_break_even", &RouteModel::passes_break_even}, {"resident_tiles", &RouteModel::resident_tiles},
+    {"int4_256_rounds", &RouteModel::int4_256_rounds},     {"int4_128x256_tiles", &RouteModel::int4_128x256_tiles},
+    {"int8_256_fill", &RouteModel::int8_256_fill},         {"int8_256x128_fill", &RouteModel::int8_256x128_fill},
+    {"int8_row_fill", &RouteModel::int8_row_fill},
+};
+
 // Time of one round of 128 x 128 tiles of the direct GEMM with `ks` K slices across
 // workgroups, in microseconds: a workgroup walks 4096 of K in 42 us; the slices' partial
 // sums (ks planes of M x N f32) are written and read back by a second launch, 6 us plus
 // 0.6 us per MB of planes (fitted at 4096..12288 x 4096..12288, M = 64..512).
-double direct_round_us(const Problem& p, int ks, double walk_4096_us = 42.0) {
+double direct_round_us(const Problem& p, int ks, double walk_4096_us) {
   const double walk = walk_4096_us * (double)p.k / 4096.0 / ks;
   if (ks <= 1) return walk;
-  return walk + 6.0 + 0.6 * (double)ks * (double)p.m * (double)p.n * 4.0 / 1e6;
+  return walk + g_model.reduce_base_us + g_model.reduce_us_per_mb * (double)ks * (double)p.m * (double)p.n * 4.0 / 1e6;
 }
 
 // Time of a launch of the staged GEMM's 128 x 128 or 64 x 128 tiles by the same model, in
@@ -221,8 +264,8 @@ double staged_launch_us(const Problem& p, const tlhip_kernel_config_t& c) {
   const int ks = c.p5 > 1 ? c.p5 : 1;
   const int64_t tiles = ((p.m + c.p0 - 1) / c.p0) * ((p.n + c.p1 - 1) / c.p1);
   const double fill = (double)(tiles * ks) / (double)cus;
-  const double rounds = fill <= 1.0 ? 1.0 : 0.45 + 0.78 * fill;
-  const double walk_us = (c.p0 <= 64 ? 42.0 : 52.0) * (double)p.k / 4096.0 / ks;
+  const double rounds = fill <= 1.0 ? 1.0 : g_model.crowd_base + g_model.crowd_slope * fill;
+  const double walk_us = (c.p0 <= 64 ? g_model.walk_staged64_us : g_model.walk_staged128_us) * (double)p.k / 4096.0 / ks;
   const double sum_us = direct_round_us(p, ks, 0.0);  // the second launch of a K-sliced one
   return rounds * walk_us + sum_us;
 }
@@ -237,7 +280,7 @@ int direct_k_split(const Problem& p) {
   const int64_t steps = p.k / 128;
   int best = 1;
   for (int ks = 2; ks <= 8; ks *= 2)
-    if (tiles * ks <= cus && steps % ks == 0 && steps / ks >= 4 && direct_round_us(p, ks) < direct_round_us(p, best)) best = ks;
+    if (tiles * ks <= cus && steps % ks == 0 && steps / ks >= 4 && direct_round_us(p, ks, g_model.walk_direct_us) < direct_round_us(p, best, g_model.walk_direct_us)) best = ks;
   return best;
 }
 
@@ -254,8 +297,9 @@ tlhip_kernel_config_t default_config(const Problem& p) {
     if (p.format == TLHIP_FMT_INT4_GROUPED) {
       const int64_t t256 = ((p.m + 255) / 256) * ((p.n + 255) / 256);
       const int64_t t128x256 = ((p.m + 127) / 128) * ((p.n + 255) / 256);
-      tlhip_kernel_config_t c = t256 >= 2 * cus ? direct_cfg(256, 256, 2, 4)
-                                : (t128x256 >= 160 ? direct_cfg(128, 256, 1, 4) : direct_cfg(128, 128, 2, 2));
+      tlhip_kernel_config_t c = (double)t256 >= g_model.int4_256_rounds * cus
+                                    ? direct_cfg(256, 256, 2, 4)
+                                    : ((double)t128x256 >= g_model.int4_128x256_tiles ? direct_cfg(128, 256, 1, 4) : direct_cfg(128, 128, 2, 2));
       if (c.p0 == 128 && c.p1 == 128) {
         // few 128 x 128 tiles: 2, 4 or 8 workgroups share a tile, each walking a slice of K
         // of at least four steps (4096 x 12288 at M = 256: 48 us against 141 us)
@@ -275,13 +319,13 @@ tlhip_kernel_config_t default_config(const Problem& p) {
     // tiles the staged kernel below is ahead by 3-40 %.  Not where the rows fill less than
     // 58 % of their 256-row tiles (128 rows on 28672 columns: 78 us against 52 us).
     if ((p.format == TLHIP_FMT_INT8_GROUPED || p.format == TLHIP_FMT_INT8_ROW) &&
-        p.m * 100 >= ((p.m + 255) / 256) * 256 * 58) {
+        (double)p.m >= (double)(((p.m + 255) / 256) * 256) * g_model.int8_row_fill) {
       const int64_t t256 = ((p.m + 255) / 256) * ((p.n + 255) / 256);
       const int64_t t256x128 = ((p.m + 255) / 256) * ((p.n + 127) / 128);
-      if (t256 * 16 >= (int64_t)cus * 9) {
+      if ((double)t256 >= g_model.int8_256_fill * cus) {
         const tlhip_kernel_config_t c = direct_cfg(256, 256, 2, 4);
         if (gemm_direct_config_applicable(p, c, nullptr)) return c;
-      } else if (t256x128 * 8 >= (int64_t)cus * 5) {
+      } else if ((double)t256x128 >= g_model.int8_256x128_fill * cus) {
         const tlhip_kernel_config_t c = direct_cfg(256, 128, 2, 4);
         if (gemm_direct_config_applicable(p, c, nullptr)) return c;
       }
@@ -734,20 +778,23 @@ Route plan_route(const Problem& p, const tlhip_kernel_config_t& c) {
   if ((c.variant == VARIANT_TILED || c.variant == VARIANT_TILED_DIRECT) && p.m > 16 && p.x_dtype == TLHIP_F16 &&
       !has_tuned_entry(p)) {
     const double packed_mb = (double)p.n * (double)p.k * (p.format == TLHIP_FMT_INT4_GROUPED ? 0.5 : 1.0) / 1e6;
-    const double pass_us = 3.0 + packed_mb / 3.2;
+    const double pass_us = g_model.pass_base_us + packed_mb / g_model.pass_mb_per_us;
     const int64_t passes = (p.m + 15) / 16;
     const int64_t tiles = ((p.m + 127) / 128) * ((p.n + 127) / 128);
-    const double rounds = tiles <= 512 ? 1.0 : (double)tiles / 512.0;
+    const double rounds = (double)tiles <= g_model.resident_tiles ? 1.0 : (double)tiles / g_model.resident_tiles;
     const double tiled_us =
-        direct_round_us(p, c.p5 > 1 ? c.p5 : 1, c.variant == VARIANT_TILED_DIRECT ? 42.0 : (c.p0 <= 64 ? 42.0 : 52.0)) * rounds;
+        direct_round_us(p, c.p5 > 1 ? c.p5 : 1,
+                        c.variant == VARIANT_TILED_DIRECT ? g_model.walk_direct_us
+                                                          : (c.p0 <= 64 ? g_model.walk_staged64_us : g_model.walk_staged128_us)) *
+        rounds;
     // Up to 64 rows per launch of the decode kernel: 1.2-1.6 times a 16-row pass for two
     // tiles of rows, 2.3-3.2 times for four (the activations a workgroup stages grow with
     // the rows, and their K slices are combined across workgroups).  More rows go 64 at a
     // time while that beats the tiles (128 rows at 4096 x 4096: 2 x 16 us against 49 us).
-    auto chunk_us = [&](int64_t rows) { return pass_us * (rows <= 16 ? 1.0 : (rows <= 32 ? 1.5 : 2.7)); };
+    auto chunk_us = [&](int64_t rows) { return pass_us * (rows <= 16 ? 1.0 : (rows <= 32 ? g_model.rows32_factor : g_model.rows64_factor)); };
     const int64_t full = p.m / 64, rest = p.m % 64;
     const double rows_us = (double)full * chunk_us(64) + (rest ? chunk_us(rest) : 0.0);
-    if (rows_us < 0.9 * tiled_us) {
+    if (rows_us < g_model.rows_break_even * tiled_us) {
       bool ok = true;
       Route q{64, c, c};
       Problem q64 = p, qr = p;
@@ -762,7 +809,7 @@ Route plan_route(const Problem& p, const tlhip_kernel_config_t& c) {
       if (!full) q.first = q.last;
       if (ok) return q;
     }
-    if ((double)passes * pass_us < 0.8 * tiled_us) {
+    if ((double)passes * pass_us < g_model.passes_break_even * tiled_us) {
       Problem q = p;
       q.m = 16;
       const tlhip_kernel_config_t c16 = select_gemv_config(q);
@@ -1041,6 +1088,16 @@ tlhip_kernel_config_t select_gemv_config(const Problem& p) {
 
 int run_kernel_config(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t stream) { return run_config(p, c, stream); }
 
+// What tlhip_gemv runs for `p` (the selected configuration and its route: one launch, rows
+// in chunks, or passes), for an entry point that brings its own scratch in p.scratch; and
+// the most K slices any launch of that route takes (1: the route needs no scratch).
+int run_gemv_route(const Problem& p, hipStream_t stream) { return run_selected(p, select_gemv_config(p), stream); }
+int gemv_route_k_slices(const Problem& p) {
+  const Route r = plan_route(p, select_gemv_config(p));
+  const int first = config_k_slices(r.first);
+  return r.chunk == 0 ? first : std::max(first, config_k_slices(r.last));
+}
+
 // The tuning file that ships next to the library: <directory of libtlhip.so>/tuning/
 // mi355x.json, or the file TLHIP_TUNING_FILE names ("none" = load nothing).  Called by
 // tlhip_init, so every binding gets the committed winners, not only the benchmark.
@@ -1112,6 +1169,39 @@ int validate_weight(const tlhip_qweight_t* w, const char* who) {
   return TLHIP_OK;
 }
 
+// The epilogue of a call with m activation rows on weight w: kinds, ops, types, and that
+// every input has the shape its step indexes it by.
+int check_epilogue(const tlhip_qweight_t* w, int64_t m, const tlhip_epilogue_t* epilogue, const char* who) {
+  if (epilogue->n_ops < 0 || epilogue->n_ops > TLHIP_MAX_EPILOGUE_OPS)
+    return set_error(TLHIP_ERR_INVALID, "%s: epilogue has %d ops (max %d)", who, epilogue->n_ops, TLHIP_MAX_EPILOGUE_OPS);
+  for (int i = 0; i < epilogue->n_ops; ++i) {
+    const tlhip_epilogue_op_t& op = epilogue->ops[i];
+    if (op.kind < TLHIP_EPI_NONE || op.kind > TLHIP_EPI_CAST_F16)
+      return set_error(TLHIP_ERR_INVALID, "%s: unknown epilogue op kind %d", who, op.kind);
+    if (op.kind == TLHIP_EPI_BINARY) {
+      if (!op.input && w->n > 0 && m > 0) return set_error(TLHIP_ERR_INVALID, "%s: binary epilogue without input", who);
+      if (op.input_dtype != TLHIP_F32 && op.input_dtype != TLHIP_F16)
+        return set_error(TLHIP_ERR_INVALID, "%s: bad binary epilogue input dtype %d", who, op.input_dtype);
+      if (op.unary < TLHIP_BINARY_ADD || op.unary > TLHIP_BINARY_MUL)
+        return set_error(TLHIP_ERR_INVALID, "%s: unknown binary epilogue op %d (add, sub, mul)", who, op.unary);
+      if ((int64_t)op.rows != m)
+        return set_error(TLHIP_ERR_INVALID, "%s: a binary epilogue input must be [M,N] = [%lld,%lld]; its rows field says %d", who,
+                         (long long)m, (long long)w->n, op.rows);
+    }
+    if (op.kind == TLHIP_EPI_BIAS) {
+      if (!op.input && w->n > 0) return set_error(TLHIP_ERR_INVALID, "%s: bias epilogue without input", who);
+      if (op.input_dtype != TLHIP_F32 && op.input_dtype != TLHIP_F16)
+        return set_error(TLHIP_ERR_INVALID, "%s: bad bias dtype %d", who, op.input_dtype);
+      if (op.rows != 1)
+        return set_error(TLHIP_ERR_INVALID, "%s: a bias epilogue input must be [N] = [%lld]; its rows field says %d", who,
+                         (long long)w->n, op.rows);
+    }
+    if (op.kind == TLHIP_EPI_UNARY && (op.unary < TLHIP_UNARY_NONE || op.unary > TLHIP_UNARY_TANH))
+      return set_error(TLHIP_ERR_INVALID, "%s: unknown unary op %d", who, op.unary);
+  }
+  return TLHIP_OK;
+}
+
 int make_problem(const tlhip_qweight_t* w, const void* x, int x_dtype, int64_t m, void* y, int y_dtype,
                  float alpha, const tlhip_epilogue_t* epilogue, Problem* p, const char* who) {
   int rc = validate_weight(w, who);
@@ -1138,28 +1228,11 @@ int make_problem(const tlhip_qweight_t* w, const void* x, int x_dtype, int64_t m
   memset(&p->pro, 0, sizeof p->pro);
   p->scratch = nullptr;
   if (epilogue) {
-    if (epilogue->n_ops < 0 || epilogue->n_ops > TLHIP_MAX_EPILOGUE_OPS)
-      return set_error(TLHIP_ERR_INVALID, "%s: epilogue has %d ops (max %d)", who, epilogue->n_ops,
-                       TLHIP_MAX_EPILOGUE_OPS);
+    const int rc = check_epilogue(w, m, epilogue, who);
+    if (rc) return rc;
     p->epi.n_ops = epilogue->n_ops;
     for (int i = 0; i < epilogue->n_ops; ++i) {
       const tlhip_epilogue_op_t& op = epilogue->ops[i];
-      if (op.kind < TLHIP_EPI_NONE || op.kind > TLHIP_EPI_CAST_F16)
-        return set_error(TLHIP_ERR_INVALID, "%s: unknown epilogue op kind %d", who, op.kind);
-      if (op.kind == TLHIP_EPI_BINARY) {
-        if (!op.input && w->n > 0 && m > 0) return set_error(TLHIP_ERR_INVALID, "%s: binary epilogue without input", who);
-        if (op.input_dtype != TLHIP_F32 && op.input_dtype != TLHIP_F16)
-          return set_error(TLHIP_ERR_INVALID, "%s: bad binary epilogue input dtype %d", who, op.input_dtype);
-        if (op.unary < TLHIP_BINARY_ADD || op.unary > TLHIP_BINARY_MUL)
-          return set_error(TLHIP_ERR_INVALID, "%s: unknown binary epilogue op %d (add, sub, mul)", who, op.unary);
-      }
-      if (op.kind == TLHIP_EPI_BIAS) {
-        if (!op.input && w->n > 0) return set_error(TLHIP_ERR_INVALID, "%s: bias epilogue without input", who);
-        if (op.input_dtype != TLHIP_F32 && op.input_dtype != TLHIP_F16)
-          return set_error(TLHIP_ERR_INVALID, "%s: bad bias dtype %d", who, op.input_dtype);
-      }
-      if (op.kind == TLHIP_EPI_UNARY && (op.unary < TLHIP_UNARY_NONE || op.unary > TLHIP_UNARY_TANH))
-        return set_error(TLHIP_ERR_INVALID, "%s: unknown unary op %d", who, op.unary);
       p->epi.kind[i] = op.kind;
       p->epi.unary[i] = op.unary;
       p->epi.input[i] = op.input;
@@ -1174,6 +1247,13 @@ int make_problem(const tlhip_qweight_t* w, const void* x, int x_dtype, int64_t m
 using namespace tlhip;
 
 extern "C" {
+
+int tlhip_epilogue_check(const tlhip_qweight_t* w, int64_t m, const tlhip_epilogue_t* epilogue) {
+  clear_error();
+  if (!w) return set_error(TLHIP_ERR_INVALID, "epilogue_check: null weight");
+  if (m < 0) return set_error(TLHIP_ERR_INVALID, "epilogue_check: negative m");
+  return epilogue ? check_epilogue(w, m, epilogue, "epilogue_check") : TLHIP_OK;
+}
 
 int tlhip_dequant(const tlhip_qweight_t* w, float* out, tlhip_stream_t stream) {
   TLHIP_REQUIRE_INIT();
@@ -1412,6 +1492,19 @@ int tlhip_candidate_get(const tlhip_qweight_t* w, int x_dtype, int64_t m, int y_
   return TLHIP_OK;
 }
 
+int tlhip_selected_route(const tlhip_qweight_t* w, int x_dtype, int64_t m, int y_dtype, int64_t* chunk_rows,
+                         tlhip_kernel_config_t* first, tlhip_kernel_config_t* last) {
+  Problem p;
+  const int rc = shape_problem(w, x_dtype, m, y_dtype, &p);
+  if (rc) return rc;
+  if (!chunk_rows || !first || !last) return set_error(TLHIP_ERR_INVALID, "selected_route: null output");
+  const Route r = plan_route(p, select_config(p));
+  *chunk_rows = r.chunk;
+  *first = r.first;
+  *last = r.last;
+  return TLHIP_OK;
+}
+
 int tlhip_selected_config(const tlhip_qweight_t* w, int x_dtype, int64_t m, int y_dtype,
                           tlhip_kernel_config_t* out) {
   Problem p;
@@ -1512,6 +1605,9 @@ int tlhip_tune_cache_export(char* buf, size_t cap, size_t* needed) {
          << "," << c.p4 << "," << c.p5 << "," << c.p6 << "]";
     }
   }
+  os << "},\"model\":{";
+  for (size_t i = 0; i < sizeof kModelFields / sizeof kModelFields[0]; ++i)
+    os << (i ? "," : "") << "\"" << kModelFields[i].name << "\":" << g_model.*(kModelFields[i].field);
   os << "}}";
   const std::string s = os.str();
   if (needed) *needed = s.size() + 1;
@@ -1555,7 +1651,34 @@ int tlhip_tune_cache_import(const char* json) {
     tlhip_kernel_config_t c = {v[0], v[1], v[2], v[3], v[4], v[5], v[6], v[7]};
     parsed[key] = c;
   }
+  // an optional "model" object: name : number pairs that override the routing model
+  RouteModel model = g_model;
+  if (const char* mp = strstr(json, "\"model\"")) {
+    mp = strchr(mp, '{');
+    if (!mp) return set_error(TLHIP_ERR_INVALID, "tune_cache_import: malformed model");
+    ++mp;
+    for (;;) {
+      while (*mp == ' ' || *mp == '\n' || *mp == '\t' || *mp == ',' || *mp == '\r') ++mp;
+      if (*mp == '}') break;
+      if (*mp != '"') return set_error(TLHIP_ERR_INVALID, "tune_cache_import: expected a model field name");
+      const char* ke = strchr(mp + 1, '"');
+      if (!ke) return set_error(TLHIP_ERR_INVALID, "tune_cache_import: unterminated model field name");
+      const std::string name(mp + 1, ke);
+      mp = strchr(ke, ':');
+      if (!mp) return set_error(TLHIP_ERR_INVALID, "tune_cache_import: expected a value for model field %s", name.c_str());
+      char* end = nullptr;
+      const double v = strtod(mp + 1, &end);
+      if (end == mp + 1 || !(v > 0.0) || v > 1e9)
+        return set_error(TLHIP_ERR_INVALID, "tune_cache_import: model field %s needs a positive number", name.c_str());
+      mp = end;
+      bool known = false;
+      for (const ModelField& f : kModelFields)
+        if (name == f.name) model.*(f.field) = v, known = true;
+      if (!known) return set_error(TLHIP_ERR_INVALID, "tune_cache_import: unknown model field %s", name.c_str());
+    }
+  }
   std::lock_guard<std::mutex> lock(g_tune_mutex);
+  g_model = model;
   for (auto& kv : parsed) {
     Problem q;
     if (parse_problem_key(kv.first, &q)) record_winner_locked(q, kv.second);  // the shape-class level too
@@ -1569,6 +1692,7 @@ int tlhip_tune_cache_clear(void) {
   g_tuned.clear();
   g_class_tuned.clear();
   g_shape_hints.clear();
+  g_model = RouteModel();
   return TLHIP_OK;
 }
 

@@ -16,6 +16,8 @@
 #include "device_utils.h"
 
 namespace tlhip {
+int run_gemv_route(const Problem& p, hipStream_t stream);  // dispatch.cpp
+int gemv_route_k_slices(const Problem& p);
 namespace {
 
 // Partial 16 x 16 f32 tiles, [row block][K slice][256], then one arrival counter per
@@ -70,9 +72,10 @@ extern "C" int tlhip_gemv_noalloc(const tlhip_qweight_t* w, const void* x, int x
                      dev, device_index());
   if (dev < 0 || dev >= kMaxDevices || !g_scratch_ptr[dev])
     return set_error(TLHIP_ERR_STATE, "gemv_noalloc: the scratch of device %d was not set up by tlhip_init", dev);
-  // the kernel and configuration tlhip_gemv would run for this problem
-  const tlhip_kernel_config_t c = select_gemv_config(p);
-  const int ks = config_k_slices(c);
+  // the configuration and the route (one launch, or the rows in chunks) tlhip_gemv would
+  // take for this problem, selected exactly as it selects them; every launch of the route
+  // combines its K slices through the fixed array, one launch after the other
+  const int ks = gemv_route_k_slices(p);
   hipStream_t s = resolve_stream(stream);
   SplitScratch sc;
   sc.tiles = (float*)g_scratch_ptr[dev];
@@ -95,5 +98,5 @@ extern "C" int tlhip_gemv_noalloc(const tlhip_qweight_t* w, const void* x, int x
     TLHIP_CHECK_HIP(hipGetLastError());
   }
   p.scratch = &sc;
-  return run_kernel_config(p, c, s);
+  return run_gemv_route(p, s);
 }
