@@ -76,6 +76,8 @@ class Bench:
         L.call("tlhip_event_create", C.byref(self.ev0))
         L.call("tlhip_event_create", C.byref(self.ev1))
         self.sink = self.be._alloc([4], "u32")
+        self.probe = None
+        self.probe_stream = None
 
     # -------------------------------------------------------------- operands
     def weight_pool(self, fmt: str, n: int, k: int, g: int, element: str, pool_bytes: float = POOL_BYTES):
@@ -115,14 +117,14 @@ class Bench:
         return self.be.ops.tensorFromArray(host, [m, k], dtype), host
 
     # ---------------------------------------------------------------- timing
-    def time_region(self, enqueue, reps: int) -> float:
-        """Microseconds per repetition of `enqueue()` (which launches on the
-        library stream), between two events recorded on that stream."""
+    def time_region(self, enqueue, reps: int, stream=None) -> float:
+        """Microseconds per repetition of `enqueue()` (which launches on `stream`;
+        None = the library's stream), between two events recorded on that stream."""
         L = self.L
-        L.call("tlhip_event_record", self.ev0, None)
+        L.call("tlhip_event_record", self.ev0, stream)
         for _ in range(reps):
             enqueue()
-        L.call("tlhip_event_record", self.ev1, None)
+        L.call("tlhip_event_record", self.ev1, stream)
         L.call("tlhip_event_synchronize", self.ev1)
         us = C.c_double()
         L.call("tlhip_event_elapsed_us", self.ev0, self.ev1, C.byref(us))
@@ -130,14 +132,14 @@ class Bench:
 
     warm_ms = 50.0
 
-    def median_time(self, enqueue, reps: int, batches: int = 5) -> float:
+    def median_time(self, enqueue, reps: int, batches: int = 5, stream=None) -> float:
         # untimed batches first, `warm_ms` of GPU time: the section before may have left the
         # GPU idle while the host prepared data, and the launches after that run at a lower
         # clock for some milliseconds (the same kernel measured 8-12 % slower without)
         spent = 0.0
         while spent < self.warm_ms * 1e3:
-            spent += self.time_region(enqueue, reps) * reps
-        return float(np.median([self.time_region(enqueue, reps) for _ in range(batches)]))
+            spent += self.time_region(enqueue, reps, stream) * reps
+        return float(np.median([self.time_region(enqueue, reps, stream) for _ in range(batches)]))
 
     def make_call(self, pool, x, m: int, out, epilogue=None, out_dtype: str = "f16"):
         L, be = self.L, self.be
@@ -157,14 +159,28 @@ class Bench:
         return call
 
     def probe_time(self, pool, nbytes: int) -> float:
-        L = self.L
+        """The read-only streaming kernel of the benchmark's own library over `nbytes` of
+        each pool buffer in turn, timed like the GEMV launches (on a stream of its own:
+        the library's stream is not visible through the C ABI)."""
+        if self.probe is None:
+            path = os.path.join(ROOT, "torchlette_amd", "libtlhip_bench.so")
+            if not os.path.exists(path):
+                raise RuntimeError(f"{path} is missing: build it with make -C torchlette_amd/csrc")
+            self.probe = C.CDLL(path).tlbench_hbm_read_probe
+            self.probe.restype = C.c_int
+            self.probe.argtypes = [C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p]
+            self.probe_stream = C.c_void_p()
+            self.L.call("tlhip_stream_create", C.byref(self.probe_stream))
         state = {"i": 0}
 
         def call():
             w = pool[state["i"] % len(pool)]
             state["i"] += 1
-            L.call("tlhip_hbm_read_probe", w.ptr, nbytes, self.sink.ptr, None)
-        return self.median_time(call, 100)
+            rc = self.probe(w.ptr, nbytes, self.sink.ptr, self.probe_stream)
+            if rc:
+                raise RuntimeError(f"tlbench_hbm_read_probe failed with code {rc}")
+        self.be.synchronize()
+        return self.median_time(call, 100, stream=self.probe_stream)
 
     def tune(self, pool, x, m: int, out, out_dtype: str = "f16", epilogue=None):
         """The library's tuner (tlhip_autotune_pool) over this pool: every candidate is
@@ -644,8 +660,46 @@ def main() -> int:
             us_sep = B.median_time(runner(sep), 40)
             us_grp = B.median_time(runner(grp), 40)
             us_gu = B.median_time(gate_up, 100)
+            # the MLP block (gate, up, act(gate) * up, down): one sequence launch
+            # (tlhip_mlp_decode, dependent steps ordered inside the kernel) beside the three
+            # launches it replaces (gate/up grouped, the gated multiply, down)
+            hbuf = be._alloc([m, 12288], "f16")
+            mlp_q = [(be._qweight(p124[(2 * li) % len(p124)], False), be._qweight(p124[(2 * li + 1) % len(p124)], False),
+                      be._qweight(p412[li % len(p412)], False)) for li in range(nlayers)]
+            mlp_fn, gm_fn = L.load().tlhip_mlp_decode, L.load().tlhip_gated_mul
+
+            def mlp_one_launch():
+                qg, qu, qd = mlp_q[state["i"] % nlayers]
+                state["i"] += 1
+                rc = mlp_fn(C.byref(qg), C.byref(qu), C.byref(qd), L.UNARY["silu"], x4.ptr, L.F16, m, hbuf.ptr, y["down"].ptr,
+                            L.F16, None, None)
+                if rc:
+                    L.check(rc)
+            down_only = [probs_of([(p412[li % len(p412)], hbuf, y["down"])]) for li in range(nlayers)]
+
+            def mlp_three_launches():
+                i = state["i"] % nlayers
+                state["i"] += 1
+                arr, cnt = gu_only[i]
+                rc = gfn(arr, cnt, L.F16, m, L.F16, 1.0, None)
+                rc = rc or gm_fn(L.UNARY["silu"], y["gate"].ptr, y["up"].ptr, L.F16, hbuf.ptr, m * 12288, None)
+                arr, cnt = down_only[i]
+                rc = rc or gfn(arr, cnt, L.F16, m, L.F16, 1.0, None)
+                if rc:
+                    L.check(rc)
+            mlp_bytes = gu_bytes + algorithmic_bytes("int4", 4096, 12288, 32, m, 2, 2)
+            us_mlp1 = B.median_time(mlp_one_launch, 40)
+            us_mlp3 = B.median_time(mlp_three_launches, 40)
+            err = C.c_int(0)
+            L.call("tlhip_sequence_status", None, C.byref(err))
+            hbuf.destroy()
             layer_rows.append({
-                "m": m, "bytes": layer_bytes, "us_7_launches": round(us_sep, 2), "us_4_launches": round(us_grp, 2),
+                "m": m, "bytes": layer_bytes,
+                "mlp_block": {"bytes": mlp_bytes, "us_one_sequence_launch": round(us_mlp1, 2),
+                              "us_three_launches": round(us_mlp3, 2),
+                              "gbps_one_sequence_launch": round(mlp_bytes / us_mlp1 / 1e3, 1),
+                              "gbps_three_launches": round(mlp_bytes / us_mlp3 / 1e3, 1),
+                              "note": "tlhip_mlp_decode vs grouped gate/up + tlhip_gated_mul + down"}, "us_7_launches": round(us_sep, 2), "us_4_launches": round(us_grp, 2),
                 "gbps_4_launches": round(layer_bytes / us_grp / 1e3, 1),
                 "frac_of_peak_4_launches": round(layer_bytes / us_grp / 1e3 / HBM_PEAK_GBPS, 4),
                 "gate_up_grouped_us": round(us_gu, 2), "gate_up_grouped_gbps": round(gu_bytes / us_gu / 1e3, 1),

@@ -399,12 +399,6 @@ int tlhip_gemv_grouped_prologue(const tlhip_gemv_problem_t* problems, int count,
                                 const tlhip_prologue_t* prologue, int x_dtype, int y_dtype, float alpha,
                                 tlhip_stream_t stream);
 
-/* Measuring stick for the decode GEMV (no counterpart in the reference): reads
- * `bytes` bytes at `ptr` once with 16-byte loads and discards them.  Timed like
- * a GEMV launch of the same size, it gives the rate a single launch of that size
- * can reach at all.  `sink4` is 4 writable device bytes. */
-int tlhip_hbm_read_probe(const void* ptr, size_t bytes, void* sink4, tlhip_stream_t stream);
-
 /* Top-k of logits[offset .. offset+length) (f32, device): the k largest values in
  * descending order, ties towards the smaller index, NaN below every number;
  * out_values f32[k], out_indices [k] relative to `offset`, as TLHIP_I32 or (the

@@ -102,6 +102,17 @@ for (const c of manifest.cases) {
         r.into_errors.push(e.message);
       }
     }
+  } else if (c.kind === "mlp") {
+    // the MLP block of a decode step as one call and one launch
+    const x = tensor(be, c.x, [c.m, c.k], "f16");
+    const [gate, up, down] = c.weights.map((wc) => weightOf(be, Object.assign({ format: c.format, element: "f16" }, wc)));
+    const g0 = H.getQuantGemvDispatchCount();
+    const y = be.mlpDecode(x, gate, up, down, c.act);
+    r.dispatches = H.getQuantGemvDispatchCount() - g0;
+    r.shape = y.shape;
+    r.dtype = y.dtype;
+    save(c.out, be.readSync(y));
+    r.status = be.sequenceStatus();
   } else if (c.kind === "side_door") {
     // the fused path's call for matmul -> bias -> unary (-> cast): executor.ts:2959-3049
     const w = weightOf(be, c);

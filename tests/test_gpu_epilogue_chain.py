@@ -114,6 +114,27 @@ def test_epilogue_chain_f16_output(be):
     assert got.dtype == np.float16 and rel_l2(got, want) <= 1e-3
 
 
+@pytest.mark.parametrize("chain", range(len(CHAINS)))
+@pytest.mark.parametrize("ydt", ["f32", "f16"])
+def test_a_binary_step_on_a_large_output_runs_behind_the_gemm(be, chain, ydt):
+    """From 4 M output elements on the chain is cut at its first binary step: the GEMM runs
+    the steps before it, one elementwise launch the rest, in place.  Same results as the
+    unfused sequence (an f16 output is rounded once more in between), and as the chain
+    inside the GEMM, which an explicit kernel config still runs."""
+    m, n, k = 1024, 4096, 256
+    got, want = run_chain(be, "int4-grouped", 32, m, n, k, CHAINS[chain], ydt=ydt, seed=40 + chain)
+    assert got.shape == (m, n) and got.dtype == (np.float16 if ydt == "f16" else np.float32)
+    assert rel_l2(got, want) <= 1e-3, rel_l2(got, want)
+    fused, _ = run_chain(be, "int4-grouped", 32, m, n, k, CHAINS[chain], ydt=ydt, seed=40 + chain, config=(3, 128, 128, 128, 2, 2))
+    assert rel_l2(got, fused) <= (1e-3 if ydt == "f16" else 2e-6), rel_l2(got, fused)
+
+
+def test_a_binary_step_stays_in_the_gemm_where_the_tail_cannot_run(be):
+    """N not a multiple of 8: no 16-byte pieces of a row, the chain stays in the GEMM."""
+    got, want = run_chain(be, "int4-grouped", 32, 1100, 4004, 256, CHAINS[0], seed=7)
+    assert rel_l2(got, want) <= 1e-3, rel_l2(got, want)
+
+
 def test_epilogue_chain_rejects(be):
     rng = np.random.default_rng(1)
     packed, scales, _ = make_weight("int4-grouped", 64, 256, 32, rng)

@@ -117,6 +117,21 @@ def run(tmp_path_factory):
     cases.append({"kind": "grouped", "name": "grouped8", "format": "int4-32", "k": k, "m": 8,
                   "x": put("g8.x", x8.astype(np.float32)), "weights": gw8, "out_noalloc": "g8.noalloc"})
 
+    # the MLP block of a decode step through the one-launch entry point
+    rng = seeded("addon", "mlp")
+    k, ff, m = 512, 1536, 4
+    x = make_x(m, k, "f16", rng)
+    mw, deqs = [], []
+    for i, (n_, k_) in enumerate(((ff, k), (ff, k), (k, ff))):
+        packed, scales, deq = make_weight("int4-grouped", n_, k_, 32, rng)
+        mw.append({"n": n_, "k": k_, "packed": put(f"mlp{i}.packed", packed), "scales": put(f"mlp{i}.scales", scales)})
+        deqs.append(deq)
+    cases.append({"kind": "mlp", "name": "mlp", "format": "int4-32", "k": k, "m": m, "act": "silu",
+                  "x": put("mlp.x", x.astype(np.float32)), "weights": mw, "out": "mlp.y"})
+    xf = x.astype(np.float32)
+    hidden = O.gated(O.linear(xf, deqs[0]), O.linear(xf, deqs[1]), "silu")
+    want["mlp"] = (O.linear(f16_round(hidden).astype(np.float32), deqs[2]), (m, k))
+
     for name, m, xdt, out_dtype in (("door_m1", 1, "f32", "f32"), ("door_m64", 64, "f16", "f16")):
         rng = seeded("addon", name)
         n, k, g = 768, 1024, 32
@@ -226,6 +241,14 @@ def test_grouped_launch_of_a_batched_step_and_the_no_alloc_entry_point(run):
     # is refused before anything is launched
     errors = run["results"]["cases"]["grouped8"]["into_errors"]
     assert len(errors) == 2 and "out must be a contiguous tensor of at least" in errors[0] and "bias must hold N" in errors[1]
+
+
+def test_mlp_block_in_one_call(run):
+    """mlpDecode: gate, up, silu(gate) * up and down as one launch (counted as its two steps)."""
+    want, shape = run["want"]["mlp"]
+    r = run["results"]["cases"]["mlp"]
+    assert tuple(r["shape"]) == shape and r["dtype"] == "f16" and r["dispatches"] == 2 and r["status"] == 0
+    assert rel_l2(run["get"]("mlp.y").reshape(shape), want) <= 1e-3
 
 
 def test_topk(run):

@@ -143,7 +143,6 @@ SIGNATURES = {
     "tlhip_unary": (_i, [_i, _vp, _i, _vp, _i64, _vp]),
     "tlhip_cast": (_i, [_vp, _i, _vp, _i, _i64, _vp]),
     "tlhip_topk": (_i, [_vp, _i64, _i64, _i, _vp, _vp, _i, _vp]),
-    "tlhip_hbm_read_probe": (_i, [_vp, _sz, _vp, _vp]),
     "tlhip_candidate_count": (_i, [_QW, _i, _i64, _i, C.POINTER(_i)]),
     "tlhip_candidate_get": (_i, [_QW, _i, _i64, _i, _i, _KC]),
     "tlhip_selected_config": (_i, [_QW, _i, _i64, _i, _KC]),

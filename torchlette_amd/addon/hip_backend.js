@@ -489,6 +489,36 @@ class HipBackend {
     return out;
   }
 
+  /** down(mul(gateActivation(gate(input)), up(input))) of a decode step's MLP block
+   *  (packages/qwen3-browser/src/model.ts:357-361) as ONE launch: int4 g32 weights, f16
+   *  activations, 1..16 rows.  One call from the host instead of three. */
+  mlpDecode(input, gate, up, down, gateActivation) {
+    const ga = this._weightArgs(gate, false), ua = this._weightArgs(up, false), da = this._weightArgs(down, false);
+    const k = ga[3], ff = ga[2];
+    if (input.dtype !== "f16" || !input.isContiguous || input.shape[input.shape.length - 1] !== k)
+      throw new Error("mlpDecode: activations must be contiguous f16 [..., K]");
+    const m = input.size / k;
+    if (!Number.isInteger(m) || m < 1 || m > 16) throw new Error("mlpDecode: 1..16 activation rows");
+    if (ua[2] !== ff || ua[3] !== k || da[3] !== ff) throw new Error("mlpDecode: gate and up are [F,K], down is [N,F]");
+    const outDtype = down.format.elementType === "f16" ? "f16" : "f32";
+    const h = this._alloc([m, ff], "f16");
+    const out = this._alloc(input.shape.slice(0, -1).concat([da[2]]), outDtype);
+    try {
+      tl.mlpDecode(ga, ua, da, UNARY[gateActivation === "gelu" ? "gelu_tanh" : gateActivation || "silu"], input.ptr, DT.f16, m, h.ptr, out.ptr, DT[outDtype]);
+    } catch (e) {
+      out.destroy();
+      throw e;
+    } finally {
+      h.destroy();  // hipFree waits for the launch
+    }
+    return out;
+  }
+
+  /** Waits for the stream; 0, or throws if a sequence launch (mlpDecode) gave up a wait. */
+  sequenceStatus() {
+    return tl.sequenceStatus();
+  }
+
   linearGroupedAfterRMSNorm(input, normWeight, eps, weights, biases, activation) {
     return this.linearGrouped(input, weights, biases, activation, { kind: PRO_RMSNORM, operand: normWeight.ptr, unary: 0, eps });
   }

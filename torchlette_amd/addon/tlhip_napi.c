@@ -532,6 +532,41 @@ static napi_value GemvNoalloc(napi_env env, napi_callback_info info) {
   CHECK(tlhip_gemv_noalloc(&w, x, xd, m, y, yd, 1.0f, ep.n_ops ? &ep : NULL, NULL));
   return undefined(env);
 }
+/* [format, groupSize, n, k, packed, scales] as one array argument. */
+static int get_weight_array(napi_env env, napi_value arr, tlhip_qweight_t* w) {
+  bool is_array = false;
+  uint32_t len = 0;
+  napi_value f[6];
+  if (napi_is_array(env, arr, &is_array) != napi_ok || !is_array) return 0;
+  napi_get_array_length(env, arr, &len);
+  if (len != 6) return 0;
+  for (uint32_t j = 0; j < 6; ++j) napi_get_element(env, arr, j, &f[j]);
+  return get_weight(env, f, w);
+}
+/* mlpDecode(gate, up, down (each [format, groupSize, n, k, packed, scales]), unary, xPtr, xDtype, m, hPtr, yPtr, yDtype):
+ * y = (unary(x gate^T) * (x up^T)) down^T in one launch; h is the caller's f16 [m, gate.n] */
+static napi_value MlpDecode(napi_env env, napi_callback_info info) {
+  ARGS(10);
+  tlhip_qweight_t gate, up, down;
+  if (!get_weight_array(env, a[0], &gate) || !get_weight_array(env, a[1], &up) || !get_weight_array(env, a[2], &down))
+    return throw_type(env, "tlhip: mlpDecode takes three weights as [format, groupSize, n, k, packed, scales]");
+  I32(3, un);
+  PTR(4, x);
+  I32(5, xd);
+  I64(6, m);
+  PTR(7, h);
+  PTR(8, y);
+  I32(9, yd);
+  CHECK(tlhip_mlp_decode(&gate, &up, &down, un, x, xd, m, h, y, yd, NULL, NULL));
+  return undefined(env);
+}
+/* sequenceStatus(): waits for the library stream; throws if a sequence launch gave up a wait */
+static napi_value SequenceStatus(napi_env env, napi_callback_info info) {
+  (void)info;
+  int error = 0;
+  CHECK(tlhip_sequence_status(NULL, &error));
+  return make_num(env, (double)error);
+}
 /* biasAdd(inPtr, dtype, biasPtr, biasDtype, outPtr, m, n) */
 static napi_value BiasAdd(napi_env env, napi_callback_info info) {
   ARGS(7);
@@ -762,7 +797,7 @@ NAPI_MODULE_INIT() {
       FN("f32ToF16Bits", F32ToF16Bits), FN("f16BitsToF32", F16BitsToF32),
       FN("quantizeInt8Grouped", QuantizeInt8Grouped), FN("quantizeInt8GroupedDevice", QuantizeInt8GroupedDevice),
       FN("dequant", Dequant), FN("matmulQuantized", MatmulQuantized), FN("matmulQuantizedOps", MatmulQuantizedOps), FN("gemvPrologue", GemvPrologue),
-      FN("gemvGrouped", GemvGrouped), FN("gemvGroupedRows", GemvGroupedRows), FN("gemvNoalloc", GemvNoalloc), FN("biasAdd", BiasAdd), FN("unary", Unary), FN("cast", Cast),
+      FN("gemvGrouped", GemvGrouped), FN("gemvGroupedRows", GemvGroupedRows), FN("gemvNoalloc", GemvNoalloc), FN("mlpDecode", MlpDecode), FN("sequenceStatus", SequenceStatus), FN("biasAdd", BiasAdd), FN("unary", Unary), FN("cast", Cast),
       FN("rmsnorm", RmsNorm), FN("gatedMul", GatedMul), FN("topk", TopK), FN("selectedConfig", SelectedConfig),
       FN("candidates", Candidates), FN("autotune", Autotune), FN("tuneCacheSeed", TuneCacheSeed),
       FN("setAutotuneEnabled", SetAutotuneEnabled), FN("isAutotuneEnabled", IsAutotuneEnabled),

@@ -4,10 +4,17 @@
 // same back-to-back launches as the GEMV, it shows how much of the 8 TB/s peak a
 // single launch of a given size can reach at all once launch overhead and the
 // ramp of the memory pipeline are paid.
-#include "device_utils.h"
+//
+// A benchmark instrument, not part of the product: built into its own shared
+// object (libtlhip_bench.so), which only the benchmark loads.
+#include <hip/hip_runtime.h>
 
-namespace tlhip {
+#include <cstddef>
+#include <cstdint>
+
 namespace {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 __global__ __launch_bounds__(256) void hbm_read_probe_kernel(const u32x4* __restrict__ p, size_t n16,
                                                             uint32_t* __restrict__ sink) {
@@ -22,21 +29,21 @@ __global__ __launch_bounds__(256) void hbm_read_probe_kernel(const u32x4* __rest
 }
 
 }  // namespace
-}  // namespace tlhip
 
-using namespace tlhip;
-
-extern "C" int tlhip_hbm_read_probe(const void* ptr, size_t bytes, void* sink4, tlhip_stream_t stream) {
-  TLHIP_REQUIRE_INIT();
-  if (!ptr || !sink4) return set_error(TLHIP_ERR_INVALID, "hbm_read_probe: null pointer");
-  if (((uintptr_t)ptr & 15) != 0) return set_error(TLHIP_ERR_INVALID, "hbm_read_probe: pointer must be 16-byte aligned");
+// Reads `bytes` bytes at `ptr` (device, 16-byte aligned) once on `stream` (a hipStream_t;
+// null = the default stream) and discards them; `sink4` is 4 writable device bytes.
+// Returns 0, -1 for bad arguments, or the HIP error code of the launch.
+extern "C" int tlbench_hbm_read_probe(const void* ptr, size_t bytes, void* sink4, void* stream) {
+  if (!ptr || !sink4 || ((uintptr_t)ptr & 15) != 0) return -1;
   const size_t n16 = bytes / 16;
-  if (n16 == 0) return TLHIP_OK;
+  if (n16 == 0) return 0;
+  int dev = 0, cus = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return -1;
+  if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) return -1;
   const size_t blocks = (n16 + 255) / 256;
-  const size_t cap = (size_t)device_cu_count() * 8;  // 8 workgroups of 4 waves per CU: the best measured shape
+  const size_t cap = (size_t)cus * 8;  // 8 workgroups of 4 waves per CU: the best measured shape
   const int grid = (int)(blocks < cap ? blocks : cap);
-  hipLaunchKernelGGL(hbm_read_probe_kernel, dim3(grid), dim3(256), 0, resolve_stream(stream), (const u32x4*)ptr, n16,
+  hipLaunchKernelGGL(hbm_read_probe_kernel, dim3(grid), dim3(256), 0, (hipStream_t)stream, (const u32x4*)ptr, n16,
                      (uint32_t*)sink4);
-  TLHIP_CHECK_HIP(hipGetLastError());
-  return TLHIP_OK;
+  return (int)hipGetLastError();
 }

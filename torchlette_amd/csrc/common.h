@@ -110,6 +110,9 @@ bool gemv_xreg_group_applicable(const Problem* ps, int count, const tlhip_kernel
 int launch_gemv_xreg_group(const Problem* ps, int count, const tlhip_kernel_config_t& c, hipStream_t stream);
 bool gemv_wave_config_applicable(const Problem& p, const tlhip_kernel_config_t& c, const char** why);
 int launch_gemv_wave(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t stream);
+// elementwise.hip: the steps of `ep` over a finished [M,N] output, in place, 8 columns a lane
+bool epilogue_tail_applicable(const void* y, int64_t n);
+int launch_epilogue_tail(void* y, int y_dtype, int64_t m, int64_t n, const DevEpilogue& ep, hipStream_t stream);
 bool gemm_config_applicable(const Problem& p, const tlhip_kernel_config_t& c, const char** why);
 int launch_gemm(const Problem& p, const tlhip_kernel_config_t& c, hipStream_t stream);
 bool gemm_direct_config_applicable(const Problem& p, const tlhip_kernel_config_t& c, const char** why);

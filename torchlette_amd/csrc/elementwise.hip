@@ -69,6 +69,41 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const XT* __restrict__ x, 
   for (int64_t i = threadIdx.x; i < d; i += 256) yr[i] = (YT)(((float)xr[i] * inv) * weight[i]);
 }
 
+// The rest of an epilogue chain over a finished [M,N] output, in place: a lane takes 8
+// consecutive columns of a row (N is a multiple of 8), the output and the steps' inputs in
+// 16-byte pieces.
+template <typename T>
+__global__ __launch_bounds__(256) void epilogue_tail_kernel(T* __restrict__ y, int64_t groups, int64_t n, const DevEpilogue ep) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < groups; t += stride) {
+    const int64_t idx = t * 8;
+    const int64_t col = idx % n;
+    float v[8];
+    if constexpr (sizeof(T) == 2) {
+      const half8_t h = *(const half8_t*)(y + idx);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] = (float)h[e];
+    } else {
+      const float4_t lo = *(const float4_t*)(y + idx), hi = *(const float4_t*)(y + idx + 4);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        v[e] = lo[e];
+        v[4 + e] = hi[e];
+      }
+    }
+    apply_epilogue_row8(ep, v, col, idx, true, n - 1);
+    if constexpr (sizeof(T) == 2) {
+      half8_t h;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) h[e] = (_Float16)v[e];
+      *(half8_t*)(y + idx) = h;
+    } else {
+      *(float4_t*)(y + idx) = (float4_t){v[0], v[1], v[2], v[3]};
+      *(float4_t*)(y + idx + 4) = (float4_t){v[4], v[5], v[6], v[7]};
+    }
+  }
+}
+
 int grid_for(int64_t count) {
   const int64_t blocks = (count + 255) / 256;
   const int64_t cap = (int64_t)device_cu_count() * 16;
@@ -76,6 +111,22 @@ int grid_for(int64_t count) {
 }
 
 }  // namespace
+
+bool epilogue_tail_applicable(const void* y, int64_t n) { return n > 0 && n % 8 == 0 && ((uintptr_t)y & 15) == 0; }
+
+int launch_epilogue_tail(void* y, int y_dtype, int64_t m, int64_t n, const DevEpilogue& ep, hipStream_t stream) {
+  if (!epilogue_tail_applicable(y, n)) return set_error(TLHIP_ERR_INVALID, "epilogue tail: N must be a multiple of 8 and the output 16-byte aligned");
+  const int64_t groups = m * n / 8;
+  if (groups == 0 || ep.n_ops == 0) return TLHIP_OK;
+  const int grid = grid_for(groups);
+  if (y_dtype == TLHIP_F16)
+    hipLaunchKernelGGL(epilogue_tail_kernel<_Float16>, dim3(grid), dim3(256), 0, stream, (_Float16*)y, groups, n, ep);
+  else
+    hipLaunchKernelGGL(epilogue_tail_kernel<float>, dim3(grid), dim3(256), 0, stream, (float*)y, groups, n, ep);
+  TLHIP_CHECK_HIP(hipGetLastError());
+  return TLHIP_OK;
+}
+
 }  // namespace tlhip
 
 using namespace tlhip;

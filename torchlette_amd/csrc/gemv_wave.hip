@@ -118,8 +118,8 @@ bool gemv_wave_config_applicable(const Problem& p, const tlhip_kernel_config_t& 
   if (p.m < 1 || p.m > 16) return fail(2);
   const int per_cu = c.p2 < 1 ? 1 : c.p2;
   const int unroll = c.p3 < 1 ? 1 : c.p3;
-  if ((c.p0 != 4 && c.p0 != 8) || c.p1 < 2 || c.p1 > 4 || (per_cu != 1 && per_cu != 2) || unroll > 2 || (c.p5 != 0 && c.p5 != 1) ||
-      (c.p5 == 1 && unroll != 2))
+  if ((c.p0 != 4 && c.p0 != 8) || c.p1 < 2 || c.p1 > 4 || (per_cu != 1 && per_cu != 2) || unroll > 2 || c.p4 != 0 ||
+      (c.p5 != 0 && c.p5 != 1) || (c.p5 == 1 && unroll != 2) || c.p6 != 0)
     return fail(3);
   if (p.k <= 0 || p.k % (128 * unroll) != 0) return fail(4);
   const int64_t lim = (int64_t)1 << 31;
@@ -161,8 +161,6 @@ int launch_gemv_wave(const Problem& p, const tlhip_kernel_config_t& c, hipStream
   a.x_bytes = (uint32_t)(p.m * p.k * 2);
   a.alpha = p.alpha;
   a.y_dtype = p.y_dtype;
-  a.abl = c.p4;
-  a.dbg = (unsigned long long*)(((uint64_t)(uint32_t)c.p6 << 32) | (uint32_t)(c.p4 ? c.p5 & ~1 : 0));
   a.epi = p.epi;
   const void* fn = wave_fn(geo.rp, geo.mq, depth, unroll, line);
   if (!fn) return set_error(TLHIP_ERR_INVALID, "gemv_wave: no kernel instance for this configuration");

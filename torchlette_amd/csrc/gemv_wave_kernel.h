@@ -63,8 +63,6 @@ struct WaveArgs {
   uint32_t packed_bytes, scales_bytes, x_bytes;
   float alpha;
   int y_dtype;
-  int abl;       // timing experiments only (results invalid when set)
-  unsigned long long* dbg;  // timing experiments only: 32 time stamps per workgroup
   DevEpilogue epi;
 };
 
@@ -101,16 +99,6 @@ __global__ __launch_bounds__(512) void gemv_wave_kernel(const WaveArgs a) {
   const __amdgpu_buffer_rsrc_t bx = wave_rsrc(a.x, a.x_bytes);
   const int st0 = wave * a.steps;  // first step of this wave's K range
 
-  int nstamp = 0;
-  auto stamp = [&]() __attribute__((always_inline)) {
-    if (a.dbg && wave == (a.abl >> 8) && nstamp < 32) {
-      const unsigned long long now = __builtin_amdgcn_s_memtime();
-      if (lane == 0) a.dbg[wg * 32 + nstamp] = now;
-      ++nstamp;
-    }
-  };
-  stamp();
-
   // ---- scales of the whole K range, first in the queue
   u32x4 sreg[kWaveScaleLoads];
 #pragma unroll
@@ -119,7 +107,7 @@ __global__ __launch_bounds__(512) void gemv_wave_kernel(const WaveArgs a) {
     const int ri = (f * a.spr_recip) >> 16;  // f / spr (exact for f < 384, spr <= 24)
     const int piece = f - ri * a.spr;
     const int row = ((ri >> 4) * nwg + wg) * 16 + (ri & 15);
-    const int ok = (int)(i < a.nsl) & (int)(ri < RP * 16) & (int)(row < a.n) & (int)!(a.abl & 4);
+    const int ok = (int)(i < a.nsl) & (int)(ri < RP * 16) & (int)(row < a.n);
     // A piece may reach past the wave's K range into the next row's scales (never read back),
     // and the last row's past the end of the buffer: a raw buffer load is range-checked dword
     // by dword, so what lies inside arrives and the rest reads as zero.
@@ -141,7 +129,7 @@ __global__ __launch_bounds__(512) void gemv_wave_kernel(const WaveArgs a) {
 #pragma unroll
     for (int q = 0; q < MQ; ++q) {
       const int row = min(RPQ * q + xrow0, a.m - 1);
-      const int off = (row * (a.kb * 4) + st * (256 * U) + xunit * 16) & ((a.abl & 1) ? 0 : mask);
+      const int off = (row * (a.kb * 4) + st * (256 * U) + xunit * 16) & mask;
       rx[s][q] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(bx, off, 0, 0));
     }
 #pragma unroll
@@ -153,7 +141,7 @@ __global__ __launch_bounds__(512) void gemv_wave_kernel(const WaveArgs a) {
           const int row = (r * nwg + wg) * 16 + 8 * h + (lane >> 3);
           const int rmask = mask & -(int)(row < a.n);
           rw[s][r][h] = __builtin_bit_cast(
-              u32x4, __builtin_amdgcn_raw_buffer_load_b128(bw, (row * a.kb + st * 128 + (lane & 7) * 16) & ((a.abl & 2) ? 0 : rmask), 0, 2));
+              u32x4, __builtin_amdgcn_raw_buffer_load_b128(bw, (row * a.kb + st * 128 + (lane & 7) * 16) & rmask, 0, 2));
         }
       } else {
         const int row = (r * nwg + wg) * 16 + nl;
@@ -161,7 +149,7 @@ __global__ __launch_bounds__(512) void gemv_wave_kernel(const WaveArgs a) {
 #pragma unroll
         for (int u = 0; u < U; ++u)
           rw[s][r][u] = __builtin_bit_cast(
-              u32x4, __builtin_amdgcn_raw_buffer_load_b128(bw, (row * a.kb + (st * U + u) * 64 + g * 16) & ((a.abl & 2) ? 0 : rmask), 0, 2));
+              u32x4, __builtin_amdgcn_raw_buffer_load_b128(bw, (row * a.kb + (st * U + u) * 64 + g * 16) & rmask, 0, 2));
       }
     }
   };
@@ -171,18 +159,7 @@ __global__ __launch_bounds__(512) void gemv_wave_kernel(const WaveArgs a) {
   for (int r = 0; r < RP; ++r) acc[r] = (float4_t){0.f, 0.f, 0.f, 0.f};
 
   auto consume = [&](int s, int j) __attribute__((always_inline)) {
-    stamp();
-    if (a.abl & 8) {
-#pragma unroll
-      for (int r = 0; r < RP; ++r) {
-        uint32_t v = 0;
-#pragma unroll
-        for (int u = 0; u < U; ++u) v ^= rw[s][r][u].x ^ rw[s][r][u].w;
-#pragma unroll
-        for (int q = 0; q < MQ; ++q) v ^= rx[s][q].x;
-        acc[r][0] += __builtin_bit_cast(float, v & 0x3fffffffu);
-      }
-    } else if (st0 + j < a.nsteps) {  // wave-uniform: a step beyond K adds nothing
+    if (st0 + j < a.nsteps) {  // wave-uniform: a step beyond K adds nothing
       // activations: into the wave's patch
 #pragma unroll
       for (int q = 0; q < MQ; ++q) patch[(RPQ * q + xrow0) * RU + xunit] = permute_x_for_int4(rx[s][q]);
@@ -242,7 +219,6 @@ __global__ __launch_bounds__(512) void gemv_wave_kernel(const WaveArgs a) {
         }
       }
     }
-    stamp();
   };
 
   // The loads of step j + D are issued behind the arithmetic of step j.  The steady-state
@@ -253,7 +229,6 @@ __global__ __launch_bounds__(512) void gemv_wave_kernel(const WaveArgs a) {
   for (int s = 0; s < D; ++s) {
     if (s < T) issue(s, s);
   }
-  stamp();
   // the scales have arrived first: side by side into the wave's LDS
 #pragma unroll
   for (int i = 0; i < kWaveScaleLoads; ++i) {
@@ -294,7 +269,6 @@ __global__ __launch_bounds__(512) void gemv_wave_kernel(const WaveArgs a) {
       store_out(a.y, a.y_dtype, idx, apply_epilogue(a.epi, sum * a.alpha, col, idx));
     }
   }
-  stamp();
 }
 
 }  // namespace
