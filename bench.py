@@ -208,7 +208,8 @@ class Bench:
 def kernel_name_of(cfg) -> str:
     return {0: "gemv_kernel (VALU dot2)", 1: "gemv_mfma_kernel (16x16x32 f16)", 2: "gemm_prefill_kernel (32x32x16 f16)",
             3: "gemm_direct_kernel (32x32x16 f16, weights dequantised in registers)",
-            4: "gemv_xreg_kernel (16x16x32 f16, activations in registers)"}[cfg.variant]
+            4: "gemv_xreg_kernel (16x16x32 f16, activations in registers)",
+            5: "gemv_wave_kernel (16x16x32 f16, every wave its own K range)"}.get(cfg.variant, f"variant {cfg.variant}")
 
 
 def cpu_step(cases, host_weights, host_x, threads: int, keep=None) -> float:
