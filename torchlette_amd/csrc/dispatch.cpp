@@ -1349,11 +1349,16 @@ int tlhip_gemv_grouped_rows(const tlhip_gemv_problem_t* problems, int count, int
     if (shared && rows > 0) {
       Problem all = ps[0];
       all.n = rows;
-      tlhip_kernel_config_t c = select_config(all);
-      if (c.variant == VARIANT_GEMV_MFMA && gemv_mfma_group_applicable(ps, count, c, nullptr))
-        return launch_gemv_mfma_group(ps, count, c, s);
-      if (c.variant == VARIANT_GEMV_XREG && gemv_xreg_group_applicable(ps, count, c, nullptr))
-        return launch_gemv_xreg_group(ps, count, c, s);
+      // ... and where that choice has no grouped form (the VALU kernel at several rows,
+      // the per-wave pipelined kernel), the heuristic default of the same problem: one
+      // launch of a slightly slower kernel beats `count` launches of the fastest one
+      const tlhip_kernel_config_t tries[2] = {select_config(all), default_config(all)};
+      for (const tlhip_kernel_config_t& c : tries) {
+        if (c.variant == VARIANT_GEMV_MFMA && gemv_mfma_group_applicable(ps, count, c, nullptr))
+          return launch_gemv_mfma_group(ps, count, c, s);
+        if (c.variant == VARIANT_GEMV_XREG && gemv_xreg_group_applicable(ps, count, c, nullptr))
+          return launch_gemv_xreg_group(ps, count, c, s);
+      }
     }
   }
   for (int i = 0; i < count; ++i) {
