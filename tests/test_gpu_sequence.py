@@ -97,6 +97,34 @@ def test_mlp_block_in_one_launch(be, m, hidden, ff, act):
     assert np.array_equal(y, y2)
 
 
+def test_a_waiting_step_never_reads_what_the_buffer_held_before(be):
+    """The hidden buffer is the caller's and lives across launches: the down projection of
+    every launch must read what THIS launch's gate/up step wrote (its activation loads are
+    agent-scope loads; nothing invalidates the caches in between), never the lines of the
+    launch before.  Three launches back to back on one hidden buffer, activations that
+    differ in sign and size, each against the oracle."""
+    import ctypes as C
+    m, hidden, ff = 8, 2048, 6144
+    rng = np.random.default_rng(77)
+    gate, dg = weight(be, ff, hidden, rng, "f16")
+    up, du = weight(be, ff, hidden, rng, "f16")
+    down, dd = weight(be, hidden, ff, rng, "f32")
+    qg, qu, qd = (be._qweight(w, transposed=False) for w in (gate, up, down))
+    h = be._alloc([m, ff], "f16")
+    xs_host = [make_x(m, hidden, "f16", rng, std=s) * sign for s, sign in ((0.5, 1.0), (2.0, -1.0), (0.1, 1.0))]
+    xts = [be.ops.tensorFromArray(x, [m, hidden], "f16") for x in xs_host]
+    ys = [be._alloc([m, hidden], "f32") for _ in xs_host]
+    for xt, y in zip(xts, ys):   # no synchronisation in between
+        L.call("tlhip_mlp_decode", C.byref(qg), C.byref(qu), C.byref(qd), L.UNARY["silu"], xt.ptr, L.F16, m, h.ptr, y.ptr,
+               L.F32, None, None)
+    assert be.sequenceStatus() == 0
+    for x, y in zip(xs_host, ys):
+        xf = x.astype(np.float32)
+        hid = O.linear(xf, dg, None, "silu", threads=8).astype(np.float32) * O.linear(xf, du, threads=8).astype(np.float32)
+        want = O.linear(f16_round(hid).astype(np.float32), dd, threads=8)
+        assert rel_l2(y.numpy(), want) <= 2e-4, rel_l2(y.numpy(), want)
+
+
 def test_a_wait_that_cannot_be_satisfied_gives_up_and_reports(be):
     """The give-up path, forced from the host: every wait's threshold is made unreachable
     and the polls are capped, so each workgroup's wait expires, the kernel leaves normally,
@@ -134,3 +162,10 @@ def test_sequence_refuses_what_it_is_not_built_for(be):
     w8 = be.createQuantizedWeight(p8, s8, 256, 4096, T.resolveWeightFormat("int8-row", "f32"))
     with pytest.raises(L.TlhipError, match="int4 weights with group size 32"):
         be.linearSequence([{"input": x2, "weight": w8}])
+    # only activations may be an earlier step's output: a residual that the first step writes
+    w3, _ = weight(be, 4096, 4096, rng, "f16")
+    first_out = be._alloc([2, 4096], "f16")
+    with pytest.raises(L.TlhipError, match="overlaps the output of step 0"):
+        be.linearSequence([{"input": x2, "weight": w3, "out": first_out},
+                           {"input": first_out, "weight": w3, "wait": True, "binary": ("add", first_out)}])
+

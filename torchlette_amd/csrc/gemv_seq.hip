@@ -87,6 +87,21 @@ int tlhip_gemv_sequence(const tlhip_sequence_step_t* steps, int count, int x_dty
       P.scales[1] = s.w_up.scales;
     }
     if (i == 0 && s.wait) return set_error(TLHIP_ERR_INVALID, "gemv_sequence: the first step has nothing to wait for");
+    // Only activations may be an earlier step's output (they are loaded at agent scope
+    // behind the wait); bias and binary inputs are loaded early and through the caches.
+    for (int op = 0; op < p.epi.n_ops; ++op) {
+      if (!p.epi.input[op]) continue;
+      const bool binary = p.epi.kind[op] == TLHIP_EPI_BINARY;
+      const char* i0 = (const char*)p.epi.input[op];
+      const char* i1 = i0 + (size_t)(binary ? m * p.n : p.n) * (p.epi.input_dtype[op] == TLHIP_F16 ? 2 : 4);
+      for (int j = 0; j < i; ++j) {
+        const char* y0 = (const char*)steps[j].y;
+        const char* y1 = y0 + (size_t)m * (size_t)steps[j].w.n * (steps[j].y_dtype == TLHIP_F16 ? 2 : 4);
+        if (y0 && i0 < y1 && y0 < i1)
+          return set_error(TLHIP_ERR_INVALID, "gemv_sequence: an epilogue input of step %d overlaps the output of step %d of the "
+                                              "same launch (only activations may be an earlier step's output)", i, j);
+      }
+    }
     P.x = p.x;
     P.y = p.y;
     P.packed_bytes = (uint32_t)(p.n * (p.k / 2));

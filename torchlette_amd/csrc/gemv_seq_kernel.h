@@ -82,6 +82,8 @@ struct SeqState {
   uint32_t pad[15];
 };
 
+constexpr int kAuxAgentScope = 16;  // the sc1 bit of a buffer load's cache policy on gfx942 / gfx950
+
 struct SeqTable {
   int count;
   int m;
@@ -207,7 +209,11 @@ __global__ __launch_bounds__(512) void gemv_seq_kernel(const SeqTable a) {
 #pragma unroll
     for (int q = 0; q < MQ; ++q) {
       const int row = min(4 * q + xrow0, mrows - 1);
-      rx[s][q] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(c.bx, (row * (c.kb * 4) + st * 256 + xunit * 16) & mask, 0, 0));
+      // The activations of a step that waits were written by other workgroups of this
+      // launch, so they are loaded at agent scope (sc1: never served from a stale line of
+      // this XCD's L2 or of the vector cache); those of other steps too, because a second
+      // form of the load under a condition multiplies the paths through the unit loop.
+      rx[s][q] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(c.bx, (row * (c.kb * 4) + st * 256 + xunit * 16) & mask, 0, kAuxAgentScope));
     }
 #pragma unroll
     for (int r = 0; r < RP; ++r) {
@@ -450,7 +456,10 @@ __global__ __launch_bounds__(512) void gemv_seq_kernel(const SeqTable a) {
         const bool gave_up = *flag == 0;
         lds_barrier();  // nobody rewrites the flag before everybody has read it
         if (gave_up) break;
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+        // No agent-scope acquire here: it invalidates the XCD's whole L2, which every other
+        // workgroup streams through, and cost a waiting launch 13 us.  What the wait orders
+        // are this problem's activation loads, and those are agent-scope loads themselves.
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
         waited = need;
       }
       // the same memory operations in the same order as a unit's last D steps and its end
