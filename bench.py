@@ -661,24 +661,40 @@ def main() -> int:
             us_sep = B.median_time(runner(sep), 40)
             us_grp = B.median_time(runner(grp), 40)
             us_gu = B.median_time(gate_up, 100)
-            # the MLP block (gate, up, act(gate) * up, down): one sequence launch
-            # (tlhip_mlp_decode, dependent steps ordered inside the kernel) beside the three
-            # launches it replaces (gate/up grouped, the gated multiply, down)
+            # the MLP block (gate, up, act(gate) * up, down) three ways: one call into the
+            # library (tlhip_mlp_decode: it issues gate/up grouped, the gated multiply and down),
+            # the same three launches as three calls, and one sequence launch
+            # (tlhip_gemv_sequence: a gated step and the down projection waiting for it)
             hbuf = be._alloc([m, 12288], "f16")
             mlp_q = [(be._qweight(p124[(2 * li) % len(p124)], False), be._qweight(p124[(2 * li + 1) % len(p124)], False),
                       be._qweight(p412[li % len(p412)], False)) for li in range(nlayers)]
-            mlp_fn, gm_fn = L.load().tlhip_mlp_decode, L.load().tlhip_gated_mul
+            mlp_fn, gm_fn, seq_fn = L.load().tlhip_mlp_decode, L.load().tlhip_gated_mul, L.load().tlhip_gemv_sequence
+            silu = be.makeEpilogue(None, "silu")
+            seq_steps = []
+            for qg, qu, qd in mlp_q:
+                arr = (L.SequenceStep * 2)()
+                arr[0].w, arr[0].w_up, arr[0].gated = qg, qu, 1
+                arr[0].x, arr[0].y, arr[0].y_dtype, arr[0].epilogue = x4.ptr, hbuf.ptr, L.F16, C.pointer(silu)
+                arr[1].w, arr[1].x, arr[1].y, arr[1].y_dtype, arr[1].wait = qd, hbuf.ptr, y["down"].ptr, L.F16, 1
+                seq_steps.append(arr)
 
-            def mlp_one_launch():
+            def mlp_one_call():
                 qg, qu, qd = mlp_q[state["i"] % nlayers]
                 state["i"] += 1
                 rc = mlp_fn(C.byref(qg), C.byref(qu), C.byref(qd), L.UNARY["silu"], x4.ptr, L.F16, m, hbuf.ptr, y["down"].ptr,
                             L.F16, None, None)
                 if rc:
                     L.check(rc)
+
+            def mlp_sequence_launch():
+                arr = seq_steps[state["i"] % nlayers]
+                state["i"] += 1
+                rc = seq_fn(arr, 2, L.F16, m, 1.0, None)
+                if rc:
+                    L.check(rc)
             down_only = [probs_of([(p412[li % len(p412)], hbuf, y["down"])]) for li in range(nlayers)]
 
-            def mlp_three_launches():
+            def mlp_three_calls():
                 i = state["i"] % nlayers
                 state["i"] += 1
                 arr, cnt = gu_only[i]
@@ -689,18 +705,21 @@ def main() -> int:
                 if rc:
                     L.check(rc)
             mlp_bytes = gu_bytes + algorithmic_bytes("int4", 4096, 12288, 32, m, 2, 2)
-            us_mlp1 = B.median_time(mlp_one_launch, 40)
-            us_mlp3 = B.median_time(mlp_three_launches, 40)
+            us_mlp1 = B.median_time(mlp_one_call, 40)
+            us_mlp3 = B.median_time(mlp_three_calls, 40)
+            us_mlps = B.median_time(mlp_sequence_launch, 40)
             err = C.c_int(0)
             L.call("tlhip_sequence_status", None, C.byref(err))
             hbuf.destroy()
             layer_rows.append({
                 "m": m, "bytes": layer_bytes,
-                "mlp_block": {"bytes": mlp_bytes, "us_one_sequence_launch": round(us_mlp1, 2),
-                              "us_three_launches": round(us_mlp3, 2),
-                              "gbps_one_sequence_launch": round(mlp_bytes / us_mlp1 / 1e3, 1),
-                              "gbps_three_launches": round(mlp_bytes / us_mlp3 / 1e3, 1),
-                              "note": "tlhip_mlp_decode vs grouped gate/up + tlhip_gated_mul + down"}, "us_7_launches": round(us_sep, 2), "us_4_launches": round(us_grp, 2),
+                "mlp_block": {"bytes": mlp_bytes, "us_one_call": round(us_mlp1, 2), "us_three_calls": round(us_mlp3, 2),
+                              "us_one_sequence_launch": round(us_mlps, 2),
+                              "gbps_one_call": round(mlp_bytes / us_mlp1 / 1e3, 1),
+                              "gbps_one_sequence_launch": round(mlp_bytes / us_mlps / 1e3, 1),
+                              "note": "tlhip_mlp_decode (gate/up grouped + gated multiply + down from one call) vs the "
+                                      "same launches as three calls vs tlhip_gemv_sequence (one launch)"},
+                "us_7_launches": round(us_sep, 2), "us_4_launches": round(us_grp, 2),
                 "gbps_4_launches": round(layer_bytes / us_grp / 1e3, 1),
                 "frac_of_peak_4_launches": round(layer_bytes / us_grp / 1e3 / HBM_PEAK_GBPS, 4),
                 "gate_up_grouped_us": round(us_gu, 2), "gate_up_grouped_gbps": round(gu_bytes / us_gu / 1e3, 1),

@@ -309,8 +309,14 @@ typedef struct {
 } tlhip_sequence_step_t;
 int tlhip_gemv_sequence(const tlhip_sequence_step_t* steps, int count, int x_dtype, int64_t m, float alpha,
                         tlhip_stream_t stream);
-/* The MLP block of a decoder layer as one sequence launch:
- * h = unary(x gate^T) * (x up^T)  (f16 [m, gate.N], caller-provided),  y = epilogue(h down^T). */
+/* The MLP block of a decoder layer from one call:
+ * h = unary(x gate^T) * (x up^T)  (f16 [m, gate.N], caller-provided),  y = epilogue(h down^T).
+ * f16 activations, 1..16 rows, any weight format.  The library runs the form that measures
+ * faster: today three launches (gate and up grouped on the shared activations, the gated
+ * multiply, down; gate and up are rounded to f16 in between, as the model's own ops would),
+ * with 2 MiB of the stream's workspace between them, so a stream's first call must not be
+ * captured.  TLHIP_MLP_ONE_LAUNCH=1 in the environment selects the sequence launch (a gated
+ * step and the down projection waiting for it: int4 g32 only, the product rounded once). */
 int tlhip_mlp_decode(const tlhip_qweight_t* gate, const tlhip_qweight_t* up, const tlhip_qweight_t* down, int unary,
                      const void* x, int x_dtype, int64_t m, void* h, void* y, int y_dtype,
                      const tlhip_epilogue_t* down_epilogue, tlhip_stream_t stream);

@@ -103,7 +103,7 @@ for (const c of manifest.cases) {
       }
     }
   } else if (c.kind === "mlp") {
-    // the MLP block of a decode step as one call and one launch
+    // the MLP block of a decode step as one call into the addon
     const x = tensor(be, c.x, [c.m, c.k], "f16");
     const [gate, up, down] = c.weights.map((wc) => weightOf(be, Object.assign({ format: c.format, element: "f16" }, wc)));
     const g0 = H.getQuantGemvDispatchCount();

@@ -68,33 +68,61 @@ def test_independent_steps_match_the_oracle_and_separate_launches(be, m):
         assert np.array_equal(g, h)  # the sums are formed in a fixed order
 
 
+@pytest.mark.parametrize("one_launch", [True, False], ids=["sequence-launch", "three-launches"])
 @pytest.mark.parametrize("act", ["silu", "gelu"])
 @pytest.mark.parametrize("m,hidden,ff", [(1, 4096, 12288), (8, 4096, 12288), (16, 4096, 12288), (5, 3072, 3072), (16, 2048, 8192)])
-def test_mlp_block_in_one_launch(be, m, hidden, ff, act):
+def test_mlp_block_from_one_call(be, m, hidden, ff, act, one_launch):
     """down(act(gate(x)) * up(x)): the reference's three Linears and two elementwise ops
-    (packages/qwen3-browser/src/model.ts:357-361; gemma2: gelu) against the oracle."""
+    (packages/qwen3-browser/src/model.ts:357-361; gemma2: gelu) against the oracle, as the
+    sequence launch and as tlhip_mlp_decode runs it by default (gate and up grouped, the
+    gated multiply, down)."""
     rng = np.random.default_rng(zlib.crc32(repr(("mlp", m, hidden, ff, act)).encode()))
     gate, dg = weight(be, ff, hidden, rng, "f16")
     up, du = weight(be, ff, hidden, rng, "f16")
     down, dd = weight(be, hidden, ff, rng, "f32")
     x = make_x(m, hidden, "f16", rng, std=0.5)
     xt = be.ops.tensorFromArray(x, [m, hidden], "f16")
-    y = be.mlpDecode(xt, gate, up, down, act).numpy()
+    before = T.getQuantGemvDispatchCount()
+    y = be.mlpDecode(xt, gate, up, down, act, oneLaunch=one_launch).numpy()
+    counted = T.getQuantGemvDispatchCount() - before
+    assert counted == 2 if one_launch else counted >= 2   # the sequence's steps / the launches' Linears
     assert be.sequenceStatus() == 0
     xf = x.astype(np.float32)
-    g = O.linear(xf, dg, None, "gelu_tanh" if act == "gelu" else act, threads=8)
-    u = O.linear(xf, du, threads=8)
-    h = (g.astype(np.float32) * u.astype(np.float32)).astype(np.float32)
+    oact = "gelu_tanh" if act == "gelu" else act
+    g_lin, u_lin = O.linear(xf, dg, threads=8), O.linear(xf, du, threads=8)
+    h = O.gated(g_lin, u_lin, oact)
     want_exact = O.linear(h, dd, threads=8)
     assert y.shape == (m, hidden) and y.dtype == np.float32
     assert rel_l2(y, want_exact) <= 1e-3, rel_l2(y, want_exact)
-    # against the same sequence on f16 tensors (h rounded to f16 once): sum order and the
-    # hardware exp of the activation only
-    want_f16 = O.linear(f16_round(h).astype(np.float32), dd, threads=8)
+    # against the same sequence on f16 tensors: the sequence launch rounds the hidden product
+    # once, the three launches round gate and up to f16 first, as the model's ops would;
+    # what is left is the order of the sums and the hardware exp of the activation
+    if one_launch:
+        h16 = f16_round(h)
+    else:
+        h16 = f16_round(O.gated(f16_round(g_lin).astype(np.float32), f16_round(u_lin).astype(np.float32), oact))
+    want_f16 = O.linear(h16.astype(np.float32), dd, threads=8)
     assert rel_l2(y, want_f16) <= 2e-4, rel_l2(y, want_f16)
-    # and the same launch twice gives the same bits
-    y2 = be.mlpDecode(xt, gate, up, down, act).numpy()
+    # and the same call twice gives the same bits
+    y2 = be.mlpDecode(xt, gate, up, down, act, oneLaunch=one_launch).numpy()
     assert np.array_equal(y, y2)
+
+
+def test_mlp_block_from_one_call_in_the_reference_format(be):
+    """tlhip_mlp_decode takes any weight format (its launches are the library's ordinary
+    ones): the reference's int8 in groups of 64, gelu as in Gemma-2."""
+    m, hidden, ff = 4, 1024, 4096
+    rng = np.random.default_rng(91)
+    ws = []
+    for n, k, element in ((ff, hidden, "f16"), (ff, hidden, "f16"), (hidden, ff, "f32")):
+        packed, scales, deq = make_weight("int8-grouped", n, k, 64, rng)
+        ws.append((be.createQuantizedWeight(packed, scales, n, k, T.resolveWeightFormat("int8-64", element)), deq))
+    (gate, dg), (up, du), (down, dd) = ws
+    x = make_x(m, hidden, "f16", rng, std=0.5)
+    y = be.mlpDecode(be.ops.tensorFromArray(x, [m, hidden], "f16"), gate, up, down, "gelu").numpy()
+    xf = x.astype(np.float32)
+    h = O.gated(O.linear(xf, dg, threads=8), O.linear(xf, du, threads=8), "gelu_tanh")
+    assert rel_l2(y, O.linear(h, dd, threads=8)) <= 1e-3
 
 
 def test_a_waiting_step_never_reads_what_the_buffer_held_before(be):
@@ -103,20 +131,18 @@ def test_a_waiting_step_never_reads_what_the_buffer_held_before(be):
     agent-scope loads; nothing invalidates the caches in between), never the lines of the
     launch before.  Three launches back to back on one hidden buffer, activations that
     differ in sign and size, each against the oracle."""
-    import ctypes as C
     m, hidden, ff = 8, 2048, 6144
     rng = np.random.default_rng(77)
     gate, dg = weight(be, ff, hidden, rng, "f16")
     up, du = weight(be, ff, hidden, rng, "f16")
     down, dd = weight(be, hidden, ff, rng, "f32")
-    qg, qu, qd = (be._qweight(w, transposed=False) for w in (gate, up, down))
     h = be._alloc([m, ff], "f16")
     xs_host = [make_x(m, hidden, "f16", rng, std=s) * sign for s, sign in ((0.5, 1.0), (2.0, -1.0), (0.1, 1.0))]
     xts = [be.ops.tensorFromArray(x, [m, hidden], "f16") for x in xs_host]
     ys = [be._alloc([m, hidden], "f32") for _ in xs_host]
     for xt, y in zip(xts, ys):   # no synchronisation in between
-        L.call("tlhip_mlp_decode", C.byref(qg), C.byref(qu), C.byref(qd), L.UNARY["silu"], xt.ptr, L.F16, m, h.ptr, y.ptr,
-               L.F32, None, None)
+        be.linearSequence([{"input": xt, "weight": gate, "up": up, "activation": "silu", "out": h},
+                           {"input": h, "weight": down, "wait": True, "out": y}])
     assert be.sequenceStatus() == 0
     for x, y in zip(xs_host, ys):
         xf = x.astype(np.float32)
@@ -134,16 +160,16 @@ def test_a_wait_that_cannot_be_satisfied_gives_up_and_reports(be):
     up, _ = weight(be, 4096, 3072, rng, "f16")
     down, dd = weight(be, 3072, 4096, rng, "f32")
     xt = be.ops.tensorFromArray(make_x(4, 3072, "f16", rng), [4, 3072], "f16")
-    good = be.mlpDecode(xt, gate, up, down, "silu").numpy()
+    good = be.mlpDecode(xt, gate, up, down, "silu", oneLaunch=True).numpy()
     assert be.sequenceStatus() == 0
     L.call("tlhip_debug_sequence", 1, 2000)
     try:
-        be.mlpDecode(xt, gate, up, down, "silu")
+        be.mlpDecode(xt, gate, up, down, "silu", oneLaunch=True)
         with pytest.raises(L.TlhipError, match="a wait for earlier steps"):
             be.sequenceStatus()
     finally:
         L.call("tlhip_debug_sequence", 0, 0)
-    again = be.mlpDecode(xt, gate, up, down, "silu").numpy()
+    again = be.mlpDecode(xt, gate, up, down, "silu", oneLaunch=True).numpy()
     assert be.sequenceStatus() == 0
     assert np.array_equal(good, again)
 

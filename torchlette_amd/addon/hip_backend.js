@@ -490,8 +490,9 @@ class HipBackend {
   }
 
   /** down(mul(gateActivation(gate(input)), up(input))) of a decode step's MLP block
-   *  (packages/qwen3-browser/src/model.ts:357-361) as ONE launch: int4 g32 weights, f16
-   *  activations, 1..16 rows.  One call from the host instead of three. */
+   *  (packages/qwen3-browser/src/model.ts:357-361) from ONE call into the addon instead
+   *  of three (the library issues the launches, whichever form is faster): f16
+   *  activations, 1..16 rows. */
   mlpDecode(input, gate, up, down, gateActivation) {
     const ga = this._weightArgs(gate, false), ua = this._weightArgs(up, false), da = this._weightArgs(down, false);
     const k = ga[3], ff = ga[2];

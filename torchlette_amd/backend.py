@@ -647,22 +647,28 @@ class HipBackend:
         return outs
 
     def mlpDecode(self, input: HipTensor, gate: HipTensor, up: HipTensor, down: HipTensor,
-                  activation: str = "silu") -> HipTensor:
-        """down(act(gate(x)) * up(x)) (packages/qwen3-browser/src/model.ts:357-361) as one launch."""
+                  activation: str = "silu", oneLaunch: bool = False) -> HipTensor:
+        """down(act(gate(x)) * up(x)) (packages/qwen3-browser/src/model.ts:357-361) from one
+        call: tlhip_mlp_decode, which runs the faster form (today the three launches the model
+        issues); oneLaunch=True asks for the sequence launch (a gated step and the down
+        projection waiting for it, int4 weights in groups of 32 only)."""
         qg, qu, qd = (self._qweight(w, transposed=False) for w in (gate, up, down))
         if input.dtype != "f16" or not input.isContiguous or input.shape[-1] != qg.k:
             raise ValueError("mlpDecode: activations must be contiguous [m, K] f16")
         m = input.size // qg.k
         h = self._alloc([m, qg.n], "f16")
-        out_dtype = "f16" if down.format.elementType == "f16" else "f32"
-        y = self._alloc(list(input.shape[:-1]) + [qd.n], out_dtype)
         act = "gelu_tanh" if activation == "gelu" else activation
         try:
+            if oneLaunch:
+                return self.linearSequence([{"input": input, "weight": gate, "up": up, "activation": act, "out": h},
+                                            {"input": h, "weight": down, "wait": True}])[1]
+            out_dtype = "f16" if down.format.elementType == "f16" else "f32"
+            y = self._alloc(list(input.shape[:-1]) + [qd.n], out_dtype)
             L.call("tlhip_mlp_decode", C.byref(qg), C.byref(qu), C.byref(qd), L.UNARY[act], input.ptr, L.F16, m, h.ptr,
                    y.ptr, _DT_CODE[out_dtype], None, self.stream)
+            return y
         finally:
             h.destroy()  # tlhip_free waits for the device: the launch that reads h is over by then
-        return y
 
     def sequenceStatus(self) -> int:
         """Waits for the stream; raises if a sequence launch gave up a wait."""

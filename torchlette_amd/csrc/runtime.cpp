@@ -43,6 +43,8 @@ bool is_initialised() { return g_init; }
 
 hipStream_t resolve_stream(tlhip_stream_t s) { return s ? static_cast<hipStream_t>(s) : g_stream; }
 
+constexpr size_t kMlpScratchBytes = (size_t)2 << 20;  // 2 x 16 rows x 32768 f16
+
 namespace {
 // One workspace per stream.  A captured graph has the pointers of its capture stream's
 // workspace baked into its kernel arguments, so the workspace outlives the stream for as
@@ -104,7 +106,9 @@ int split_workspace(hipStream_t stream, float** workspace, int** counters) {
                        "split-K workspace of this stream does not exist yet and cannot be created during "
                        "capture: run the same call once on this stream before capturing");
     SplitWorkspace w{nullptr, nullptr, 0, 0, true};
-    TLHIP_CHECK_HIP(hipMalloc((void**)&w.workspace, kSplitWorkspaceFloats * sizeof(float)));
+    // + kMlpScratchBytes behind the workspace proper: the gate and up projections of
+    // tlhip_mlp_decode's three-launch form (nobody else indexes past kSplitWorkspaceFloats)
+    TLHIP_CHECK_HIP(hipMalloc((void**)&w.workspace, kSplitWorkspaceFloats * sizeof(float) + kMlpScratchBytes));
     // + 512 words behind the counters: the state of sequence launches on this stream
     hipError_t e = hipMalloc((void**)&w.counters, (kSplitCounters + 512) * sizeof(int));
     // on the stream that will use them (not capturing: checked above), so the clear is
@@ -119,6 +123,18 @@ int split_workspace(hipStream_t stream, float** workspace, int** counters) {
   }
   *workspace = it->second.workspace;
   *counters = it->second.counters;
+  return TLHIP_OK;
+}
+
+// 2 MiB of the stream's own behind its split-K workspace (gemv_seq.hip: the gate and up
+// outputs of the MLP block between its launches).
+int mlp_scratch(hipStream_t stream, void** scratch, size_t* bytes) {
+  float* workspace = nullptr;
+  int* counters = nullptr;
+  const int rc = split_workspace(stream, &workspace, &counters);
+  if (rc) return rc;
+  *scratch = workspace + kSplitWorkspaceFloats;
+  *bytes = kMlpScratchBytes;
   return TLHIP_OK;
 }
 
